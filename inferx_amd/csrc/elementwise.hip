@@ -1,0 +1,220 @@
+// Embedding gather, residual-add + RMSNorm, SwiGLU product, rotary table,
+// and the fused bias + rotation + cache-append that follows the q/k/v product.
+//
+// The residual stream `h` is float32 in every run; activations that feed
+// matrix products have the run's type (float32 or bfloat16).  Sums of squares,
+// the reciprocal root, rotation angles and the bias add are float32.
+#include "common.h"
+
+// ---------------------------------------------------------------------------
+// h[t, :] = table[ids[t], :]        (reference: EmbeddingKernel, layers.cu:465-481;
+// an id outside the table gives a zero row here instead of row 0 -- the host
+// rejects such ids before any launch)
+template <typename TW>
+__global__ void embed_kernel(float* __restrict__ h, const TW* __restrict__ table,
+                             const int32_t* __restrict__ ids, int64_t width, int64_t vocab) {
+  const int64_t t = blockIdx.x;
+  const int64_t id = ids[t];
+  const bool ok = id >= 0 && id < vocab;
+  const TW* row = table + (ok ? id : 0) * width;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) h[t * width + i] = ok ? ix_load(row + i) : 0.f;
+}
+
+extern "C" int ix_embed(void* h, const void* table, int table_dtype, const int32_t* ids, int64_t tokens,
+                        int64_t width, int64_t vocab, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "sizes must be positive");
+  if (tokens == 0) return 0;
+  dim3 grid(tokens), block(256);
+  if (table_dtype == IX_F32)
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (float*)h, (const float*)table, ids, width, vocab);
+  else if (table_dtype == IX_BF16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (float*)h, (const bf16_t*)table, ids, width,
+                       vocab);
+  else
+    IX_REQUIRE(false, "table dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_embed");
+}
+
+// ---------------------------------------------------------------------------
+// v = h[row] (+ delta[row]);  out[r] = v * rsqrt(mean(v^2) + eps) * w
+// (reference: RmsNormKernel, layers.cu:50-76: one reciprocal root per row, the
+// product x*inv*w formed in float32 and rounded once).
+// With `rows` == null every row r is normalised in place order and h is
+// updated with the sum; with `rows` given, out[r] comes from row rows[r] and h
+// is left alone (a row may be asked for twice).
+template <typename TD, typename TO>
+__global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__ delta, const void* __restrict__ w,
+                                   int w_dtype, TO* __restrict__ out, const int32_t* __restrict__ rows,
+                                   int64_t width, float eps) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t row = rows ? rows[r] : r;
+  float* hr = h + row * width;
+  const TD* dr = delta ? delta + row * width : nullptr;
+  const bool write_back = (rows == nullptr) && (dr != nullptr);
+  float sumsq = 0.f;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = hr[i];
+    if (dr) v += ix_load(dr + i);
+    if (write_back) hr[i] = v;
+    sumsq += v * v;
+  }
+  sumsq = ix_block_sum(sumsq, red);
+  const float inv = 1.0f / sqrtf(sumsq / static_cast<float>(width) + eps);
+  TO* outr = out + r * width;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) {
+    float v = hr[i];
+    if (dr && !write_back) v += ix_load(dr + i);
+    ix_store(outr + i, v * inv * ix_load_rt(w, w_dtype, i));
+  }
+}
+
+extern "C" int ix_add_rmsnorm(void* h, const void* delta, int delta_dtype, const void* w, int w_dtype, void* out,
+                              int out_dtype, const int32_t* rows, int64_t n_out_rows, int64_t width, float eps,
+                              hipStream_t stream) {
+  IX_REQUIRE(width > 0 && n_out_rows >= 0, "sizes must be positive");
+  IX_REQUIRE(w_dtype == IX_F32 || w_dtype == IX_BF16, "weight dtype must be float32 or bfloat16");
+  if (n_out_rows == 0) return 0;
+  dim3 grid(n_out_rows), block(width >= 4096 ? 1024 : (width >= 1024 ? 512 : 256));
+#define LAUNCH(TD, TO)                                                                                          \
+  hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), grid, block, 0, stream, (float*)h, (const TD*)delta, w, w_dtype, \
+                     (TO*)out, rows, width, eps)
+  if (delta_dtype == IX_F32 && out_dtype == IX_F32) LAUNCH(float, float);
+  else if (delta_dtype == IX_F32 && out_dtype == IX_BF16) LAUNCH(float, bf16_t);
+  else if (delta_dtype == IX_BF16 && out_dtype == IX_F32) LAUNCH(bf16_t, float);
+  else if (delta_dtype == IX_BF16 && out_dtype == IX_BF16) LAUNCH(bf16_t, bf16_t);
+  else IX_REQUIRE(false, "dtypes must be float32 or bfloat16");
+#undef LAUNCH
+  return ix_check_launch("ix_add_rmsnorm");
+}
+
+// ---------------------------------------------------------------------------
+// out[t, i] = silu(gu[t, i]) * gu[t, width + i],  silu(g) = g / (1 + exp(-g))
+// (reference: SiluMulFusedKernel, layers.cu:512-529)
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int64_t tokens, int64_t width) {
+  const int64_t n = tokens * width;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = i / width, c = i - t * width;
+    const float g = ix_load(gu + t * 2 * width + c);
+    const float u = ix_load(gu + t * 2 * width + width + c);
+    ix_store(out + i, g / (1.0f + expf(-g)) * u);
+  }
+}
+
+extern "C" int ix_silu_mul(const void* gu, void* out, int dtype, int64_t tokens, int64_t width, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  if (tokens == 0) return 0;
+  const int64_t n = tokens * width;
+  dim3 grid(static_cast<unsigned>(std::min<int64_t>((n + 255) / 256, 65536))), block(256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, tokens, width);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, tokens,
+                       width);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_silu_mul");
+}
+
+// ---------------------------------------------------------------------------
+// cs[t, j] = (cos a, sin a),  a = float(pos[t]) * inv_freq[j],  j < half
+// (reference: RopeKernel, layers.cu:80-115, which recomputes the angle per head
+// with fast intrinsics; here it is computed once per step with sincosf)
+__global__ void rope_table_kernel(float2* __restrict__ cs, const int32_t* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, int64_t tokens, int half) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= tokens * half) return;
+  const int64_t t = i / half;
+  const int j = static_cast<int>(i - t * half);
+  const float a = static_cast<float>(positions[t]) * inv_freq[j];
+  float s, c;
+  sincosf(a, &s, &c);
+  cs[i] = make_float2(c, s);
+}
+
+extern "C" int ix_rope_table(void* cs, const int32_t* positions, const float* inv_freq, int64_t tokens, int half,
+                             hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && half > 0, "sizes must be positive");
+  if (tokens == 0) return 0;
+  const int64_t n = tokens * half;
+  hipLaunchKernelGGL(rope_table_kernel, dim3((n + 255) / 256), dim3(256), 0, stream, (float2*)cs, positions, inv_freq,
+                     tokens, half);
+  return ix_check_launch("ix_rope_table");
+}
+
+// ---------------------------------------------------------------------------
+// After the fused q/k/v product: add the bias, rotate q and k (half-split
+// pairs (j, j + d/2): x'_j = x_j cos - x_{j+d/2} sin, x'_{j+d/2} = x_{j+d/2} cos
+// + x_j sin; reference RopeKernel layers.cu:80-115), write q to its own buffer
+// and k, v into the cache page of the token's slot (rotated keys are what the
+// cache holds; reference AppendKvKernel layers.cu:195-219, SplitQkvKernel :485-510).
+// Cache layout per layer: [page][kv_head][offset in page][head_dim].
+// A negative slot, or null caches, writes nothing to the cache.
+template <typename T>
+__global__ void qkv_rope_append_kernel(const T* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
+                                       const float2* __restrict__ cs, const int32_t* __restrict__ slots,
+                                       T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                       int heads, int kv_heads, int head_dim, int page_size, int64_t total_slots) {
+  const int64_t t = blockIdx.x;
+  const int half = head_dim / 2;
+  const int items = (heads + 2 * kv_heads) * half;
+  const int64_t in_width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
+  const T* in = qkv + t * in_width;
+  const int64_t slot = slots ? slots[t] : -1;
+  const bool cache_ok = k_cache != nullptr && slot >= 0 && slot < total_slots;
+  const int64_t page = cache_ok ? slot / page_size : 0;
+  const int off = cache_ok ? static_cast<int>(slot % page_size) : 0;
+  for (int p = blockIdx.y * blockDim.x + threadIdx.x; p < items; p += gridDim.y * blockDim.x) {
+    const int head = p / half, j = p - head * half;
+    const int col = head * head_dim + j;
+    float lo = ix_load(in + col), hi = ix_load(in + col + half);
+    if (bias) {
+      lo += ix_load_rt(bias, bias_dtype, col);
+      hi += ix_load_rt(bias, bias_dtype, col + half);
+    }
+    const bool is_v = head >= heads + kv_heads;
+    if (!is_v && cs) {
+      const float2 c = cs[t * half + j];
+      const float rlo = lo * c.x - hi * c.y;
+      const float rhi = hi * c.x + lo * c.y;
+      lo = rlo;
+      hi = rhi;
+    }
+    if (head < heads) {
+      T* dst = q_out + (t * heads + head) * head_dim + j;
+      ix_store(dst, lo);
+      ix_store(dst + half, hi);
+    } else if (cache_ok) {
+      const int g = is_v ? head - heads - kv_heads : head - heads;
+      T* base = is_v ? v_cache : k_cache;
+      T* dst = base + ((page * kv_heads + g) * page_size + off) * head_dim + j;
+      ix_store(dst, lo);
+      ix_store(dst + half, hi);
+    }
+  }
+}
+
+extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const void* cs,
+                                  const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int64_t tokens,
+                                  int heads, int kv_heads, int head_dim, int page_size, int64_t total_slots,
+                                  hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0, "sizes must be positive");
+  IX_REQUIRE(head_dim % 2 == 0, "head_dim must be even");
+  IX_REQUIRE((k_cache == nullptr) == (v_cache == nullptr), "give both caches or neither");
+  if (tokens == 0) return 0;
+  const int items = (heads + 2 * kv_heads) * (head_dim / 2);
+  dim3 grid(tokens, std::min((items + 255) / 256, 8)), block(256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(qkv_rope_append_kernel<float>, grid, block, 0, stream, (const float*)qkv, bias, bias_dtype,
+                       (const float2*)cs, slots, (float*)q_out, (float*)k_cache, (float*)v_cache, heads, kv_heads,
+                       head_dim, page_size, total_slots);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(qkv_rope_append_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)qkv, bias, bias_dtype,
+                       (const float2*)cs, slots, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads,
+                       head_dim, page_size, total_slots);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_qkv_rope_append");
+}

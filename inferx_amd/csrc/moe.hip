@@ -1,0 +1,342 @@
+// Mixture-of-experts feed-forward: router (product, softmax, top-k in float32),
+// grouping of assignments by expert, the plain grouped matrix products, and
+// the weighted sum with the shared expert.
+//
+// Placement is deterministic: no floating-point atomics anywhere, rows of one
+// expert keep token order (reference: ops/moe.h:26-33, moe.cu:130-221).
+#include "common.h"
+
+#define ROUTE_THREADS 256
+#define IX_MAX_TOP_K 32
+#define IX_MAX_EXPERTS 1024
+
+// ---------------------------------------------------------------------------
+// Router.  z_e = x . Wr[e] in float32 (the reference rounds z to bfloat16 first,
+// moe_ffn.cc:200-203); p = softmax(z) over all experts with the maximum
+// subtracted; k rounds of argmax with strict '>' so that the lowest index wins
+// a tie; optional renormalisation by the sum of the chosen; times `scale`
+// (reference: RouteTopKKernel, moe.cu:36-127).  Output order: descending score.
+// If `shared_gate_w` is given, sigmoid(x . shared_gate_w) is written too
+// (reference: AddSharedExpertKernel, moe.cu:275-287).
+template <typename T>
+__global__ void __launch_bounds__(ROUTE_THREADS)
+moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dtype,
+                 const void* __restrict__ shared_gate_w, int sg_dtype, float* __restrict__ topk_w,
+                 int32_t* __restrict__ topk_e, float* __restrict__ shared_gate, int64_t width, int experts, int k,
+                 int renormalize, float scale) {
+  extern __shared__ float smem[];
+  float* xs = smem;            // [width]
+  float* z = smem + width;     // [experts + 1]
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int64_t i = tid; i < width; i += ROUTE_THREADS) xs[i] = ix_load(x + t * width + i);
+  __syncthreads();
+  const int rows = experts + (shared_gate_w ? 1 : 0);
+  for (int e = wave; e < rows; e += ROUTE_THREADS / 64) {
+    const void* w = e < experts ? wr : shared_gate_w;
+    const int dt = e < experts ? wr_dtype : sg_dtype;
+    const int64_t base = e < experts ? static_cast<int64_t>(e) * width : 0;
+    float dot = 0.f;
+    for (int64_t i = lane; i < width; i += 64) dot += xs[i] * ix_load_rt(w, dt, base + i);
+    dot = ix_wave_sum(dot);
+    if (lane == 0) z[e] = dot;
+  }
+  __syncthreads();
+  if (shared_gate_w && tid == 0) shared_gate[t] = 1.0f / (1.0f + expf(-z[experts]));
+  float mx = -INFINITY;
+  for (int e = tid; e < experts; e += ROUTE_THREADS) mx = fmaxf(mx, z[e]);
+  mx = ix_block_max(mx, red);
+  float sum = 0.f;
+  for (int e = tid; e < experts; e += ROUTE_THREADS) {
+    const float p = expf(z[e] - mx);
+    z[e] = p;
+    sum += p;
+  }
+  sum = ix_block_sum(sum, red);  // its barriers also publish z
+  if (wave != 0) return;
+  const float inv_sum = 1.0f / sum;
+  float chosen = 0.f;  // lane s keeps the weight of slot s
+  float total = 0.f;
+  for (int slot = 0; slot < k; ++slot) {
+    float bv = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int e = lane; e < experts; e += 64) {
+      const float v = z[e];
+      if (v > bv) { bv = v; bi = e; }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float ov = __shfl_xor(bv, off, 64);
+      const int oi = __shfl_xor(bi, off, 64);
+      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    }
+    if (bi < 0 || bi >= experts) bi = 0;  // only when every score is NaN
+    const float wgt = bv * inv_sum;
+    total += wgt;
+    if (lane == slot) chosen = wgt;
+    if (lane == 0) {
+      topk_e[t * k + slot] = bi;
+      z[bi] = -INFINITY;
+    }
+    __builtin_amdgcn_wave_barrier();
+    __threadfence_block();
+  }
+  const float f = ((renormalize && total > 0.f) ? 1.0f / total : 1.0f) * scale;
+  if (lane < k) topk_w[t * k + lane] = chosen * f;
+}
+
+extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dtype, const void* shared_gate_w,
+                            int sg_dtype, float* topk_w, int32_t* topk_e, float* shared_gate, int64_t tokens,
+                            int64_t width, int experts, int k, int renormalize, float scale, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
+  IX_REQUIRE(k > 0 && k <= experts && k <= IX_MAX_TOP_K, "top_k must be between 1 and min(experts, 32)");
+  const size_t smem = (width + experts + 1) * sizeof(float);
+  IX_REQUIRE(smem <= 60 * 1024, "hidden width too large for the router kernel (limit about 15000)");
+  if (tokens == 0) return 0;
+  dim3 grid(tokens), block(ROUTE_THREADS);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, smem, stream, (const float*)x, wr, wr_dtype,
+                       shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, smem, stream, (const bf16_t*)x, wr, wr_dtype,
+                       shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_moe_route");
+}
+
+// ---------------------------------------------------------------------------
+// Grouping.  From topk_e[A] (assignment a = token * k + slot) make
+//   offsets[E + 1]  rows of expert e are [offsets[e], offsets[e + 1])
+//   rows[A]         grouped row -> token
+//   dest[A]         assignment  -> grouped row
+// stable: within an expert, rows keep assignment order
+// (reference: MoeBuildDispatch, moe.cu:452-513; kernels :130-221).
+__global__ void __launch_bounds__(1024)
+moe_count_scan_kernel(const int32_t* __restrict__ topk_e, int32_t* __restrict__ offsets, int64_t assignments,
+                      int experts) {
+  __shared__ int32_t counts[IX_MAX_EXPERTS];
+  for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
+  __syncthreads();
+  for (int64_t a = threadIdx.x; a < assignments; a += blockDim.x) {
+    const int e = topk_e[a];
+    if (e >= 0 && e < experts) atomicAdd(&counts[e], 1);  // integer counts: order does not matter
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int32_t run = 0;
+    for (int e = 0; e < experts; ++e) {
+      offsets[e] = run;
+      run += counts[e];
+    }
+    offsets[experts] = run;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+moe_scatter_kernel(const int32_t* __restrict__ topk_e, const int32_t* __restrict__ offsets,
+                   int32_t* __restrict__ rows, int32_t* __restrict__ dest, int64_t assignments, int k) {
+  __shared__ int32_t wave_count[4];
+  const int e = blockIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  int32_t next = offsets[e];
+  for (int64_t base = 0; base < assignments; base += 256) {
+    const int64_t a = base + threadIdx.x;
+    const bool mine = a < assignments && topk_e[a] == e;
+    const unsigned long long ballot = __ballot(mine);
+    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
+    __syncthreads();
+    if (lane == 0) wave_count[wave] = __popcll(ballot);
+    __syncthreads();
+    int wave_base = 0, total = 0;
+    for (int w = 0; w < 4; ++w) {
+      if (w < wave) wave_base += wave_count[w];
+      total += wave_count[w];
+    }
+    if (mine) {
+      const int32_t r = next + wave_base + before;
+      rows[r] = static_cast<int32_t>(a / k);
+      dest[a] = r;
+    }
+    next += total;
+  }
+}
+
+extern "C" int ix_moe_dispatch(const int32_t* topk_e, int32_t* offsets, int32_t* rows, int32_t* dest,
+                               int64_t assignments, int experts, int k, hipStream_t stream) {
+  IX_REQUIRE(assignments >= 0 && k > 0, "sizes must be positive");
+  IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
+  hipLaunchKernelGGL(moe_count_scan_kernel, dim3(1), dim3(1024), 0, stream, topk_e, offsets, assignments, experts);
+  if (assignments > 0)
+    hipLaunchKernelGGL(moe_scatter_kernel, dim3(experts), dim3(256), 0, stream, topk_e, offsets, rows, dest,
+                       assignments, k);
+  return ix_check_launch("ix_moe_dispatch");
+}
+
+// ---------------------------------------------------------------------------
+// Plain grouped product over device-resident offsets.
+//   GATE_UP: out[r, n] = silu(x[src(r)] . W[e][n]) * (x[src(r)] . W[e][inner + n]),  n < inner
+//            with src(r) = rows[r] (the gather is fused), W [E, 2*inner, width]
+//   else:    out[r, n] = a[r] . W[e][n],  W [E, n_out, width]
+// (reference: GroupedGemmBf16Kernel, moe.cu:323-392; SwiGLU moe_ffn.cc:288-291).
+// 64 x 64 output tile per workgroup, 4 x 4 per thread, float32 accumulation.
+// Tile index -> expert: experts are walked in order, each owning ceil(count/64) tiles.
+#define GG_BM 64
+#define GG_BN 64
+#define GG_BK 16
+
+template <typename TA, typename TW, typename TO, bool GATE_UP>
+__global__ void __launch_bounds__(256)
+moe_grouped_plain_kernel(const TA* __restrict__ a, const TW* __restrict__ w, TO* __restrict__ out,
+                         const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows, int experts,
+                         int64_t n_out, int64_t width) {
+  __shared__ float As[GG_BK][GG_BM + 4];
+  __shared__ float Ws[GATE_UP ? 2 : 1][GG_BK][GG_BN + 4];
+  __shared__ int32_t src_row[GG_BM];
+
+  // which expert owns m-tile blockIdx.y
+  int tile = blockIdx.y, e = 0, row0 = 0, row_end = 0;
+  for (; e < experts; ++e) {
+    const int begin = offsets[e], end = offsets[e + 1];
+    const int tiles = (end - begin + GG_BM - 1) / GG_BM;
+    if (tile < tiles) {
+      row0 = begin + tile * GG_BM;
+      row_end = end;
+      break;
+    }
+    tile -= tiles;
+  }
+  if (e == experts) return;
+
+  const int tid = threadIdx.x;
+  const int64_t n0 = static_cast<int64_t>(blockIdx.x) * GG_BN;
+  const int64_t w_rows = GATE_UP ? 2 * n_out : n_out;
+  const TW* we = w + static_cast<int64_t>(e) * w_rows * width;
+  if (tid < GG_BM) {
+    const int r = row0 + tid;
+    src_row[tid] = r < row_end ? (rows ? rows[r] : r) : -1;
+  }
+  __syncthreads();
+
+  const int tx = tid & 15, ty = tid >> 4;  // thread owns rows ty*4.., cols tx*4..
+  float acc[GATE_UP ? 2 : 1][4][4] = {};
+  for (int64_t k0 = 0; k0 < width; k0 += GG_BK) {
+    // stage A: 64 rows x 16 k, W: 64 cols x 16 k (x2 with the gate)
+    for (int i = tid; i < GG_BM * GG_BK; i += 256) {
+      const int r = i / GG_BK, kk = i % GG_BK;
+      const int sr = src_row[r];
+      const int64_t kc = k0 + kk;
+      As[kk][r] = (sr >= 0 && kc < width) ? ix_load(a + static_cast<int64_t>(sr) * width + kc) : 0.f;
+    }
+    for (int i = tid; i < GG_BN * GG_BK; i += 256) {
+      const int c = i / GG_BK, kk = i % GG_BK;
+      const int64_t n = n0 + c, kc = k0 + kk;
+      const bool ok = n < n_out && kc < width;
+      Ws[0][kk][c] = ok ? ix_load(we + n * width + kc) : 0.f;
+      if (GATE_UP) Ws[1][kk][c] = ok ? ix_load(we + (n_out + n) * width + kc) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < GG_BK; ++kk) {
+      float av[4], wv[GATE_UP ? 2 : 1][4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) av[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        wv[0][j] = Ws[0][kk][tx * 4 + j];
+        if (GATE_UP) wv[1][j] = Ws[1][kk][tx * 4 + j];
+      }
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          acc[0][i][j] += av[i] * wv[0][j];
+          if (GATE_UP) acc[1][i][j] += av[i] * wv[1][j];
+        }
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = row0 + ty * 4 + i;
+    if (r >= row_end) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int64_t n = n0 + tx * 4 + j;
+      if (n >= n_out) continue;
+      float v = acc[0][i][j];
+      if (GATE_UP) v = v / (1.0f + expf(-v)) * acc[1][i][j];
+      ix_store(out + static_cast<int64_t>(r) * n_out + n, v);
+    }
+  }
+}
+
+template <bool GATE_UP>
+static int launch_grouped_plain(const void* a, int a_dtype, const void* w, int w_dtype, void* out,
+                                const int32_t* offsets, const int32_t* rows, int64_t assignments, int experts,
+                                int64_t n_out, int64_t width, hipStream_t stream) {
+  const int64_t m_tiles = std::min<int64_t>(assignments, (assignments + GG_BM - 1) / GG_BM + experts);
+  dim3 grid((n_out + GG_BN - 1) / GG_BN, m_tiles), block(256);
+#define LAUNCH(TA, TW)                                                                                            \
+  hipLaunchKernelGGL((moe_grouped_plain_kernel<TA, TW, TA, GATE_UP>), grid, block, 0, stream, (const TA*)a,        \
+                     (const TW*)w, (TA*)out, offsets, rows, experts, n_out, width)
+  if (a_dtype == IX_F32 && w_dtype == IX_F32) LAUNCH(float, float);
+  else if (a_dtype == IX_F32 && w_dtype == IX_BF16) LAUNCH(float, bf16_t);
+  else if (a_dtype == IX_BF16 && w_dtype == IX_F32) LAUNCH(bf16_t, float);
+  else if (a_dtype == IX_BF16 && w_dtype == IX_BF16) LAUNCH(bf16_t, bf16_t);
+  else { ix_set_error("grouped product: dtypes must be float32 or bfloat16"); return 1; }
+#undef LAUNCH
+  return ix_check_launch("ix_moe_grouped_plain");
+}
+
+extern "C" int ix_moe_grouped_plain(const void* a, int a_dtype, const void* w, int w_dtype, void* out,
+                                    const int32_t* offsets, const int32_t* rows, int64_t assignments, int experts,
+                                    int64_t n_out, int64_t width, int gate_up, hipStream_t stream) {
+  IX_REQUIRE(assignments >= 0 && n_out > 0 && width > 0 && experts > 0, "sizes must be positive");
+  IX_REQUIRE(assignments < (1ll << 31) / GG_BM, "too many assignments");
+  if (assignments == 0) return 0;
+  return gate_up ? launch_grouped_plain<true>(a, a_dtype, w, w_dtype, out, offsets, rows, assignments, experts, n_out,
+                                              width, stream)
+                 : launch_grouped_plain<false>(a, a_dtype, w, w_dtype, out, offsets, rows, assignments, experts,
+                                               n_out, width, stream);
+}
+
+// ---------------------------------------------------------------------------
+// out[t, :] = sum over slots, in slot order, of topk_w[t, s] * y[dest[t*k + s], :]
+//             (+ shared_gate[t] * shared[t, :], or + shared[t, :] without a gate)
+// (reference: CombineRowsKernel moe.cu:237-255, AddSharedExpertKernel :275-287)
+template <typename T>
+__global__ void moe_combine_kernel(const T* __restrict__ y, const int32_t* __restrict__ dest,
+                                   const float* __restrict__ topk_w, const T* __restrict__ shared,
+                                   const float* __restrict__ shared_gate, T* __restrict__ out, int64_t width, int k) {
+  const int64_t t = blockIdx.x;
+  const float sg = shared ? (shared_gate ? shared_gate[t] : 1.0f) : 0.f;
+  for (int64_t c = threadIdx.x; c < width; c += blockDim.x) {
+    float acc = 0.f;
+    for (int s = 0; s < k; ++s) {
+      const int64_t a = t * k + s;
+      acc += topk_w[a] * ix_load(y + static_cast<int64_t>(dest[a]) * width + c);
+    }
+    if (shared) acc += sg * ix_load(shared + t * width + c);
+    ix_store(out + t * width + c, acc);
+  }
+}
+
+extern "C" int ix_moe_combine(const void* y, int dtype, const int32_t* dest, const float* topk_w, const void* shared,
+                              const float* shared_gate, void* out, int64_t tokens, int64_t width, int k,
+                              hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0 && k > 0, "sizes must be positive");
+  if (tokens == 0) return 0;
+  dim3 grid(tokens), block(256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(moe_combine_kernel<float>, grid, block, 0, stream, (const float*)y, dest, topk_w,
+                       (const float*)shared, shared_gate, (float*)out, width, k);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(moe_combine_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)y, dest, topk_w,
+                       (const bf16_t*)shared, shared_gate, (bf16_t*)out, width, k);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_moe_combine");
+}

@@ -1,0 +1,176 @@
+// Token selection on float32 logits [rows, vocab]: greedy, and temperature
+// sampling with optional top-k / top-p / min-p cut-offs.
+//
+// Order of operations follows the reference's host sampler
+// (src/engine/host_sampling.cc:50-110): temperature, softmax, cut-offs, one
+// uniform draw scaled by the kept mass, walk of the cumulative sum.  Cut-offs
+// are found as probability thresholds by bisection, the reference's device
+// variant (layers.cu:1142-1302), so tokens tied at a threshold stay together.
+// The walk is in index order, which samples the same truncated distribution.
+#include "common.h"
+
+#define SAMPLE_THREADS 1024
+
+struct ArgPair {
+  float v;
+  int i;
+};
+
+__device__ __forceinline__ ArgPair better(ArgPair a, ArgPair b) {
+  // larger value wins; equal values: lower index (reference: ArgmaxKernel, layers.cu:413-452)
+  return (b.v > a.v || (b.v == a.v && b.i < a.i)) ? b : a;
+}
+
+__device__ ArgPair block_argmax(ArgPair p, ArgPair* red) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    ArgPair o{__shfl_xor(p.v, off, 64), __shfl_xor(p.i, off, 64)};
+    p = better(p, o);
+  }
+  __syncthreads();
+  if (lane == 0) red[wave] = p;
+  __syncthreads();
+  ArgPair r = red[0];
+  for (int w = 1; w < (int)(blockDim.x >> 6); ++w) r = better(r, red[w]);
+  return r;
+}
+
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+argmax_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, int64_t vocab) {
+  __shared__ ArgPair red[16];
+  const float* row = logits + blockIdx.x * vocab;
+  ArgPair p{-INFINITY, 0x7fffffff};
+  for (int64_t i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float v = row[i];
+    if (v > p.v) { p.v = v; p.i = (int)i; }
+  }
+  p = block_argmax(p, red);
+  if (threadIdx.x == 0) out[blockIdx.x] = (p.i >= 0 && p.i < vocab) ? p.i : 0;
+}
+
+extern "C" int ix_argmax(const float* logits, int32_t* out, int64_t rows, int64_t vocab, hipStream_t stream) {
+  IX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "sizes must be positive");
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, out, vocab);
+  return ix_check_launch("ix_argmax");
+}
+
+// 64-bit mix (splitmix64 finaliser) of key and counter -> uniform in [0, 1)
+__device__ __forceinline__ float uniform_from(uint64_t key, uint64_t counter) {
+  uint64_t z = key + 0x9e3779b97f4a7c15ull * (counter + 1ull);
+  z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+  z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+  z = z ^ (z >> 31);
+  return static_cast<float>(z >> 40) * (1.0f / 16777216.0f);
+}
+
+// One workgroup per row.  temperature <= 0 means greedy for that row.
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+sample_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, const float* __restrict__ temperature,
+              const float* __restrict__ top_p, const int32_t* __restrict__ top_k, const float* __restrict__ min_p,
+              const uint64_t* __restrict__ rng_key, const uint64_t* __restrict__ rng_counter, int64_t vocab) {
+  __shared__ ArgPair ared[16];
+  __shared__ float red[16];
+  __shared__ float seg[SAMPLE_THREADS];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float* row = logits + static_cast<int64_t>(r) * vocab;
+  const float temp = temperature[r];
+
+  ArgPair best{-INFINITY, 0x7fffffff};
+  for (int64_t i = tid; i < vocab; i += SAMPLE_THREADS) {
+    const float v = row[i];
+    if (v > best.v) { best.v = v; best.i = (int)i; }
+  }
+  best = block_argmax(best, ared);
+  if (best.i < 0 || best.i >= vocab) best.i = 0;
+  if (temp <= 0.f) {
+    if (tid == 0) out[r] = best.i;
+    return;
+  }
+  const float inv_t = 1.0f / temp;
+  const float mx = best.v * inv_t;
+  // p_i = exp(l_i / t - max) in (0, 1], p_max = 1; total = sum p_i
+  float s = 0.f;
+  for (int64_t i = tid; i < vocab; i += SAMPLE_THREADS) s += expf(row[i] * inv_t - mx);
+  const float total = ix_block_sum(s, red);
+
+  // threshold on p: keep p >= thr
+  float thr = 0.f;
+  const float mp = min_p[r];
+  if (mp > 0.f) thr = fmaxf(thr, fminf(mp, 1.0f));
+  const int kk = top_k[r];
+  if (kk > 0 && kk < vocab) {
+    // largest threshold that still keeps at least kk tokens
+    float lo = 0.f, hi = 1.0f;  // count(p >= lo) >= kk always; p_max = 1
+    for (int it = 0; it < 32; ++it) {
+      const float mid = 0.5f * (lo + hi);
+      float c = 0.f;
+      for (int64_t i = tid; i < vocab; i += SAMPLE_THREADS) c += (expf(row[i] * inv_t - mx) >= mid) ? 1.f : 0.f;
+      c = ix_block_sum(c, red);
+      if (c >= (float)kk) lo = mid; else hi = mid;
+    }
+    thr = fmaxf(thr, lo);
+  }
+  const float tp = top_p[r];
+  if (tp < 1.0f) {
+    // largest threshold whose kept mass still reaches top_p
+    float lo = 0.f, hi = 1.0f;
+    for (int it = 0; it < 32; ++it) {
+      const float mid = 0.5f * (lo + hi);
+      float msum = 0.f;
+      for (int64_t i = tid; i < vocab; i += SAMPLE_THREADS) {
+        const float p = expf(row[i] * inv_t - mx);
+        msum += (p >= mid) ? p : 0.f;
+      }
+      msum = ix_block_sum(msum, red);
+      if (msum >= tp * total) lo = mid; else hi = mid;
+    }
+    thr = fmaxf(thr, lo);
+  }
+  thr = fminf(thr, 1.0f);  // the most probable token always stays
+
+  // contiguous segment per thread, kept mass per segment
+  const int64_t per = (vocab + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int64_t b = min<int64_t>(tid * per, vocab), e = min<int64_t>(b + per, vocab);
+  float mine = 0.f;
+  for (int64_t i = b; i < e; ++i) {
+    const float p = expf(row[i] * inv_t - mx);
+    mine += (p >= thr) ? p : 0.f;
+  }
+  seg[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    float mass = 0.f;
+    for (int i = 0; i < SAMPLE_THREADS; ++i) mass += seg[i];
+    const float target = uniform_from(rng_key[r], rng_counter[r]) * mass;
+    float run = 0.f;
+    int s_idx = 0;
+    for (; s_idx < SAMPLE_THREADS - 1; ++s_idx) {
+      if (run + seg[s_idx] > target) break;
+      run += seg[s_idx];
+    }
+    // walk the chosen segment; fall back to the most probable token
+    const int64_t sb = min<int64_t>((int64_t)s_idx * per, vocab), se = min<int64_t>(sb + per, vocab);
+    int pick = best.i;
+    for (int64_t i = sb; i < se; ++i) {
+      const float p = expf(row[i] * inv_t - mx);
+      if (p >= thr) {
+        run += p;
+        pick = (int)i;
+        if (run > target) break;
+      }
+    }
+    out[r] = pick;
+  }
+}
+
+extern "C" int ix_sample(const float* logits, int32_t* out, const float* temperature, const float* top_p,
+                         const int32_t* top_k, const float* min_p, const uint64_t* rng_key,
+                         const uint64_t* rng_counter, int64_t rows, int64_t vocab, hipStream_t stream) {
+  IX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "sizes must be positive");
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, out, temperature, top_p,
+                     top_k, min_p, rng_key, rng_counter, vocab);
+  return ix_check_launch("ix_sample");
+}

@@ -1,0 +1,113 @@
+"""What a run is made of besides the model: device, the activations' type, the
+library matrix product, and the per-step context that parts read.
+
+Library matrix products stand where the reference calls its vendor library
+(`CublasLtGemm::LinearBF16`, include/inferx/ops/gemm.h:68-80: y = x . W^T with
+weights [out, in] as on disk, float32 accumulation).  In a float32 run every
+product is true float32: reduced-precision matrix modes are switched off.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Dict, List, Optional
+
+import torch
+
+
+def _dtype_of(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name in (torch.float32, torch.bfloat16):
+            return name
+    table = {"float32": torch.float32, "fp32": torch.float32, "float": torch.float32,
+             "bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "auto": torch.bfloat16}
+    if name in table:
+        return table[name]
+    raise ValueError(f"dtype {name!r} is not one of float32, bfloat16")
+
+
+class Runtime:
+    def __init__(self, dtype="bfloat16", device: str = "cuda:0"):
+        self.dtype = _dtype_of(dtype)
+        self.device = torch.device(device)
+        if self.device.type != "cuda" or not torch.cuda.is_available():
+            raise RuntimeError("inferx_amd runs on a GPU only: no HIP device is visible (there is no CPU path)")
+        torch.cuda.set_device(self.device)
+        # true 32-bit products: no TF32-like or reduced-precision reduction modes
+        torch.backends.cuda.matmul.allow_tf32 = False
+        torch.backends.cudnn.allow_tf32 = False
+        torch.set_float32_matmul_precision("highest")
+        if hasattr(torch.backends.cuda.matmul, "allow_bf16_reduced_precision_reduction"):
+            torch.backends.cuda.matmul.allow_bf16_reduced_precision_reduction = False
+        from .. import ops
+        ops.lib()  # fail now, loudly, if the HIP library cannot be had
+        self._mm_out_dtype_ok: Optional[bool] = None
+
+    @property
+    def is_fp32(self) -> bool:
+        return self.dtype == torch.float32
+
+    def empty(self, shape, dtype=None) -> torch.Tensor:
+        return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)
+
+    def place(self, t: torch.Tensor) -> torch.Tensor:
+        """A loaded tensor on the device in the type it keeps for this run: in a
+        float32 run everything becomes float32 (exact); in a bfloat16 run bfloat16
+        stays, a tensor stored in 32 bits stays so, float16 is widened to float32."""
+        if t.dtype in (torch.int32, torch.int64, torch.int16, torch.int8, torch.uint8):
+            return t.to(self.device, torch.int32)
+        if self.is_fp32 or t.dtype in (torch.float32, torch.float16, torch.float64):
+            return t.to(self.device, torch.float32)
+        return t.to(self.device, torch.bfloat16)
+
+    def linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """x [T, in] . w[out, in]^T -> [T, out] in the run's type, float32 accumulation.
+        A weight kept in float32 during a bfloat16 run is multiplied in float32."""
+        if w.dtype == x.dtype:
+            return torch.matmul(x, w.t())
+        return torch.matmul(x.to(torch.float32), w.to(torch.float32).t()).to(self.dtype)
+
+    def linear_f32(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+        """As `linear`, result float32 (the logits)."""
+        if x.dtype == torch.float32 and w.dtype == torch.float32:
+            return torch.matmul(x, w.t())
+        if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+            if self._mm_out_dtype_ok is not False:
+                try:
+                    out = torch.mm(x, w.t(), out_dtype=torch.float32)
+                    self._mm_out_dtype_ok = True
+                    return out
+                except (TypeError, RuntimeError):
+                    if self._mm_out_dtype_ok:  # it worked before: a real failure
+                        raise
+                    self._mm_out_dtype_ok = False
+            return torch.matmul(x, w.t()).to(torch.float32)
+        return torch.matmul(x.to(torch.float32), w.to(torch.float32).t())
+
+
+@dataclass
+class CacheBinding:
+    """What one layer execution sees of the cache manager's memory."""
+
+    group: int = -1
+    k: Optional[torch.Tensor] = None       # [pages, kv_heads, page_size, head_dim]
+    v: Optional[torch.Tensor] = None
+    writes: bool = True                    # False: reads another execution's cache
+    state: Optional[torch.Tensor] = None   # [slots, *shape] float32
+
+
+@dataclass
+class StepContext:
+    rt: Runtime
+    num_tokens: int
+    num_requests: int
+    token_ids: torch.Tensor
+    positions: torch.Tensor
+    seq_of_token: torch.Tensor
+    q_start: torch.Tensor
+    seq_lens: torch.Tensor
+    state_slots: torch.Tensor
+    logits_rows: torch.Tensor
+    slots: List[torch.Tensor]
+    block_tables: List[torch.Tensor]
+    host: Any = None                       # the StepBatch (host arrays), for parts that plan on the host
+    memo: Dict[Any, Any] = field(default_factory=dict)  # per-step results shared between layers

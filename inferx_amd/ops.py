@@ -1,0 +1,254 @@
+"""Python face of the HIP library: one function per kernel entry point.
+
+Each function checks on the host what its kernel assumes (device, dtype,
+contiguity, shapes, index ranges where cheap), passes raw device pointers and
+the current HIP stream, and raises `KernelError` with the library's message when
+a launch is refused.  There is no fallback: without a GPU and the built library
+these functions fail.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional
+
+import torch
+
+from .csrc import build as _build
+
+F32, BF16 = 0, 1
+_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+def lib():
+    return _build.load()
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _CODE[t.dtype]
+    except KeyError:
+        raise KernelError(f"dtype {t.dtype} is not float32 or bfloat16") from None
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    if t is None:
+        return ctypes.c_void_p(0)
+    if not t.is_cuda:
+        raise KernelError("kernel operands must live on the GPU (no CPU path exists)")
+    if not t.is_contiguous():
+        raise KernelError("kernel operands must be contiguous")
+    return ctypes.c_void_p(t.data_ptr())
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _i64(v):
+    return ctypes.c_int64(int(v))
+
+
+def _i32(v):
+    return ctypes.c_int(int(v))
+
+
+def _f32(v):
+    return ctypes.c_float(float(v))
+
+
+def _call(name: str, *args):
+    fn = getattr(lib(), name)
+    rc = fn(*args)
+    if rc != 0:
+        raise KernelError(lib().ix_last_error().decode("utf-8", "replace"))
+
+
+def _need(cond: bool, msg: str):
+    if not cond:
+        raise KernelError(msg)
+
+
+def _is_i32(t, n=None):
+    _need(t.dtype == torch.int32, "index arrays must be int32")
+    if n is not None:
+        _need(t.numel() >= n, f"index array holds {t.numel()} entries, {n} needed")
+
+
+# ---------------------------------------------------------------------------
+def embed(h: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+    """h[t] = table[ids[t]]; h float32 [T, H]."""
+    T, H = h.shape
+    _need(h.dtype == torch.float32, "the residual stream is float32")
+    _need(table.dim() == 2 and table.shape[1] == H, "table width differs from h")
+    _is_i32(ids, T)
+    _call("ix_embed", _ptr(h), _ptr(table), _i32(_dt(table)), _ptr(ids), _i64(T), _i64(H), _i64(table.shape[0]),
+          _stream())
+
+
+def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, out: torch.Tensor, eps: float,
+                rows: Optional[torch.Tensor] = None) -> None:
+    """out = rmsnorm(h + delta) * weight; h += delta in place when `rows` is None.
+    With `rows`, out[r] is computed from row rows[r] and h is not changed."""
+    H = h.shape[1]
+    _need(h.dtype == torch.float32, "the residual stream is float32")
+    _need(weight.numel() == H and out.shape[1] == H, "width mismatch")
+    n_out = out.shape[0]
+    if rows is None:
+        _need(n_out == h.shape[0], "out must have a row per row of h")
+    else:
+        _is_i32(rows, n_out)
+    if delta is not None:
+        _need(delta.shape == h.shape, "delta must have the shape of h")
+    _call("ix_add_rmsnorm", _ptr(h), _ptr(delta), _i32(_dt(delta) if delta is not None else F32), _ptr(weight),
+          _i32(_dt(weight)), _ptr(out), _i32(_dt(out)), _ptr(rows), _i64(n_out), _i64(H), _f32(eps), _stream())
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, W + i]."""
+    T, W2 = gate_up.shape
+    _need(W2 % 2 == 0 and out.shape == (T, W2 // 2) and out.dtype == gate_up.dtype, "shape or dtype mismatch")
+    _call("ix_silu_mul", _ptr(gate_up), _ptr(out), _i32(_dt(out)), _i64(T), _i64(W2 // 2), _stream())
+
+
+def rope_table(cos_sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:
+    """cos_sin[t, j] = (cos, sin)(positions[t] * inv_freq[j]); float32 [T, half, 2]."""
+    T, half, two = cos_sin.shape
+    _need(two == 2 and cos_sin.dtype == torch.float32 and inv_freq.dtype == torch.float32, "float32 tables needed")
+    _need(inv_freq.numel() == half, "inv_freq length differs")
+    _is_i32(positions, T)
+    _call("ix_rope_table", _ptr(cos_sin), _ptr(positions), _ptr(inv_freq), _i64(T), _i32(half), _stream())
+
+
+def qkv_rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
+                    slots: Optional[torch.Tensor], q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
+                    v_cache: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int) -> None:
+    """Bias, rotation and cache append after the fused q/k/v product.
+    qkv [T, (heads + 2 kv_heads) * d]; caches [pages, kv_heads, page_size, d]."""
+    T = qkv.shape[0]
+    width = (heads + 2 * kv_heads) * head_dim
+    _need(qkv.shape == (T, width), f"qkv must be [T, {width}]")
+    _need(q_out.dtype == qkv.dtype and q_out.numel() == T * heads * head_dim, "q_out mismatch")
+    if bias is not None:
+        _need(bias.numel() == width, "bias length differs")
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.shape == (T, head_dim // 2, 2), "rotary table mismatch")
+    page_size, total = 1, 0
+    if k_cache is not None:
+        _need(v_cache is not None and k_cache.shape == v_cache.shape and k_cache.dtype == qkv.dtype
+              and v_cache.dtype == qkv.dtype, "cache mismatch")
+        _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim, "cache layout")
+        page_size = k_cache.shape[2]
+        total = k_cache.shape[0] * page_size
+        _need(slots is not None, "slots needed to write the cache")
+        _is_i32(slots, T)
+    _call("ix_qkv_rope_append", _ptr(qkv), _i32(_dt(qkv)), _ptr(bias), _i32(_dt(bias) if bias is not None else F32),
+          _ptr(cos_sin), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _i64(T), _i32(heads),
+          _i32(kv_heads), _i32(head_dim), _i32(page_size), _i64(total), _stream())
+
+
+def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                    seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float,
+                    window: int) -> None:
+    """Paged attention, one workgroup per (token, head).  q, out [T, heads, d]."""
+    T, heads, d = q.shape
+    _need(out.shape == q.shape and out.dtype == q.dtype, "out mismatch")
+    _need(k_cache.shape == v_cache.shape and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "cache mismatch")
+    _need(k_cache.dim() == 4 and k_cache.shape[3] == d, "cache layout")
+    kv_heads, page_size = k_cache.shape[1], k_cache.shape[2]
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    _is_i32(block_table)
+    _is_i32(seq_of_token, T)
+    _is_i32(positions, T)
+    _call("ix_attention_plain", _ptr(q), _ptr(k_cache), _ptr(v_cache), _i32(_dt(q)), _ptr(block_table),
+          _ptr(seq_of_token), _ptr(positions), _ptr(out), _i64(T), _i32(heads), _i32(kv_heads), _i32(d),
+          _i32(page_size), _i32(block_table.shape[1]), _f32(scale), _i32(window), _stream())
+
+
+def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor], topk_w: torch.Tensor,
+              topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor], renormalize: bool, scale: float) -> None:
+    """Router product, softmax and top-k in float32; optional sigmoid gate of the shared expert."""
+    T, H = x.shape
+    E = router_w.shape[0]
+    k = topk_w.shape[1]
+    _need(router_w.shape == (E, H), "router weight must be [experts, hidden]")
+    _need(topk_w.shape == (T, k) and topk_w.dtype == torch.float32, "topk_w must be float32 [T, k]")
+    _need(topk_e.shape == (T, k) and topk_e.dtype == torch.int32, "topk_e must be int32 [T, k]")
+    if shared_gate_w is not None:
+        _need(shared_gate_w.numel() == H, "shared gate weight must hold `hidden` numbers")
+        _need(shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= T,
+              "shared_gate must be float32 [T]")
+    _call("ix_moe_route", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
+          _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(topk_w), _ptr(topk_e),
+          _ptr(shared_gate if shared_gate_w is not None else None), _i64(T), _i64(H), _i32(E), _i32(k),
+          _i32(1 if renormalize else 0), _f32(scale), _stream())
+
+
+def moe_dispatch(topk_e: torch.Tensor, offsets: torch.Tensor, rows: torch.Tensor, dest: torch.Tensor,
+                 experts: int) -> None:
+    """Group assignments by expert: offsets [E+1], rows [A] (grouped row -> token), dest [A]."""
+    T, k = topk_e.shape
+    A = T * k
+    _is_i32(topk_e)
+    _is_i32(offsets, experts + 1)
+    _is_i32(rows, A)
+    _is_i32(dest, A)
+    _call("ix_moe_dispatch", _ptr(topk_e), _ptr(offsets), _ptr(rows), _ptr(dest), _i64(A), _i32(experts), _i32(k),
+          _stream())
+
+
+def moe_grouped_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
+                      rows: Optional[torch.Tensor], gate_up: bool) -> None:
+    """Grouped product over device offsets.  gate_up: a [T, H] gathered through `rows`,
+    w [E, 2n, H], out [A, n] = silu(gate) * up.  Otherwise a [A, K], w [E, n, K], out [A, n]."""
+    E = w.shape[0]
+    A, n_out = out.shape
+    K = a.shape[1]
+    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if gate_up else n_out),
+          "expert weight shape does not fit")
+    _need(out.dtype == a.dtype, "out must have the activations' dtype")
+    _is_i32(offsets, E + 1)
+    if rows is not None:
+        _is_i32(rows, A)
+    else:
+        _need(a.shape[0] >= A, "a has fewer rows than out")
+    _call("ix_moe_grouped_plain", _ptr(a), _i32(_dt(a)), _ptr(w), _i32(_dt(w)), _ptr(out), _ptr(offsets), _ptr(rows),
+          _i64(A), _i32(E), _i64(n_out), _i64(K), _i32(1 if gate_up else 0), _stream())
+
+
+def moe_combine(y: torch.Tensor, dest: torch.Tensor, topk_w: torch.Tensor, shared: Optional[torch.Tensor],
+                shared_gate: Optional[torch.Tensor], out: torch.Tensor) -> None:
+    """out[t] = sum_s topk_w[t, s] * y[dest[t, s]] (+ shared_gate[t] * shared[t])."""
+    T, k = topk_w.shape
+    H = y.shape[1]
+    _need(out.shape == (T, H) and out.dtype == y.dtype, "out mismatch")
+    _need(y.shape[0] >= T * k, "y has too few rows")
+    _is_i32(dest, T * k)
+    if shared is not None:
+        _need(shared.shape == (T, H) and shared.dtype == y.dtype, "shared mismatch")
+    _call("ix_moe_combine", _ptr(y), _i32(_dt(y)), _ptr(dest), _ptr(topk_w), _ptr(shared),
+          _ptr(shared_gate if shared is not None else None), _ptr(out), _i64(T), _i64(H), _i32(k), _stream())
+
+
+def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32, "logits must be float32")
+    _is_i32(out, R)
+    _call("ix_argmax", _ptr(logits), _ptr(out), _i64(R), _i64(V), _stream())
+
+
+def sample(logits: torch.Tensor, out: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
+           top_k: torch.Tensor, min_p: torch.Tensor, rng_key: torch.Tensor, rng_counter: torch.Tensor) -> None:
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32, "logits must be float32")
+    _is_i32(out, R)
+    _is_i32(top_k, R)
+    for t in (temperature, top_p, min_p):
+        _need(t.dtype == torch.float32 and t.numel() >= R, "sampling parameters must be float32 [rows]")
+    for t in (rng_key, rng_counter):
+        _need(t.dtype == torch.int64 and t.numel() >= R, "rng key and counter must be int64 [rows]")
+    _call("ix_sample", _ptr(logits), _ptr(out), _ptr(temperature), _ptr(top_p), _ptr(top_k), _ptr(min_p),
+          _ptr(rng_key), _ptr(rng_counter), _i64(R), _i64(V), _stream())

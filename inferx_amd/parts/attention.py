@@ -1,0 +1,85 @@
+"""Causal attention over the paged cache, grouped-query, with optional bias on
+q/k/v, an optional window and a pluggable position encoding.
+
+One fused product gives q|k|v (rows of the three weights stacked, reference
+src/model/qwen2.cc:1368-1403); one kernel adds the bias, rotates q and k and
+appends k, v to the cache (:920-969); attention reads keys [start, p] through
+the request's block table (layers.cu:256-318, window :329-407); then the output
+product (:1026-1027).
+"""
+from __future__ import annotations
+
+from typing import List, Optional
+
+from .. import ops
+from ..config.spec import PartSpec
+from .base import CacheNeed, Mixer, ParamSpec, build_part, register_part
+from .dense_mlp import stack_rows
+
+
+class PagedAttention(Mixer):
+    def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, qkv_bias: bool = True,
+                 out_bias: bool = False, window: int = 0, scale: Optional[float] = None,
+                 position: Optional[PartSpec] = None, init_std: float = 0.02):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
+        if head_dim % 2 or head_dim > 256:
+            raise ValueError(f"head_dim {head_dim} must be even and at most 256")
+        if out_bias:
+            raise ValueError("a bias on the output projection is not supported")
+        self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
+        self.head_dim, self.qkv_bias, self.window = int(head_dim), bool(qkv_bias), int(window)
+        self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
+        self.init_std = float(init_std)
+        self.position = build_part("position", position) if position is not None else None
+        if self.position is not None and getattr(self.position, "rotary_dim", self.head_dim) != self.head_dim:
+            raise ValueError("rotation of part of a head is not supported: rotary_dim must equal head_dim")
+        self.w_qkv = self.b_qkv = self.w_out = None
+
+    @property
+    def q_dim(self) -> int:
+        return self.num_heads * self.head_dim
+
+    @property
+    def kv_dim(self) -> int:
+        return self.num_kv_heads * self.head_dim
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+
+    def param_specs(self) -> List[ParamSpec]:
+        H, s = self.hidden_size, self.init_std
+        specs = [ParamSpec("q_proj.weight", (self.q_dim, H), std=s), ParamSpec("k_proj.weight", (self.kv_dim, H), std=s),
+                 ParamSpec("v_proj.weight", (self.kv_dim, H), std=s), ParamSpec("o_proj.weight", (H, self.q_dim), std=s)]
+        if self.qkv_bias:
+            specs += [ParamSpec("q_proj.bias", (self.q_dim,), std=s), ParamSpec("k_proj.bias", (self.kv_dim,), std=s),
+                      ParamSpec("v_proj.bias", (self.kv_dim,), std=s)]
+        return specs
+
+    def bind(self, tensors, rt) -> None:
+        self.w_qkv = stack_rows([tensors[f"{n}_proj.weight"] for n in "qkv"])
+        self.b_qkv = stack_rows([tensors[f"{n}_proj.bias"] for n in "qkv"]) if self.qkv_bias else None
+        self.w_out = tensors["o_proj.weight"].contiguous()
+        if self.position is not None:
+            self.position.bind({}, rt)
+
+    def forward(self, ctx, x, cache):
+        rt = ctx.rt
+        T = x.shape[0]
+        qkv = rt.linear(x, self.w_qkv)
+        table = self.position.prepare(ctx) if self.position is not None else None
+        q = rt.empty((T, self.num_heads, self.head_dim))
+        writes = cache.writes
+        ops.qkv_rope_append(qkv, self.b_qkv, table, ctx.slots[cache.group] if writes else None, q,
+                            cache.k if writes else None, cache.v if writes else None,
+                            self.num_heads, self.num_kv_heads, self.head_dim)
+        out = rt.empty((T, self.num_heads, self.head_dim))
+        self.attend(ctx, q, cache, out)
+        return rt.linear(out.view(T, self.q_dim), self.w_out)
+
+    def attend(self, ctx, q, cache, out) -> None:
+        ops.attention_plain(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.seq_of_token, ctx.positions, out,
+                            self.scale, self.window)
+
+
+register_part("mixer", "attention", PagedAttention)

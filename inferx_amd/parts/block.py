@@ -1,0 +1,22 @@
+"""Arrangement of a layer's parts.  `prenorm`:
+
+    h += pending;  a = mixer(norm1(h));  h += a;  f = feed_forward(norm2(h));  pending = f
+
+(reference: src/model/qwen2.cc:908-1051).  The residual stream h is float32 and
+is updated inside the norm kernel, so each add is fused with the norm after it;
+the last pending delta is added by the model's final norm.
+"""
+from __future__ import annotations
+
+from .base import Block, register_part
+
+
+class PreNormBlock(Block):
+    def forward(self, ctx, h, pending, cache):
+        x = self.mixer_norm.forward(ctx, h, pending)
+        a = self.mixer.forward(ctx, x, cache)
+        x = self.feed_forward_norm.forward(ctx, h, a)
+        return self.feed_forward.forward(ctx, x)
+
+
+register_part("block", "prenorm", PreNormBlock)

@@ -1,0 +1,110 @@
+"""Mixture-of-experts feed-forward with an optional (sigmoid-gated) shared expert.
+
+route -> group -> gate|up of the routed experts (+SwiGLU) -> down -> weighted
+sum in slot order + shared expert (reference: MoeFfn::ForwardImpl,
+src/model/moe_ffn.cc:158-367; kernels src/backends/cuda/ops/moe.cu).  Expert
+weights are stacked at load: w13 [E, 2*mi, H] (gate rows, then up rows, per
+expert) and w2 [E, H, mi] (reference: moe_ffn.h:25-34; stacking pattern
+src/model/deepseek_v2.cc:515-542).  Router scores and the shared gate are
+float32 from the product on.
+"""
+from __future__ import annotations
+
+from typing import List
+
+import torch
+
+from .. import ops
+from .base import FeedForward, ParamSpec, register_part
+from .dense_mlp import stack_rows
+
+
+class MoeFeedForward(FeedForward):
+    def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_width: int, shared_width: int = 0,
+                 shared_gated: bool = True, renormalize: bool = False, routed_scale: float = 1.0,
+                 init_std: float = 0.02):
+        if not 0 < top_k <= num_experts:
+            raise ValueError(f"top_k {top_k} must be between 1 and num_experts {num_experts}")
+        if num_experts > 1024 or top_k > 32:
+            raise ValueError("at most 1024 experts and top_k 32 are supported")
+        self.hidden_size, self.num_experts, self.top_k = int(hidden_size), int(num_experts), int(top_k)
+        self.expert_width, self.shared_width = int(expert_width), int(shared_width)
+        self.shared_gated, self.renormalize = bool(shared_gated), bool(renormalize)
+        self.routed_scale, self.init_std = float(routed_scale), float(init_std)
+        self.w_router = self.w13 = self.w2 = None
+        self.w_shared_gate_up = self.w_shared_down = self.w_shared_gate = None
+
+    def param_specs(self) -> List[ParamSpec]:
+        H, mi, si, s = self.hidden_size, self.expert_width, self.shared_width, self.init_std
+        specs = [ParamSpec("gate.weight", (self.num_experts, H), std=s)]
+        for e in range(self.num_experts):
+            specs += [ParamSpec(f"experts.{e}.gate_proj.weight", (mi, H), std=s),
+                      ParamSpec(f"experts.{e}.up_proj.weight", (mi, H), std=s),
+                      ParamSpec(f"experts.{e}.down_proj.weight", (H, mi), std=s)]
+        if si > 0:
+            specs += [ParamSpec("shared_expert.gate_proj.weight", (si, H), std=s),
+                      ParamSpec("shared_expert.up_proj.weight", (si, H), std=s),
+                      ParamSpec("shared_expert.down_proj.weight", (H, si), std=s)]
+            if self.shared_gated:
+                specs.append(ParamSpec("shared_expert_gate.weight", (1, H), std=s))
+        return specs
+
+    def bind(self, tensors, rt) -> None:
+        E = self.num_experts
+        self.w_router = tensors["gate.weight"].contiguous()
+        parts = []
+        for e in range(E):
+            parts += [tensors[f"experts.{e}.gate_proj.weight"], tensors[f"experts.{e}.up_proj.weight"]]
+        self.w13 = stack_rows(parts).view(E, 2 * self.expert_width, self.hidden_size)
+        self.w2 = stack_rows([tensors[f"experts.{e}.down_proj.weight"] for e in range(E)]).view(
+            E, self.hidden_size, self.expert_width)
+        if self.shared_width > 0:
+            self.w_shared_gate_up = stack_rows([tensors["shared_expert.gate_proj.weight"],
+                                                tensors["shared_expert.up_proj.weight"]])
+            self.w_shared_down = tensors["shared_expert.down_proj.weight"].contiguous()
+            if self.shared_gated:
+                self.w_shared_gate = tensors["shared_expert_gate.weight"].contiguous()
+
+    # -- the steps, separately callable so tests can look between them ----
+    def route(self, ctx, x):
+        rt, T, k = ctx.rt, x.shape[0], self.top_k
+        topk_w = rt.empty((T, k), torch.float32)
+        topk_e = rt.empty((T, k), torch.int32)
+        gate = rt.empty((T,), torch.float32) if self.w_shared_gate is not None else None
+        ops.moe_route(x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate, self.renormalize, self.routed_scale)
+        return topk_w, topk_e, gate
+
+    def dispatch(self, ctx, topk_e):
+        rt, A = ctx.rt, topk_e.numel()
+        offsets = rt.empty((self.num_experts + 1,), torch.int32)
+        rows = rt.empty((A,), torch.int32)
+        dest = rt.empty((A,), torch.int32)
+        ops.moe_dispatch(topk_e, offsets, rows, dest, self.num_experts)
+        return offsets, rows, dest
+
+    def experts(self, ctx, x, offsets, rows):
+        rt, A = ctx.rt, rows.numel()
+        act = rt.empty((A, self.expert_width))
+        ops.moe_grouped_plain(x, self.w13, act, offsets, rows, gate_up=True)
+        y = rt.empty((A, self.hidden_size))
+        ops.moe_grouped_plain(act, self.w2, y, offsets, None, gate_up=False)
+        return y
+
+    def shared(self, ctx, x):
+        rt = ctx.rt
+        gate_up = rt.linear(x, self.w_shared_gate_up)
+        act = rt.empty((x.shape[0], self.shared_width))
+        ops.silu_mul(gate_up, act)
+        return rt.linear(act, self.w_shared_down)
+
+    def forward(self, ctx, x):
+        topk_w, topk_e, gate = self.route(ctx, x)
+        offsets, rows, dest = self.dispatch(ctx, topk_e)
+        y = self.experts(ctx, x, offsets, rows)
+        shared = self.shared(ctx, x) if self.shared_width > 0 else None
+        out = ctx.rt.empty((x.shape[0], self.hidden_size))
+        ops.moe_combine(y, dest, topk_w, shared, gate, out)
+        return out
+
+
+register_part("feed_forward", "moe", MoeFeedForward)

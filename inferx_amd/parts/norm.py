@@ -1,0 +1,34 @@
+"""RMSNorm, fused with the residual add that precedes it.
+
+y = v * rsqrt(mean(v^2) + eps) * weight with v = h + delta, everything in
+float32, rounded once (reference: RmsNormKernel, src/backends/cuda/ops/layers.cu:50-76).
+"""
+from __future__ import annotations
+
+from typing import List
+
+from .. import ops
+from .base import Norm, ParamSpec, register_part
+
+
+class RMSNorm(Norm):
+    def __init__(self, width: int, eps: float):
+        self.width, self.eps = int(width), float(eps)
+        self.weight = None
+
+    def param_specs(self) -> List[ParamSpec]:
+        return [ParamSpec("weight", (self.width,), init="ones")]
+
+    def bind(self, tensors, rt) -> None:
+        self.weight = tensors["weight"].contiguous()
+
+    def forward(self, ctx, h, delta=None, rows=None):
+        """h [T, width] float32 is updated in place with `delta` (unless `rows`
+        picks rows out); returns the normalised rows in the run's type."""
+        n = h.shape[0] if rows is None else rows.numel()
+        out = ctx.rt.empty((n, self.width))
+        ops.add_rmsnorm(h, delta, self.weight, out, self.eps, rows)
+        return out
+
+
+register_part("norm", "rmsnorm", RMSNorm)

@@ -1,0 +1,46 @@
+"""Rotary position encoding, half-split pairing (j, j + d/2).
+
+f_j = theta^(-2j/d), angle = position * f_j; the rotation itself is fused into
+the kernel that follows the q/k/v product (reference: RopeKernel,
+src/backends/cuda/ops/layers.cu:80-115; ops/layers.h:35-58).  The frequencies
+are computed once in float64 and rounded to float32; the angle and its cosine
+and sine are float32, once per step for all layers.
+
+Interface of a position encoding: `prepare(ctx)` returns a float32 table
+[T, d/2, 2] of (cos, sin) for this step's tokens, or None for no rotation.
+"""
+from __future__ import annotations
+
+import torch
+
+from .. import ops
+from .base import PositionEncoding, register_part
+
+
+class Rotary(PositionEncoding):
+    def __init__(self, theta: float, rotary_dim: int):
+        if rotary_dim <= 0 or rotary_dim % 2:
+            raise ValueError(f"rotary_dim {rotary_dim} must be positive and even")
+        if theta <= 0:
+            raise ValueError("theta must be positive")
+        self.theta, self.rotary_dim = float(theta), int(rotary_dim)
+        self.inv_freq = None
+
+    def frequencies(self) -> torch.Tensor:
+        j = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
+        return torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * j / self.rotary_dim).to(torch.float32)
+
+    def bind(self, tensors, rt) -> None:
+        self.inv_freq = self.frequencies().to(rt.device)
+
+    def prepare(self, ctx):
+        key = ("rope", self.theta, self.rotary_dim)
+        table = ctx.memo.get(key)
+        if table is None:
+            table = ctx.rt.empty((ctx.num_tokens, self.rotary_dim // 2, 2), torch.float32)
+            ops.rope_table(table, ctx.positions, self.inv_freq)
+            ctx.memo[key] = table
+        return table
+
+
+register_part("position", "rope", Rotary)

@@ -1,0 +1,55 @@
+"""Binding a checkpoint's tensors to a model by name.
+
+The model says what it needs (`DecoderModel.expected_tensors`); the loader
+compares that with what the folder holds and raises ONE error that lists every
+missing tensor, every unexpected one and every wrong shape (the reference
+reports them one at a time: NotFound `src/model/safetensors.cc:389-392`, shape
+mismatch `:417-421`).  Tensors keep their stored floating type in a bfloat16
+run (bfloat16 stays, 32-bit stays 32-bit) and all become float32 in a float32
+run; integer tables become int32.
+"""
+from __future__ import annotations
+
+from typing import Dict, List
+
+import torch
+
+from .safetensors_io import Checkpoint, CheckpointError
+
+# tensors some writers add that no part asks for
+_IGNORED_SUFFIXES = ("rotary_emb.inv_freq",)
+
+
+def check_names_and_shapes(expected: Dict[str, tuple], ckpt: Checkpoint, tied_head_name: str = "lm_head.weight",
+                           head_is_tied: bool = False) -> None:
+    missing: List[str] = sorted(n for n in expected if n not in ckpt)
+    unexpected = sorted(
+        n for n in ckpt.names()
+        if n not in expected and not n.endswith(_IGNORED_SUFFIXES) and not (head_is_tied and n == tied_head_name))
+    wrong = sorted(
+        f"{n}: expected {list(expected[n])}, file has {list(ckpt.shape(n))}"
+        for n in expected if n in ckpt and tuple(ckpt.shape(n)) != tuple(expected[n]))
+    bad_type = sorted(f"{n}: {ckpt.dtype(n)}" for n in expected
+                      if n in ckpt and not ckpt.dtype(n).is_floating_point)
+    if not (missing or unexpected or wrong or bad_type):
+        return
+
+    def block(title, items):
+        if not items:
+            return ""
+        shown = items[:40]
+        more = f"\n    ... and {len(items) - 40} more" if len(items) > 40 else ""
+        return f"\n  {title} ({len(items)}):\n    " + "\n    ".join(shown) + more
+
+    raise CheckpointError(
+        "the checkpoint does not fit the model:"
+        + block("missing tensors", missing) + block("unexpected tensors", unexpected)
+        + block("wrong shapes", wrong) + block("not floating point", bad_type))
+
+
+def load_weights(model, model_dir: str, rt) -> Dict[str, torch.Tensor]:
+    """All tensors the model needs, on the device, keyed by checkpoint name."""
+    ckpt = Checkpoint.open(model_dir)
+    expected = {name: tuple(p.shape) for name, p in model.expected_tensors().items()}
+    check_names_and_shapes(expected, ckpt, head_is_tied=model.spec.head_name is None)
+    return {name: rt.place(ckpt.get(name)) for name in expected}

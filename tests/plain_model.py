@@ -1,0 +1,237 @@
+"""The plain implementation: Qwen2-MoE written the obvious way, on the CPU, in
+float64, whole sequences, no cache, no batching, one function per part.
+
+It shares no code with `inferx_amd`: it reads config.json keys and checkpoint
+tensor names itself.  Every function cites the place in the reference
+(/root/reference, paths relative to it) whose formula it follows.  The
+reference was read, not run.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+F64 = torch.float64
+
+
+# --------------------------------------------------------------------------
+def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """y_i = x_i * rsqrt(sum(x^2)/H + eps) * w_i
+    src/backends/cuda/ops/layers.cu:50-76 (RmsNormKernel: sumsq / hidden + eps, rsqrtf, x*inv*w)."""
+    inv = torch.rsqrt((x * x).sum(-1, keepdim=True) / x.shape[-1] + eps)
+    return x * inv * weight
+
+
+def rope_frequencies(theta: float, head_dim: int) -> torch.Tensor:
+    """inv_freq[j] = theta^(-2j/d), j < d/2.   layers.cu:93-94 (RopeKernel).
+    Rounded to float32 as a device table would hold it."""
+    j = torch.arange(head_dim // 2, dtype=F64)
+    return (theta ** (-2.0 * j / head_dim)).to(torch.float32).to(F64)
+
+
+def apply_rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.Tensor:
+    """Half-split rotation: pairs (j, j + d/2);
+    x'_j = x_j cos a - x_{j+d/2} sin a;  x'_{j+d/2} = x_{j+d/2} cos a + x_j sin a;  a = pos * inv_freq[j].
+    layers.cu:80-115 (RopeKernel: lo*c - hi*s, hi*c + lo*s).   x: [T, heads, d]."""
+    d = x.shape[-1]
+    half = d // 2
+    # the angle is formed in float32 (float(pos) * inv_freq), layers.cu:87, 95
+    angle = (positions.to(torch.float32)[:, None] * rope_frequencies(theta, d).to(torch.float32)[None, :]).to(F64)
+    c, s = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
+    lo, hi = x[..., :half], x[..., half:]
+    return torch.cat([lo * c - hi * s, hi * c + lo * s], dim=-1)
+
+
+def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor, scale: float,
+              window: int = 0) -> torch.Tensor:
+    """Causal grouped-query attention, by position, no mask tensor.
+    Query head h reads kv head h // (heads // kv_heads); a query at position p reads keys [start, p],
+    start = 0 or, with a window W, max(0, p + 1 - W); s_j = (q . k_j) * scale; softmax with the maximum
+    subtracted; o = sum(e_j v_j) / sum(e_j).
+    layers.cu:329-407 (PagedAttentionWithLseKernel; window :346-354; contiguous variant :133-191).
+    q: [T, heads, d]; k, v: [T, kv_heads, d]."""
+    T, heads, d = q.shape
+    kv_heads = k.shape[1]
+    group = heads // kv_heads
+    out = torch.zeros_like(q)
+    for t in range(T):
+        p = int(positions[t])
+        start = p + 1 - window if (window > 0 and p + 1 > window) else 0
+        keys = torch.tensor([j for j in range(T) if start <= int(positions[j]) <= p])
+        for h in range(heads):
+            g = h // group
+            s = (k[keys, g] @ q[t, h]) * scale
+            e = torch.exp(s - s.max())
+            out[t, h] = (e[:, None] * v[keys, g]).sum(0) / e.sum()
+    return out
+
+
+def silu(g: torch.Tensor) -> torch.Tensor:
+    """silu(g) = g / (1 + exp(-g)).   layers.cu:512-529 (SiluMulFusedKernel)."""
+    return g / (1.0 + torch.exp(-g))
+
+
+def gated_mlp(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+    """y = (silu(x Wg^T) * (x Wu^T)) Wd^T.   src/model/qwen2.cc:1042-1048; weights [out, in], gemm.h:51-57."""
+    return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
+
+
+def route(x: torch.Tensor, w_router: torch.Tensor, top_k: int, renormalize: bool,
+          scale: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+    """p = softmax(x Wr^T) over all experts; k rounds of argmax with strict '>' (lowest index wins a tie),
+    chosen weight = p_e, chosen expert masked to -inf; optional division by the sum of the chosen; times scale.
+    src/backends/cuda/ops/moe.cu:36-127 (RouteTopKKernel); src/model/moe_ffn.cc:200-221.
+    Returns weights [T, k] and experts [T, k], slots in descending score."""
+    z = x @ w_router.T
+    T, E = z.shape
+    weights = torch.zeros(T, top_k, dtype=x.dtype)
+    experts = torch.zeros(T, top_k, dtype=torch.int64)
+    for t in range(T):
+        e = torch.exp(z[t] - z[t].max())
+        inv_sum = 1.0 / e.sum()
+        row = e.clone()
+        total = 0.0
+        for slot in range(top_k):
+            best, best_value = -1, -math.inf
+            for i in range(E):
+                if float(row[i]) > best_value:
+                    best_value, best = float(row[i]), i
+            weights[t, slot] = best_value * inv_sum
+            total += float(weights[t, slot])
+            experts[t, slot] = best
+            row[best] = -math.inf
+        if renormalize and total > 0:
+            weights[t] = weights[t] / total
+        weights[t] = weights[t] * scale
+    return weights, experts
+
+
+def moe_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, num_experts: int, top_k: int,
+              renormalize: bool, shared_width: int) -> torch.Tensor:
+    """Every chosen expert applied per token and summed in slot order, plus the sigmoid-gated shared expert:
+    out_t = sum_slot w_{t,slot} * MLP_e(x_t)  +  sigmoid(x_t . Wsg) * MLP_shared(x_t).
+    src/model/moe_ffn.cc:158-367 (route, experts, combine :305-306, shared :308-351);
+    moe.cu:237-255 (CombineRowsKernel), :275-287 (AddSharedExpertKernel: 1/(1+exp(-g)))."""
+    weights, experts = route(x, w[prefix + "gate.weight"], top_k, renormalize)
+    out = torch.zeros_like(x)
+    for t in range(x.shape[0]):
+        for slot in range(top_k):
+            e = int(experts[t, slot])
+            p = f"{prefix}experts.{e}."
+            out[t] += weights[t, slot] * gated_mlp(x[t:t + 1], w[p + "gate_proj.weight"], w[p + "up_proj.weight"],
+                                                   w[p + "down_proj.weight"])[0]
+    if shared_width > 0:
+        p = prefix + "shared_expert."
+        shared = gated_mlp(x, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+        gate = 1.0 / (1.0 + torch.exp(-(x @ w[prefix + "shared_expert_gate.weight"].T)))  # [T, 1]
+        out = out + gate * shared
+    return out
+
+
+# --------------------------------------------------------------------------
+def is_moe_layer(cfg: dict, layer: int) -> bool:
+    """Sparse unless listed in mlp_only_layers or (layer + 1) % decoder_sparse_step != 0.
+    The reference's rule is another architecture's (include/inferx/model/config.h:121-126); these two keys are the
+    Qwen2-MoE ones, which the reference never reads."""
+    if layer in (cfg.get("mlp_only_layers") or []):
+        return False
+    return cfg.get("num_experts", 0) > 0 and (layer + 1) % cfg.get("decoder_sparse_step", 1) == 0
+
+
+def window_of_layer(cfg: dict, layer: int) -> int:
+    """Windowed iff use_sliding_window and layer >= max_window_layers (window semantics layers.cu:346-354)."""
+    if cfg.get("use_sliding_window", False) and cfg.get("sliding_window", 0) and \
+            layer >= cfg.get("max_window_layers", cfg["num_hidden_layers"]):
+        return int(cfg["sliding_window"])
+    return 0
+
+
+def forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequence[int],
+            positions: Optional[Sequence[int]] = None,
+            schedule: Optional[List[Tuple[int, Optional[int]]]] = None) -> torch.Tensor:
+    """Logits [T, vocab] of one whole sequence.  Layer order and the place of every norm and residual:
+    src/model/qwen2.cc:902-1066 (embed :902; input norm :912; qkv + bias :920-923; rope :925-926; attention
+    :1021-1023; o_proj + residual :1026-1030; post norm :1036; feed-forward :1042-1048; residual :1051; final norm
+    and head :1059-1066).  `schedule`: (layer, cache_from) per execution, default each layer once."""
+    w = {k: v.to(F64) for k, v in weights.items()}
+    H = cfg["hidden_size"]
+    heads = cfg["num_attention_heads"]
+    kv_heads = cfg.get("num_key_value_heads", heads)
+    d = cfg.get("head_dim") or H // heads
+    eps = cfg.get("rms_norm_eps", 1e-6)
+    theta = float(cfg.get("rope_theta", 10000.0))
+    T = len(token_ids)
+    pos = torch.arange(T) if positions is None else torch.tensor(list(positions))
+    scale = 1.0 / math.sqrt(d)  # qwen2.cc:890
+    h = w["model.embed_tokens.weight"][torch.tensor(list(token_ids))]  # layers.cu:465-481
+    if schedule is None:
+        schedule = [(l, None) for l in range(cfg["num_hidden_layers"])]
+    kept: List[Tuple[torch.Tensor, torch.Tensor]] = []
+    for layer, cache_from in schedule:
+        p = f"model.layers.{layer}."
+        x = rms_norm(h, w[p + "input_layernorm.weight"], eps)
+        a = p + "self_attn."
+        q = x @ w[a + "q_proj.weight"].T
+        k = x @ w[a + "k_proj.weight"].T
+        v = x @ w[a + "v_proj.weight"].T
+        if a + "q_proj.bias" in w:  # SplitQkvKernel adds the bias after the product, layers.cu:485-510
+            q, k, v = q + w[a + "q_proj.bias"], k + w[a + "k_proj.bias"], v + w[a + "v_proj.bias"]
+        q = apply_rope(q.view(T, heads, d), pos, theta)
+        k = apply_rope(k.view(T, kv_heads, d), pos, theta)  # rotated keys are what is cached, qwen2.cc:928-969
+        v = v.view(T, kv_heads, d)
+        if cache_from is not None:
+            k, v = kept[cache_from]
+        kept.append((k, v))
+        att = attention(q, k, v, pos, scale, window_of_layer(cfg, layer))
+        h = h + att.reshape(T, heads * d) @ w[a + "o_proj.weight"].T
+        x = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
+        m = p + "mlp."
+        if is_moe_layer(cfg, layer):
+            f = moe_block(x, w, m, cfg["num_experts"], cfg["num_experts_per_tok"],
+                          bool(cfg.get("norm_topk_prob", False)), cfg.get("shared_expert_intermediate_size", 0))
+        else:
+            f = gated_mlp(x, w[m + "gate_proj.weight"], w[m + "up_proj.weight"], w[m + "down_proj.weight"])
+        h = h + f
+    x = rms_norm(h, w["model.norm.weight"], eps)
+    head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
+    return x @ head.T
+
+
+# --------------------------------------------------------------------------
+def greedy(logits_row: torch.Tensor) -> int:
+    """First maximum, lowest index on ties.   src/engine/host_sampling.cc:52-53; layers.cu:413-452."""
+    best, best_value = 0, -math.inf
+    for i, v in enumerate(logits_row.tolist()):
+        if v > best_value:
+            best, best_value = i, v
+    return best
+
+
+def sampling_support(logits_row: torch.Tensor, temperature: float, top_k: int = 0, top_p: float = 1.0,
+                     min_p: float = 0.0) -> List[int]:
+    """Token ids that temperature sampling with the given cut-offs may return.
+    p = softmax(logits / t); sort descending (ties by index); keep the first top_k, then those with
+    p >= min_p * p_max, then the smallest prefix whose mass reaches top_p.
+    src/engine/host_sampling.cc:60-97."""
+    p = torch.softmax(logits_row.to(F64) / temperature, dim=-1)
+    order = sorted(range(p.numel()), key=lambda i: (-float(p[i]), i))
+    keep = len(order)
+    if top_k > 0:
+        keep = min(keep, top_k)
+    if min_p > 0:
+        floor = min_p * float(p[order[0]])
+        n = 0
+        while n < keep and float(p[order[n]]) >= floor:
+            n += 1
+        keep = max(n, 1)
+    if top_p < 1.0:
+        mass, n = 0.0, 0
+        while n < keep:
+            mass += float(p[order[n]])
+            n += 1
+            if mass >= top_p:
+                break
+        keep = max(n, 1)
+    return order[:keep]

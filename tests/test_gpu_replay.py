@@ -1,0 +1,88 @@
+"""The engine against the plain implementation, four ways of running each request,
+in float32 and in bfloat16, on two tiny configurations that differ in every size."""
+import pytest
+import torch
+
+import replay_util as ru
+import tiny
+
+pytestmark = pytest.mark.gpu
+
+PROMPT_LENGTHS = {"A": (5, 9, 17, 70), "B": (7, 23, 40, 75), "C": (11, 50)}
+
+
+@pytest.fixture(scope="module")
+def folders(tmp_path_factory):
+    out = {}
+    for name, cfg in tiny.CONFIGS.items():
+        for dtype in ("float32", "bfloat16"):
+            d = tmp_path_factory.mktemp(f"model_{name}_{dtype}")
+            tiny.make_folder(cfg, seed=11, out_dir=str(d), dtype=dtype)
+            out[(name, dtype)] = str(d)
+    return out
+
+
+def prompts_for(name):
+    cfg = tiny.CONFIGS[name]
+    return {f"r{i}": tiny.random_tokens(n, cfg["vocab_size"], seed=100 + i)
+            for i, n in enumerate(PROMPT_LENGTHS[name])}
+
+
+_expected_cache = {}
+
+
+def expected_for(folders, name, dtype):
+    key = (name, dtype)
+    if key not in _expected_cache:
+        cfg, weights = tiny.read_folder(folders[key])
+        _expected_cache[key] = ru.expected_logits(cfg, weights, prompts_for(name))
+    return _expected_cache[key]
+
+
+def make_runner(folders, name, dtype, num_pages=64, page_size=16):
+    from inferx_amd.engine.runner import ModelRunner
+    return ModelRunner.from_directory(folders[(name, dtype)], dtype=dtype, page_size=page_size, num_pages=num_pages,
+                                      max_requests=4, max_seq_len=num_pages * page_size)
+
+
+def tol_of(dtype):
+    return ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_whole(folders, name, dtype):
+    runner = make_runner(folders, name, dtype)
+    got = ru.replay(runner, ru.whole(prompts_for(name)))
+    worst = ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"whole {name} {dtype}")
+    print(f"whole {name} {dtype}: worst {worst:.2e}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_last_tokens_one_by_one(folders, name, dtype):
+    runner = make_runner(folders, name, dtype)
+    got = ru.replay(runner, ru.tail_decoded(prompts_for(name), 32))
+    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"tail {name} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_portions_of_changing_size(folders, name, dtype):
+    runner = make_runner(folders, name, dtype)
+    got = ru.replay(runner, ru.chunked(prompts_for(name)))
+    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"chunked {name} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_mixed_with_few_pages(folders, name, dtype):
+    prompts = prompts_for(name)
+    # room for about two of the longer requests: pages are given back and used again
+    max_tokens = 192
+    runner = make_runner(folders, name, dtype, num_pages=max_tokens // 16)
+    used = set()
+    steps = ru.mixed(prompts, seed=5, max_tokens=max_tokens)
+    got = ru.replay(runner, steps)
+    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"mixed {name} {dtype}")
+    assert all(p.used_pages == 0 for p in runner.cache.pools)

@@ -1,0 +1,60 @@
+"""Two tiny Qwen2-MoE configurations that differ in every size and option, and
+helpers that make a model folder and read it back for the plain implementation."""
+import json
+import os
+
+import torch
+
+CONFIG_A = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "num_hidden_layers": 2, "hidden_size": 64, "num_attention_heads": 4, "num_key_value_heads": 2, "head_dim": 16,
+    "num_experts": 4, "num_experts_per_tok": 2, "moe_intermediate_size": 32, "shared_expert_intermediate_size": 64,
+    "intermediate_size": 128, "decoder_sparse_step": 1, "mlp_only_layers": [], "norm_topk_prob": False,
+    "vocab_size": 256, "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 128,
+    "use_sliding_window": False, "tie_word_embeddings": False,
+}
+
+CONFIG_B = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "num_hidden_layers": 4, "hidden_size": 96, "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 32,
+    "num_experts": 8, "num_experts_per_tok": 3, "moe_intermediate_size": 48, "shared_expert_intermediate_size": 80,
+    "intermediate_size": 160, "decoder_sparse_step": 2, "mlp_only_layers": [0], "norm_topk_prob": True,
+    "vocab_size": 384, "rope_theta": 1000000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 256,
+    "use_sliding_window": True, "sliding_window": 16, "max_window_layers": 2, "tie_word_embeddings": True,
+}
+
+# sizes that are no power of two and no multiple of 16 where the architecture allows it
+CONFIG_C = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "num_hidden_layers": 3, "hidden_size": 72, "num_attention_heads": 6, "num_key_value_heads": 3, "head_dim": 48,
+    "num_experts": 5, "num_experts_per_tok": 1, "moe_intermediate_size": 40, "shared_expert_intermediate_size": 0,
+    "intermediate_size": 104, "decoder_sparse_step": 1, "mlp_only_layers": [1], "norm_topk_prob": False,
+    "vocab_size": 301, "rope_theta": 50000.0, "rms_norm_eps": 1e-5, "max_position_embeddings": 512,
+    "use_sliding_window": True, "sliding_window": 24, "max_window_layers": 1, "tie_word_embeddings": False,
+    "qkv_bias": False,
+}
+
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
+
+
+def make_folder(raw_config: dict, seed: int, out_dir: str, dtype: str = "bfloat16", std_scale: float = 1.0) -> str:
+    from inferx_amd.config import config_from_dict
+    from inferx_amd.weights import write_model_folder
+    raw = dict(raw_config)
+    if std_scale != 1.0:
+        raw["initializer_range"] = 0.02 * std_scale
+    write_model_folder(config_from_dict(raw), seed, out_dir, dtype)
+    return out_dir
+
+
+def read_folder(model_dir: str):
+    """config dict and tensors, through the safetensors library (not the framework's reader)."""
+    from safetensors.torch import load_file
+    with open(os.path.join(model_dir, "config.json")) as f:
+        cfg = json.load(f)
+    return cfg, load_file(os.path.join(model_dir, "model.safetensors"))
+
+
+def random_tokens(n: int, vocab: int, seed: int):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
