@@ -1,0 +1,199 @@
+"""Decode and prefill throughput at the Qwen1.5-MoE-A2.7B shape, random weights.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
+
+A step is one decode step of the whole batch through the model runner (batch
+build, upload, every kernel, greedy choice of the next tokens).  Prints ONE
+JSON line: decoded tokens a second at the default batch, the prefill of one
+2,048-token prompt, the decode step's HBM roofline fraction, and decode at
+batch 1 and 64.  One GPU only.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# Qwen1.5-MoE-A2.7B's sizes
+SHAPE = {
+    "architectures": ["Qwen2MoeForCausalLM"], "num_hidden_layers": 24, "hidden_size": 2048,
+    "num_attention_heads": 16, "num_key_value_heads": 16, "head_dim": 128, "num_experts": 60,
+    "num_experts_per_tok": 4, "moe_intermediate_size": 1408, "shared_expert_intermediate_size": 5632,
+    "intermediate_size": 5632, "decoder_sparse_step": 1, "mlp_only_layers": [], "norm_topk_prob": False,
+    "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 8192,
+    "use_sliding_window": False, "tie_word_embeddings": False,
+}
+CONTEXT = 4096
+PROMPT = 2048
+PAGE = 16
+PEAK_HBM_GBS = 8000.0
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+
+def log(msg):
+    print(f"[bench] {msg}", file=sys.stderr, flush=True)
+
+
+def decode_bytes(cfg, batch, context, elt):
+    """Bytes one decode step has to read: every weight it uses once, and the cache of the live requests."""
+    H, L = cfg.hidden_size, cfg.num_hidden_layers
+    qd, kvd = cfg.q_dim, cfg.kv_dim
+    E, k, mi, si = cfg.num_experts, cfg.num_experts_per_tok, cfg.moe_intermediate_size, cfg.shared_expert_intermediate_size
+    distinct = E * (1.0 - (1.0 - k / E) ** batch)  # expected number of experts a batch touches
+    per_layer = (qd + 2 * kvd) * H + (qd + 2 * kvd) + H * qd + 2 * H  # attention + norms
+    per_layer += E * H + distinct * 3 * mi * H + 3 * si * H + H      # router, routed, shared, shared gate
+    weights = L * per_layer + H + cfg.vocab_size * H + batch * H     # final norm, head, embedding rows
+    cache = L * 2 * kvd * context * batch
+    return (weights + cache) * elt
+
+
+def prefill_flops(cfg, tokens):
+    H, L = cfg.hidden_size, cfg.num_hidden_layers
+    qd, kvd = cfg.q_dim, cfg.kv_dim
+    E, k, mi, si = cfg.num_experts, cfg.num_experts_per_tok, cfg.moe_intermediate_size, cfg.shared_expert_intermediate_size
+    per_token = (qd + 2 * kvd) * H + H * qd + E * H + k * 3 * mi * H + 3 * si * H + H
+    linear = 2.0 * tokens * L * per_token + 2.0 * cfg.vocab_size * H  # head on the last row only
+    attention = L * 2.0 * 2.0 * qd * tokens * (tokens + 1) / 2.0     # causal half of QK^T and PV
+    return linear + attention
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=32)
+    ap.add_argument("--warmup", type=int, default=4)
+    ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
+                    help="fewer layers than the configuration has (sizes of a layer are never reduced)")
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
+    ap.add_argument("--no-prefill", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
+        return 2
+
+    import torch
+    from inferx_amd.config import config_from_dict
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_model
+    from inferx_amd.sampling import Sampler, SamplingParams
+    from inferx_amd.weights import random_tensors
+
+    raw = dict(SHAPE)
+    raw["num_hidden_layers"] = args.layers
+    cfg = config_from_dict(raw)
+    rt = Runtime(args.dtype, "cuda:0")
+    elt = 2 if args.dtype == "bfloat16" else 4
+    points = [int(p) for p in args.points.split(",") if p]
+    max_batch = max([args.batch] + points)
+    log(f"drawing random weights on the device ({args.layers} layers, {args.dtype})")
+    t0 = time.time()
+    model = build_model(cfg.model_spec())
+    weights = random_tensors(model, seed=0, dtype=args.dtype, device="cuda:0")
+    weights = {k: rt.place(v) for k, v in weights.items()}
+    pages = max_batch * CONTEXT // PAGE
+    runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=max_batch,
+                         max_seq_len=CONTEXT, model=model)
+    torch.cuda.synchronize()
+    log(f"model ready in {time.time() - t0:.1f}s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB on the device")
+    sampler = Sampler(rt)
+    greedy = SamplingParams()
+    gen = torch.Generator().manual_seed(1234)
+
+    def prompt():
+        return torch.randint(0, cfg.vocab_size, (PROMPT,), generator=gen).tolist()
+
+    def run_decode(batch, steps, warmup):
+        """Prefill `batch` prompts of PROMPT tokens, then time `steps` decode steps."""
+        ids = [f"b{batch}_{i}" for i in range(batch)]
+        nxt = {}
+        for n, rid in enumerate(ids):
+            runner.add_request(rid)
+            logits = runner.run_entries([(rid, prompt(), [PROMPT - 1])])
+            nxt[rid] = sampler.sample(logits, [(greedy, 0, [])])[0]
+            if n % 8 == 7:
+                log(f"  prefilled {n + 1}/{batch}")
+
+        def one_step():
+            logits = runner.run_entries([(rid, [nxt[rid]], [0]) for rid in ids])
+            toks = sampler.sample(logits, [(greedy, 0, [])] * batch)
+            for rid, t in zip(ids, toks):
+                nxt[rid] = t
+
+        for _ in range(warmup):
+            one_step()
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for _ in range(steps):
+            one_step()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t
+        for rid in ids:
+            runner.end_request(rid)
+        return dt
+
+    # ---- prefill of one 2,048-token prompt ---------------------------------
+    prefill = None
+    if not args.no_prefill:
+        log("prefill")
+        times = []
+        for i in range(3):
+            runner.add_request("p")
+            toks = prompt()
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            runner.run_entries([("p", toks, [PROMPT - 1])])
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - t)
+            runner.end_request("p")
+        sec = min(times[1:])
+        flops = prefill_flops(cfg, PROMPT)
+        prefill = {"value": round(PROMPT / sec, 1), "tokens": PROMPT, "ms": round(sec * 1e3, 3),
+                   "frac": round(flops / sec / (PEAK_TFLOPS["bf16" if elt == 2 else "fp32"] * 1e12), 5)}
+        log(f"prefill {prefill}")
+
+    # ---- decode ----------------------------------------------------------------
+    log(f"decode at batch {args.batch}")
+    dt = run_decode(args.batch, args.steps, args.warmup)
+    ms = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    context = PROMPT + args.warmup + args.steps // 2
+    gbs = decode_bytes(cfg, args.batch, context, elt) / (dt / args.steps) / 1e9
+    pts = {}
+    for b in points:
+        log(f"decode at batch {b}")
+        steps = max(8, args.steps // 2)
+        d = run_decode(b, steps, max(2, args.warmup // 2))
+        pts[f"decode_b{b}"] = round(b * steps / d, 1)
+
+    line = {
+        "metric": "Qwen1.5-MoE-A2.7B decode tok/s @ batch 8 (2048-token prompts)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if elt == 2 else "fp32", "data": "synthetic: seeded random weights and token ids",
+        "config": {
+            "model": "Qwen1.5-MoE-A2.7B shape", "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT,
+            "parallelism": "single GPU", "layers": args.layers, "layers_of_shape": SHAPE["num_hidden_layers"],
+            "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "experts": cfg.num_experts, "top_k": cfg.num_experts_per_tok,
+            "moe_intermediate": cfg.moe_intermediate_size, "shared_intermediate": cfg.shared_expert_intermediate_size,
+            "vocab": cfg.vocab_size, "page_size": PAGE,
+        },
+        "prefill": prefill,
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                     "frac": round(gbs / PEAK_HBM_GBS, 5)},
+        "points": pts,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -174,3 +174,44 @@ extern "C" int ix_sample(const float* logits, int32_t* out, const float* tempera
                      top_k, min_p, rng_key, rng_counter, vocab);
   return ix_check_launch("ix_sample");
 }
+
+// ---------------------------------------------------------------------------
+// Penalties and masks on the logits, before selection (reference:
+// ApplyPenaltiesKernel layers.cu:1310-1345; host_sampling.cc:21-48).  Row r's
+// history is ids[hist_begin[r] .. hist_begin[r+1]) with counts; for each id:
+//   v = v > 0 ? v / repetition : v * repetition;  v -= presence;  v -= frequency * count
+// and its masked ids mask_ids[mask_begin[r] .. mask_begin[r+1]) are set to -inf.
+__global__ void penalties_kernel(float* __restrict__ logits, const int32_t* __restrict__ hist_begin,
+                                 const int32_t* __restrict__ hist_ids, const int32_t* __restrict__ hist_counts,
+                                 const float* __restrict__ presence, const float* __restrict__ frequency,
+                                 const float* __restrict__ repetition, const int32_t* __restrict__ mask_begin,
+                                 const int32_t* __restrict__ mask_ids, int64_t vocab) {
+  const int r = blockIdx.x;
+  float* row = logits + static_cast<int64_t>(r) * vocab;
+  const float rep = repetition[r], pres = presence[r], freq = frequency[r];
+  for (int i = hist_begin[r] + threadIdx.x; i < hist_begin[r + 1]; i += blockDim.x) {
+    const int id = hist_ids[i];  // ids are distinct within a row
+    if (id < 0 || id >= vocab) continue;
+    float v = row[id];
+    if (rep != 1.0f) v = v > 0.f ? v / rep : v * rep;
+    v -= pres;
+    v -= freq * static_cast<float>(hist_counts[i]);
+    row[id] = v;
+  }
+  __syncthreads();
+  for (int i = mask_begin[r] + threadIdx.x; i < mask_begin[r + 1]; i += blockDim.x) {
+    const int id = mask_ids[i];
+    if (id >= 0 && id < vocab) row[id] = -INFINITY;
+  }
+}
+
+extern "C" int ix_apply_penalties(float* logits, const int32_t* hist_begin, const int32_t* hist_ids,
+                                  const int32_t* hist_counts, const float* presence, const float* frequency,
+                                  const float* repetition, const int32_t* mask_begin, const int32_t* mask_ids,
+                                  int64_t rows, int64_t vocab, hipStream_t stream) {
+  IX_REQUIRE(rows >= 0 && vocab > 0, "sizes must be positive");
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(penalties_kernel, dim3(rows), dim3(256), 0, stream, logits, hist_begin, hist_ids, hist_counts,
+                     presence, frequency, repetition, mask_begin, mask_ids, vocab);
+  return ix_check_launch("ix_apply_penalties");
+}

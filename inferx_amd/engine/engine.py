@@ -1,0 +1,163 @@
+"""The engine: model runner + scheduler + sampler in one loop, and the Python
+entry point.
+
+    engine = LLMEngine("model_dir", dtype="bfloat16")
+    outputs = engine.generate([[1, 2, 3], [4, 5]], SamplingParams(max_tokens=8))
+
+One iteration is prepare_step -> step -> sample -> commit_step (reference:
+Engine::Impl::RunModel, src/engine/engine.cc:526-666).  Option names follow the
+reference's command line (src/support/options.cc:47-174).  Token ids in, token
+ids out: tokenizers and servers are not part of this engine.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence, Union
+
+import torch
+
+from ..config import config_from_directory
+from ..parts import build_model
+from ..sampling import Sampler, SamplingParams
+from ..weights import load_weights
+from .batch import build_step_batch
+from .runner import ModelRunner
+from .runtime import Runtime
+from .scheduler import Completion, Scheduler
+
+KV_HEADROOM_BYTES = 1 << 30
+
+
+def resolve_kv_blocks(block_bytes: int, *, explicit_blocks: Optional[int] = None,
+                      kv_cache_memory_bytes: Optional[int] = None, gpu_memory_utilization: float = 0.92,
+                      total_bytes: int = 0, used_bytes: int = 0, min_blocks: int = 1) -> int:
+    """How many pages the pool gets.  An explicit count wins; else explicit bytes;
+    else utilization * total - used - 1 GiB of headroom (reference: ResolveKvBlocks,
+    src/engine/kv_autosize.cc:10-47; vector tests/unit/kv_autosize_test.cc:33-42)."""
+    if block_bytes <= 0:
+        raise ValueError("block_bytes must be positive")
+    if explicit_blocks is not None:
+        if explicit_blocks <= 0:
+            raise ValueError("--num-gpu-blocks-override must be positive")
+        return explicit_blocks
+    if kv_cache_memory_bytes is not None:
+        blocks = kv_cache_memory_bytes // block_bytes
+        what = f"--kv-cache-memory-bytes {kv_cache_memory_bytes}"
+    else:
+        if not 0.0 < gpu_memory_utilization <= 1.0:
+            raise ValueError("--gpu-memory-utilization must be within (0, 1]")
+        budget = int(gpu_memory_utilization * total_bytes) - used_bytes - KV_HEADROOM_BYTES
+        blocks = max(0, budget) // block_bytes
+        what = (f"--gpu-memory-utilization {gpu_memory_utilization} of {total_bytes} bytes with {used_bytes} in use "
+                f"and {KV_HEADROOM_BYTES} of headroom")
+    if blocks < min_blocks:
+        raise ValueError(f"{what} gives {blocks} cache pages of {block_bytes} bytes; {min_blocks} are needed for one "
+                         "sequence of --max-model-len: lower --max-model-len or give the cache more memory")
+    return blocks
+
+
+@dataclass
+class Stats:
+    steps: int = 0
+    tokens_in: int = 0
+    tokens_out: int = 0
+    preemptions: int = 0
+    step_seconds: float = 0.0
+
+
+class LLMEngine:
+    def __init__(self, model: str, dtype: str = "bfloat16", *, max_num_seqs: int = 8, max_model_len: int = 2048,
+                 max_num_batched_tokens: Optional[int] = None, block_size: int = 16,
+                 num_gpu_blocks_override: Optional[int] = None, kv_cache_memory_bytes: Optional[int] = None,
+                 gpu_memory_utilization: float = 0.92, device: str = "cuda:0", runner: Optional[ModelRunner] = None):
+        if max_num_batched_tokens is None:
+            max_num_batched_tokens = max(2048, max_model_len)  # reference: options.cc:332-336
+        if runner is None:
+            config = config_from_directory(model)
+            rt = Runtime(dtype, device)
+            net = build_model(config.model_spec())
+            weights = load_weights(net, model, rt)
+            # page count needs the per-token bytes, which need the cache plan: lay out with one page, then size
+            probe = ModelRunner(config, weights, rt, page_size=block_size, num_pages=1, max_requests=max_num_seqs,
+                                max_seq_len=max_model_len, model=net)
+            block_bytes = probe.kv_bytes_per_token() * block_size
+            free, total = torch.cuda.mem_get_info(rt.device)
+            pages = resolve_kv_blocks(max(block_bytes, 1), explicit_blocks=num_gpu_blocks_override,
+                                      kv_cache_memory_bytes=kv_cache_memory_bytes,
+                                      gpu_memory_utilization=gpu_memory_utilization, total_bytes=total,
+                                      used_bytes=total - free, min_blocks=-(-max_model_len // block_size))
+            pages = min(pages, max_num_seqs * -(-max_model_len // block_size))  # more could never be used
+            probe._lay_out_cache(pages)
+            runner = probe
+        self.runner = runner
+        self.scheduler = Scheduler(runner.cache, max_running=max_num_seqs, max_batch_tokens=max_num_batched_tokens,
+                                   max_seq_len=max_model_len)
+        self.sampler = Sampler(runner.rt)
+        self.stats = Stats()
+        self._next_id = 0
+
+    # ---- requests -----------------------------------------------------------
+    def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,
+                    request_id: Optional[Hashable] = None) -> Hashable:
+        vocab = self.runner.spec.vocab_size
+        bad = [t for t in prompt_token_ids if not 0 <= int(t) < vocab]
+        if bad:
+            raise ValueError(f"prompt token id {bad[0]} is outside the vocabulary of {vocab}")
+        if request_id is None:
+            request_id = self._next_id
+            self._next_id += 1
+        self.scheduler.add_request(request_id, [int(t) for t in prompt_token_ids], params)
+        return request_id
+
+    def cancel(self, request_id: Hashable) -> None:
+        self.scheduler.cancel(request_id)
+
+    def has_unfinished(self) -> bool:
+        return self.scheduler.has_work()
+
+    # ---- the loop -------------------------------------------------------------
+    def step(self) -> List[Completion]:
+        """One scheduler step.  Returns the requests that finished in it."""
+        plan = self.scheduler.prepare_step()
+        if plan is None:
+            return self.scheduler.take_completed()
+        t0 = time.perf_counter()
+        batch = build_step_batch(self.runner.cache, plan.entries())
+        logits = self.runner.step(batch)
+        rows = []
+        for c in plan.contributions:
+            if c.samples:
+                s = self.scheduler.sequence(c.rid)
+                rows.append((s.params, s.draws, s.tokens[s.prompt_len:]))
+        sampled = self.sampler.sample(logits, rows)
+        self.scheduler.commit_step(sampled)
+        self.stats.steps += 1
+        self.stats.tokens_in += plan.num_tokens
+        self.stats.tokens_out += len(sampled)
+        self.stats.preemptions = self.scheduler.preemptions
+        self.stats.step_seconds += time.perf_counter() - t0
+        return self.scheduler.take_completed()
+
+    def generate(self, prompts: Sequence[Sequence[int]],
+                 params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
+                 with_reasons: bool = False):
+        """Generated token ids per prompt, in the order of the prompts."""
+        if params is None or isinstance(params, SamplingParams):
+            params = [params or SamplingParams()] * len(prompts)
+        if len(params) != len(prompts):
+            raise ValueError("one SamplingParams per prompt is needed")
+        ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
+        done: Dict[Hashable, Completion] = {}
+        while len(done) < len(ids):
+            finished = self.step()
+            for c in finished:
+                done[c.rid] = c
+            if not finished and not self.scheduler.has_work():
+                break
+        missing = [i for i in ids if i not in done]
+        if missing:
+            raise RuntimeError(f"requests {missing} never finished")
+        if with_reasons:
+            return [(done[i].output_tokens, done[i].reason) for i in ids]
+        return [done[i].output_tokens for i in ids]

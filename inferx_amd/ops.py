@@ -252,3 +252,19 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: torch.Tensor, t
         _need(t.dtype == torch.int64 and t.numel() >= R, "rng key and counter must be int64 [rows]")
     _call("ix_sample", _ptr(logits), _ptr(out), _ptr(temperature), _ptr(top_p), _ptr(top_k), _ptr(min_p),
           _ptr(rng_key), _ptr(rng_counter), _i64(R), _i64(V), _stream())
+
+
+def apply_penalties(logits: torch.Tensor, hist_begin: torch.Tensor, hist_ids: torch.Tensor,
+                    hist_counts: torch.Tensor, presence: torch.Tensor, frequency: torch.Tensor,
+                    repetition: torch.Tensor, mask_begin: torch.Tensor, mask_ids: torch.Tensor) -> None:
+    """In place on float32 logits [R, V]; histories and masks in CSR form (begin arrays hold R + 1 entries)."""
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32, "logits must be float32")
+    for t in (hist_begin, mask_begin):
+        _is_i32(t, R + 1)
+    for t in (hist_ids, hist_counts, mask_ids):
+        _is_i32(t)
+    for t in (presence, frequency, repetition):
+        _need(t.dtype == torch.float32 and t.numel() >= R, "penalties must be float32 [rows]")
+    _call("ix_apply_penalties", _ptr(logits), _ptr(hist_begin), _ptr(hist_ids), _ptr(hist_counts), _ptr(presence),
+          _ptr(frequency), _ptr(repetition), _ptr(mask_begin), _ptr(mask_ids), _i64(R), _i64(V), _stream())

@@ -1,0 +1,68 @@
+"""Choosing the next token of each sampling row, on the device.
+
+Order (reference: src/engine/host_sampling.cc:21-111): penalties and masks on
+the logits, then greedy (temperature <= 0: first maximum, lowest index on
+ties) or temperature softmax with top-k / min-p / top-p cut-offs and one
+uniform draw.  The draw of a request's n-th sampled token depends only on
+(seed, n), so a preempted request that is recomputed draws the same numbers.
+"""
+from __future__ import annotations
+
+from collections import Counter
+from typing import List, Sequence, Tuple
+
+import torch
+
+from .. import ops
+from .params import SamplingParams
+
+# (params, number of tokens sampled so far for this request, its generated tokens so far)
+Row = Tuple[SamplingParams, int, Sequence[int]]
+
+
+class Sampler:
+    def __init__(self, rt):
+        self.rt = rt
+
+    def _dev(self, values, dtype) -> torch.Tensor:
+        return torch.tensor(list(values), dtype=dtype).to(self.rt.device)
+
+    def sample(self, logits: torch.Tensor, rows: List[Row]) -> List[int]:
+        """logits float32 [R, V] on the device (changed in place when penalties apply)."""
+        R = logits.shape[0]
+        if R != len(rows):
+            raise ValueError(f"{R} logits rows for {len(rows)} sampling rows")
+        if R == 0:
+            return []
+        out = self.rt.empty((R,), torch.int32)
+        masks = [list(p.stop_tokens) if len(gen) < p.min_tokens else [] for p, _, gen in rows]
+        if any(p.needs_penalties for p, _, _ in rows) or any(masks):
+            hist_begin, hist_ids, hist_counts, mask_begin, mask_ids = [0], [], [], [0], []
+            for (p, _, gen), m in zip(rows, masks):
+                if p.needs_penalties:
+                    for tok, cnt in sorted(Counter(gen).items()):
+                        hist_ids.append(tok)
+                        hist_counts.append(cnt)
+                hist_begin.append(len(hist_ids))
+                mask_ids.extend(m)
+                mask_begin.append(len(mask_ids))
+            ops.apply_penalties(
+                logits, self._dev(hist_begin, torch.int32), self._dev(hist_ids or [0], torch.int32),
+                self._dev(hist_counts or [0], torch.int32),
+                self._dev([p.presence_penalty for p, _, _ in rows], torch.float32),
+                self._dev([p.frequency_penalty for p, _, _ in rows], torch.float32),
+                self._dev([p.repetition_penalty for p, _, _ in rows], torch.float32),
+                self._dev(mask_begin, torch.int32), self._dev(mask_ids or [0], torch.int32))
+        if all(p.temperature <= 0 for p, _, _ in rows):
+            ops.argmax(logits, out)
+        else:
+            to_i64 = lambda v: v - (1 << 64) if v >= (1 << 63) else v
+            ops.sample(
+                logits, out,
+                self._dev([p.temperature for p, _, _ in rows], torch.float32),
+                self._dev([p.top_p for p, _, _ in rows], torch.float32),
+                self._dev([p.top_k for p, _, _ in rows], torch.int32),
+                self._dev([p.min_p for p, _, _ in rows], torch.float32),
+                self._dev([to_i64(p.seed % (1 << 64)) for p, _, _ in rows], torch.int64),
+                self._dev([n for _, n, _ in rows], torch.int64))
+        return out.tolist()
