@@ -1,0 +1,240 @@
+// Paged attention on the matrix cores (bfloat16), for prompt portions and for
+// decoding alike.  Same arithmetic as the plain kernel (attention_plain.hip):
+// keys [start, p] through the block table, scores * scale, softmax online in
+// float32, PV accumulated in float32.
+//
+// Unit of work = one wavefront: a tile of up to 16 consecutive queries of one
+// request and one query head, over one slice of that tile's keys (split-KV).
+// There is no LDS and no barrier: a workgroup is four independent wavefronts.
+//
+// The transposed products are formed so that no operand has to be shuffled:
+//   S^T[key][query]  = K[key][:] . Q[query][:]     (A = K rows, B = Q rows)
+//   O^T[d][query]   += V^T[d][key] * P^T[key][query]  (A = V^T rows, B = P^T)
+// v_mfma_f32_16x16x32_bf16 gives lane l of the result rows 4*(l/16)+i, column
+// l%16.  Row m of the first key block of an iteration is key 8*(m/4) + m%4 and
+// of the second key 8*(m/4) + 4 + m%4, so a lane ends up with the scores of
+// eight consecutive keys (8*(l/16) .. +7) of its query: exactly the B operand
+// of the second product, while V^T (values are stored [d][offset] within a
+// page) supplies eight consecutive keys of one column as 16 contiguous bytes.
+//
+// With more than one split, each wavefront writes (max, sum, unnormalised O)
+// and `attn_combine_kernel` merges them.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+#define ATTN_KEYS_PER_ITER 32
+
+template <int NB>  // head_dim = 16 * NB
+__global__ void __launch_bounds__(256)
+attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
+                 const int32_t* __restrict__ block_table, const int32_t* __restrict__ tile_seq,
+                 const int32_t* __restrict__ tile_q0, const int32_t* __restrict__ tile_rows,
+                 const int32_t* __restrict__ positions, __bf16* __restrict__ out, float* __restrict__ part_o,
+                 float* __restrict__ part_ml, int n_tiles, int n_splits, int heads, int kv_heads, int page_size,
+                 int max_blocks, float scale_log2, int window) {
+  constexpr int D = 16 * NB;
+  constexpr int NC = (NB + 1) / 2;  // 32-wide chunks of the head dimension
+  const int lane = threadIdx.x & 63;
+  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (unit >= n_tiles * n_splits) return;
+  const int tile = unit / n_splits, split = unit - tile * n_splits;
+  const int head = blockIdx.y;
+  const int kvh = head / (heads / kv_heads);
+  const int n = lane & 15, g = lane >> 4;
+
+  const int tq0 = tile_q0[tile];
+  const int rows = tile_rows[tile];
+  const int pos0 = positions[tq0];
+  const int32_t* table = block_table + static_cast<int64_t>(tile_seq[tile]) * max_blocks;
+
+  // keys this tile reads at all: [lo, hi); this wavefront's slice [ks, ke)
+  const int lo = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;
+  const int hi = pos0 + rows;
+  const int lo_al = lo & ~(ATTN_KEYS_PER_ITER - 1);
+  const int per = (((hi - lo_al + n_splits - 1) / n_splits) + ATTN_KEYS_PER_ITER - 1) & ~(ATTN_KEYS_PER_ITER - 1);
+  const int ks = lo_al + split * per;
+  const int ke = min(hi, ks + per);
+
+  const int my_pos = pos0 + n;  // this lane's query (column n)
+  const bool my_row = n < rows;
+  const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
+
+  // Q as B operand: lane (n, g) holds Q[query n][32 c + 8 g .. +8]
+  bf16x8 qf[NC];
+#pragma unroll
+  for (int c = 0; c < NC; ++c) {
+    const int d0 = 32 * c + 8 * g;
+    if (my_row && d0 < D)
+      qf[c] = *reinterpret_cast<const bf16x8*>(q + (static_cast<int64_t>(tq0 + n) * heads + head) * D + d0);
+    else
+      for (int j = 0; j < 8; ++j) qf[c][j] = (__bf16)0.f;
+  }
+
+  f32x4 o[NB];
+#pragma unroll
+  for (int b = 0; b < NB; ++b) o[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m = -INFINITY, lsum = 0.f;
+
+  for (int kb = ks; kb < ke; kb += ATTN_KEYS_PER_ITER) {
+    // ---- S^T for 32 keys: two blocks of 16 rows ----
+    f32x4 s[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      int key = kb + 8 * (n >> 2) + 4 * b + (n & 3);  // A row n of block b
+      key = min(key, hi - 1);                          // rows past the end are masked below
+      int page = table[key / page_size];
+      page = max(page, 0);                             // a page the window has passed: masked below
+      const __bf16* kr =
+          k_cache + ((static_cast<int64_t>(page) * kv_heads + kvh) * page_size + key % page_size) * D;
+      s[b] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int d0 = 32 * c + 8 * g;
+        bf16x8 kf;
+        if (d0 < D)
+          kf = *reinterpret_cast<const bf16x8*>(kr + d0);
+        else
+          for (int j = 0; j < 8; ++j) kf[j] = (__bf16)0.f;
+        s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], s[b], 0, 0, 0);
+      }
+    }
+    // ---- V^T fragments: lane (dd = n, g) holds V^T[16 blk + dd][kb + 8 g .. +8] ----
+    bf16x8 vf[NB];
+    {
+      int key = min(kb + 8 * g, hi - 1) & ~7;
+      int page = max(table[key / page_size], 0);
+      const __bf16* vr = v_cache + (static_cast<int64_t>(page) * kv_heads + kvh) * D * page_size + key % page_size;
+#pragma unroll
+      for (int b = 0; b < NB; ++b)
+        vf[b] = *reinterpret_cast<const bf16x8*>(vr + static_cast<int64_t>(16 * b + n) * page_size);
+    }
+    // ---- mask, online softmax for this lane's query over its 8 keys ----
+    float sv[8];
+    float mx = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const int key = kb + 8 * g + j;
+      const bool ok = my_row && key >= my_lo && key <= my_pos && key < ke;
+      sv[j] = ok ? s[j >> 2][j & 3] * scale_log2 : -INFINITY;
+      mx = fmaxf(mx, sv[j]);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    const float m_new = fmaxf(m, mx);
+    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+    const float alpha = exp2f(m - m_safe);
+    float psum = 0.f;
+    bf16x8 pf;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float p = exp2f(sv[j] - m_safe);
+      psum += p;
+      pf[j] = (__bf16)p;
+    }
+    lsum = lsum * alpha + psum;
+    m = m_new;
+    // ---- O^T += V^T P^T ----
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      o[b] *= alpha;
+      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf, o[b], 0, 0, 0);
+    }
+  }
+  lsum += __shfl_xor(lsum, 16, 64);
+  lsum += __shfl_xor(lsum, 32, 64);
+  if (!my_row) return;
+
+  // lane holds O^T rows d = 16 b + 4 g + i of column n
+  if (n_splits == 1) {
+    const float inv = 1.0f / lsum;
+    __bf16* dst = out + (static_cast<int64_t>(tq0 + n) * heads + head) * D + 4 * g;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      bf16x4 v;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = (__bf16)(o[b][i] * inv);
+      *reinterpret_cast<bf16x4*>(dst + 16 * b) = v;
+    }
+  } else {
+    const int64_t p = (static_cast<int64_t>(tq0 + n) * heads + head) * n_splits + split;
+    float* dst = part_o + p * D + 4 * g;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) *reinterpret_cast<f32x4*>(dst + 16 * b) = o[b];
+    if (g == 0) {
+      part_ml[2 * p] = m;
+      part_ml[2 * p + 1] = lsum;
+    }
+  }
+}
+
+// out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M),  M = max_s m_s
+__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
+                                    __bf16* __restrict__ out, int n_splits, int head_dim) {
+  const int64_t th = blockIdx.x;  // token * heads + head
+  const float* ml = part_ml + th * n_splits * 2;
+  float M = -INFINITY;
+  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, ml[2 * s]);
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    float acc = 0.f, l = 0.f;
+    for (int s = 0; s < n_splits; ++s) {
+      const float m_s = ml[2 * s];
+      if (m_s == -INFINITY) continue;
+      const float w = exp2f(m_s - M);
+      acc += w * part_o[(th * n_splits + s) * head_dim + d];
+      l += w * ml[2 * s + 1];
+    }
+    out[th * head_dim + d] = (__bf16)(acc / l);
+  }
+}
+
+template <int NB>
+static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void* k, const void* v,
+                        const int32_t* table, const int32_t* tile_seq, const int32_t* tile_q0,
+                        const int32_t* tile_rows, const int32_t* positions, void* out, float* part_o, float* part_ml,
+                        int n_tiles, int n_splits, int heads, int kv_heads, int page_size, int max_blocks,
+                        float scale_log2, int window) {
+  hipLaunchKernelGGL(attn_mfma_kernel<NB>, grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
+                     (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, positions, (__bf16*)out, part_o, part_ml,
+                     n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window);
+}
+
+// Workspace (when n_splits > 1): part_o float32 [tokens * heads * n_splits * head_dim],
+// part_ml float32 [tokens * heads * n_splits * 2].
+extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
+                                 const int32_t* tile_seq, const int32_t* tile_q0, const int32_t* tile_rows,
+                                 const int32_t* positions, void* out, float* part_o, float* part_ml, int64_t tokens,
+                                 int n_tiles, int n_splits, int heads, int kv_heads, int head_dim, int page_size,
+                                 int max_blocks, float scale, int window, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && n_tiles >= 0 && heads > 0 && kv_heads > 0 && max_blocks > 0, "sizes must be positive");
+  IX_REQUIRE(heads % kv_heads == 0, "heads must be a multiple of kv_heads");
+  IX_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256, "head_dim must be a multiple of 16 up to 256");
+  IX_REQUIRE(page_size % 16 == 0 && page_size > 0, "page_size must be a multiple of 16");
+  IX_REQUIRE(n_splits >= 1 && n_splits <= 256, "n_splits must be between 1 and 256");
+  IX_REQUIRE(n_splits == 1 || (part_o != nullptr && part_ml != nullptr), "workspace needed for split keys");
+  IX_REQUIRE(window >= 0, "window must not be negative");
+  IX_REQUIRE(heads <= 65535, "too many heads");
+  if (n_tiles == 0 || tokens == 0) return 0;
+  const int64_t units = static_cast<int64_t>(n_tiles) * n_splits;
+  dim3 grid(static_cast<unsigned>((units + 3) / 4), heads);
+  const float scale_log2 = scale * 1.4426950408889634f;
+#define CASE(NB)                                                                                                   \
+  case NB:                                                                                                         \
+    launch_attn<NB>(grid, stream, q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, positions, out,  \
+                    part_o, part_ml, n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window); \
+    break;
+  switch (head_dim / 16) {
+    CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+    CASE(9) CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
+  }
+#undef CASE
+  if (ix_check_launch("ix_attention_mfma")) return 1;
+  if (n_splits > 1) {
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(static_cast<unsigned>(tokens * heads)), dim3(64), 0, stream, part_o,
+                       part_ml, (__bf16*)out, n_splits, head_dim);
+    return ix_check_launch("ix_attention_combine");
+  }
+  return 0;
+}

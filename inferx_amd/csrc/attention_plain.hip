@@ -7,7 +7,8 @@
 // A query at position p reads keys [start, p], start = 0 or, with a window W,
 // max(0, p + 1 - W) (reference: PagedAttentionWithLseKernel, layers.cu:329-407;
 // window rule :346-354).  Query head h reads kv head h / (heads / kv_heads).
-// Key j of a request lives in page table[j / page_size] at offset j % page_size.
+// Key j of a request lives in page table[j / page_size] at offset j % page_size;
+// keys are stored [page][kv_head][offset][d], values [page][kv_head][d][offset].
 #include "common.h"
 
 #define ATTN_PLAIN_THREADS 256
@@ -62,8 +63,8 @@ attn_plain_kernel(const T* __restrict__ q, const T* __restrict__ k_cache, const 
       for (int jj = 0; jj < n; ++jj) {
         const int key = base + jj;
         const T* vr =
-            v_cache + ((static_cast<int64_t>(pg[jj]) * kv_heads + g) * page_size + key % page_size) * head_dim;
-        acc += sc[jj] * ix_load(vr + tid);
+            v_cache + ((static_cast<int64_t>(pg[jj]) * kv_heads + g) * head_dim + tid) * page_size + key % page_size;
+        acc += sc[jj] * ix_load(vr);
       }
     }
     __syncthreads();

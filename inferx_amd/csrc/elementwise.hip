@@ -150,8 +150,10 @@ extern "C" int ix_rope_table(void* cs, const int32_t* positions, const float* in
 // + x_j sin; reference RopeKernel layers.cu:80-115), write q to its own buffer
 // and k, v into the cache page of the token's slot (rotated keys are what the
 // cache holds; reference AppendKvKernel layers.cu:195-219, SplitQkvKernel :485-510).
-// Cache layout per layer: [page][kv_head][offset in page][head_dim].
-// A negative slot, or null caches, writes nothing to the cache.
+// Cache layout per layer: keys [page][kv_head][offset in page][head_dim],
+// values transposed [page][kv_head][head_dim][offset in page] (so that eight
+// consecutive keys of one value column are 16 contiguous bytes for the
+// matrix-core kernel).  A negative slot, or null caches, writes nothing.
 template <typename T>
 __global__ void qkv_rope_append_kernel(const T* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
                                        const float2* __restrict__ cs, const int32_t* __restrict__ slots,
@@ -187,11 +189,17 @@ __global__ void qkv_rope_append_kernel(const T* __restrict__ qkv, const void* __
       ix_store(dst, lo);
       ix_store(dst + half, hi);
     } else if (cache_ok) {
-      const int g = is_v ? head - heads - kv_heads : head - heads;
-      T* base = is_v ? v_cache : k_cache;
-      T* dst = base + ((page * kv_heads + g) * page_size + off) * head_dim + j;
-      ix_store(dst, lo);
-      ix_store(dst + half, hi);
+      if (is_v) {
+        const int g = head - heads - kv_heads;
+        T* dst = v_cache + ((page * kv_heads + g) * head_dim + j) * page_size + off;
+        ix_store(dst, lo);
+        ix_store(dst + static_cast<int64_t>(half) * page_size, hi);
+      } else {
+        const int g = head - heads;
+        T* dst = k_cache + ((page * kv_heads + g) * page_size + off) * head_dim + j;
+        ix_store(dst, lo);
+        ix_store(dst + half, hi);
+      }
     }
   }
 }

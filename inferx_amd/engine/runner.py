@@ -73,7 +73,10 @@ class ModelRunner:
                     raise ValueError(f"schedule entry {i} reads the cache of entry {src}, whose layout differs")
                 g = needs.index(need)
                 j = owners[g].index(src)
-                b.group, b.k, b.v, b.writes = g, self.kv[g][j, 0], self.kv[g][j, 1], cache_from is None
+                n_ = needs[g]
+                b.group, b.k, b.writes = g, self.kv[g][j, 0], cache_from is None
+                # values are kept transposed within a page: [pages, kv_heads, head_dim, page_size]
+                b.v = self.kv[g][j, 1].view(-1, n_.kv_heads, n_.head_dim, self.page_size)
             if state is not None:
                 b.state = torch.zeros((self.max_requests,) + tuple(state.shape), dtype=torch.float32,
                                       device=rt.device)

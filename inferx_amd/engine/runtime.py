@@ -90,7 +90,7 @@ class CacheBinding:
 
     group: int = -1
     k: Optional[torch.Tensor] = None       # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None       # [pages, kv_heads, head_dim, page_size] (transposed within a page)
     writes: bool = True                    # False: reads another execution's cache
     state: Optional[torch.Tensor] = None   # [slots, *shape] float32
 

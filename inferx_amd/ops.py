@@ -127,7 +127,8 @@ def qkv_rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: Op
                     slots: Optional[torch.Tensor], q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
                     v_cache: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int) -> None:
     """Bias, rotation and cache append after the fused q/k/v product.
-    qkv [T, (heads + 2 kv_heads) * d]; caches [pages, kv_heads, page_size, d]."""
+    qkv [T, (heads + 2 kv_heads) * d]; key cache [pages, kv_heads, page_size, d], value cache
+    [pages, kv_heads, d, page_size]."""
     T = qkv.shape[0]
     width = (heads + 2 * kv_heads) * head_dim
     _need(qkv.shape == (T, width), f"qkv must be [T, {width}]")
@@ -138,9 +139,9 @@ def qkv_rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: Op
         _need(cos_sin.dtype == torch.float32 and cos_sin.shape == (T, head_dim // 2, 2), "rotary table mismatch")
     page_size, total = 1, 0
     if k_cache is not None:
-        _need(v_cache is not None and k_cache.shape == v_cache.shape and k_cache.dtype == qkv.dtype
-              and v_cache.dtype == qkv.dtype, "cache mismatch")
+        _need(v_cache is not None and k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "cache mismatch")
         _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim, "cache layout")
+        _need(v_cache.shape == (k_cache.shape[0], kv_heads, head_dim, k_cache.shape[2]), "value cache layout")
         page_size = k_cache.shape[2]
         total = k_cache.shape[0] * page_size
         _need(slots is not None, "slots needed to write the cache")
@@ -150,14 +151,21 @@ def qkv_rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: Op
           _i32(kv_heads), _i32(head_dim), _i32(page_size), _i64(total), _stream())
 
 
+def _check_caches(q, k_cache, v_cache):
+    d = q.shape[2]
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "cache dtype differs from q")
+    _need(k_cache.dim() == 4 and k_cache.shape[3] == d, "key cache must be [pages, kv_heads, page_size, d]")
+    _need(v_cache.shape == (k_cache.shape[0], k_cache.shape[1], d, k_cache.shape[2]),
+          "value cache must be [pages, kv_heads, d, page_size]")
+
+
 def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                     seq_of_token: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float,
                     window: int) -> None:
     """Paged attention, one workgroup per (token, head).  q, out [T, heads, d]."""
     T, heads, d = q.shape
     _need(out.shape == q.shape and out.dtype == q.dtype, "out mismatch")
-    _need(k_cache.shape == v_cache.shape and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "cache mismatch")
-    _need(k_cache.dim() == 4 and k_cache.shape[3] == d, "cache layout")
+    _check_caches(q, k_cache, v_cache)
     kv_heads, page_size = k_cache.shape[1], k_cache.shape[2]
     _need(block_table.dim() == 2, "block table must be [requests, pages]")
     _is_i32(block_table)
@@ -166,6 +174,36 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     _call("ix_attention_plain", _ptr(q), _ptr(k_cache), _ptr(v_cache), _i32(_dt(q)), _ptr(block_table),
           _ptr(seq_of_token), _ptr(positions), _ptr(out), _i64(T), _i32(heads), _i32(kv_heads), _i32(d),
           _i32(page_size), _i32(block_table.shape[1]), _f32(scale), _i32(window), _stream())
+
+
+def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                   tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, n_splits: int,
+                   workspace: Optional[torch.Tensor], scale: float, window: int) -> None:
+    """Paged attention on the matrix cores (bfloat16).  `tiles` int32 [3, n_tiles]: request, first token row and
+    number of rows (<= 16) of each query tile.  `workspace` float32 with T * heads * n_splits * (d + 2) entries
+    when n_splits > 1."""
+    T, heads, d = q.shape
+    _need(q.dtype == torch.bfloat16, "the matrix-core attention kernel is bfloat16 only")
+    _need(out.shape == q.shape and out.dtype == q.dtype, "out mismatch")
+    _check_caches(q, k_cache, v_cache)
+    kv_heads, page_size = k_cache.shape[1], k_cache.shape[2]
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    _is_i32(block_table)
+    _is_i32(positions, T)
+    _is_i32(tiles)
+    _need(tiles.dim() == 2 and tiles.shape[0] == 3 and tiles.is_contiguous(), "tiles must be int32 [3, n_tiles]")
+    n_tiles = tiles.shape[1]
+    part_o = part_ml = None
+    if n_splits > 1:
+        need = T * heads * n_splits * (d + 2)
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
+              f"workspace of {need} float32 needed")
+        part_o = workspace
+        part_ml = workspace[T * heads * n_splits * d:]
+    _call("ix_attention_mfma", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
+          _ptr(tiles[1]), _ptr(tiles[2]), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), _i64(T),
+          _i32(n_tiles), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(page_size),
+          _i32(block_table.shape[1]), _f32(scale), _i32(window), _stream())
 
 
 def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor], topk_w: torch.Tensor,

@@ -1,0 +1,151 @@
+"""Each kernel alone against a plain float32/float64 PyTorch reference of the same
+operation, at sizes other than the engine's tiny configurations."""
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def close(got, want, tol, what=""):
+    want = want.double().cpu()
+    err = float((got.double().cpu() - want).abs().max()) / max(float(want.abs().max()), 1e-30)
+    assert err <= tol, f"{what}: error {err:.3e} of the largest value, tolerance {tol:.1e}"
+    return err
+
+
+TOL = {torch.float32: 1e-5, torch.bfloat16: 1.5e-2}
+
+
+# ---------------------------------------------------------------------------
+def build_paged(seq_lens, q_lens, heads, kv_heads, d, page_size, dtype, seed=0, shuffle_pages=True):
+    """Random q/k/v for requests of the given context and query lengths, written into a paged cache whose pages
+    are handed out in a scrambled order.  Returns everything the attention kernels need plus dense k, v."""
+    from inferx_amd import ops  # noqa: F401
+    S = len(seq_lens)
+    max_blocks = max(-(-L // page_size) for L in seq_lens) + 1
+    total_pages = sum(-(-L // page_size) for L in seq_lens) + 3
+    order = torch.randperm(total_pages, generator=torch.Generator().manual_seed(seed)).tolist() if shuffle_pages \
+        else list(range(total_pages))
+    table = torch.full((S, max_blocks), -1, dtype=torch.int32)
+    k_cache = torch.zeros(total_pages, kv_heads, page_size, d, dtype=dtype)
+    v_cache = torch.zeros(total_pages, kv_heads, d, page_size, dtype=dtype)
+    dense, qs, positions, seq_of_token = [], [], [], []
+    nxt = 0
+    for s, (L, n) in enumerate(zip(seq_lens, q_lens)):
+        k = (torch.randn(L, kv_heads, d, generator=torch.Generator().manual_seed(seed * 100 + s))).to(dtype)
+        v = (torch.randn(L, kv_heads, d, generator=torch.Generator().manual_seed(seed * 100 + s + 50))).to(dtype)
+        dense.append((k, v))
+        for j in range(-(-L // page_size)):
+            page = order[nxt]
+            nxt += 1
+            table[s, j] = page
+            chunk = slice(j * page_size, min(L, (j + 1) * page_size))
+            m = chunk.stop - chunk.start
+            k_cache[page, :, :m, :] = k[chunk].transpose(0, 1)
+            v_cache[page, :, :, :m] = v[chunk].permute(1, 2, 0)
+        qs.append(torch.randn(n, heads, d, generator=torch.Generator().manual_seed(seed * 100 + s + 77)).to(dtype))
+        positions += list(range(L - n, L))
+        seq_of_token += [s] * n
+    return dict(q=torch.cat(qs).to(DEV), k_cache=k_cache.to(DEV), v_cache=v_cache.to(DEV), table=table.to(DEV),
+                positions=torch.tensor(positions, dtype=torch.int32, device=DEV),
+                seq_of_token=torch.tensor(seq_of_token, dtype=torch.int32, device=DEV), dense=dense, qs=qs)
+
+
+def attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window):
+    outs = []
+    for (k, v), q, L, n in zip(p["dense"], p["qs"], seq_lens, q_lens):
+        q, k, v = q.double(), k.double(), v.double()
+        kk, vv = k.repeat_interleave(heads // kv_heads, 1), v.repeat_interleave(heads // kv_heads, 1)
+        s = torch.einsum("qhd,khd->hqk", q, kk) * scale
+        qpos = torch.arange(L - n, L)[:, None]
+        kpos = torch.arange(L)[None, :]
+        ok = kpos <= qpos
+        if window > 0:
+            ok &= kpos >= qpos + 1 - window
+        s = s.masked_fill(~ok[None], -math.inf)
+        outs.append(torch.einsum("hqk,khd->qhd", torch.softmax(s, -1), vv))
+    return torch.cat(outs)
+
+
+ATTN_CASES = [
+    # seq_lens, q_lens, heads, kv_heads, d, page, window
+    ([40], [40], 4, 2, 32, 16, 0),
+    ([300, 5, 129], [300, 5, 129], 6, 2, 48, 16, 0),
+    ([700, 33, 1], [1, 1, 1], 8, 8, 128, 16, 0),          # decoding, long context: keys are split
+    ([513, 260], [2, 17], 4, 1, 64, 32, 0),               # portions on top of a context
+    ([400, 90, 31], [400, 1, 31], 3, 3, 16, 16, 24),      # window
+    ([1000, 999], [1, 3], 2, 1, 80, 64, 100),             # window, decoding, big pages
+    ([2100], [1], 16, 16, 128, 16, 0),
+]
+
+
+@pytest.mark.parametrize("case", ATTN_CASES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_plain(case, dtype):
+    from inferx_amd import ops
+    seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    if sum(q_lens) * max(seq_lens) > 300 * 400:
+        pytest.skip("large for the plain kernel's test")
+    p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, dtype, seed=3)
+    out = torch.empty_like(p["q"])
+    scale = d ** -0.5
+    ops.attention_plain(p["q"], p["k_cache"], p["v_cache"], p["table"], p["seq_of_token"], p["positions"], out, scale,
+                        window)
+    close(out, attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window), TOL[dtype], "attention_plain")
+
+
+def tiles_for(q_lens):
+    rows, at = [], 0
+    for s, n in enumerate(q_lens):
+        for q0 in range(0, n, 16):
+            rows.append((s, at + q0, min(16, n - q0)))
+        at += n
+    return torch.tensor(rows, dtype=torch.int32).t().contiguous().to(DEV)
+
+
+@pytest.mark.parametrize("n_splits", [1, 3, 8])
+@pytest.mark.parametrize("case", ATTN_CASES)
+def test_attention_mfma(case, n_splits):
+    from inferx_amd import ops
+    seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, torch.bfloat16, seed=4)
+    out = torch.full_like(p["q"], float("nan"))
+    T = p["q"].shape[0]
+    work = torch.empty(T * heads * n_splits * (d + 2), dtype=torch.float32, device=DEV) if n_splits > 1 else None
+    scale = d ** -0.5
+    ops.attention_mfma(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for(q_lens), p["positions"], out,
+                       n_splits, work, scale, window)
+    close(out, attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window), TOL[torch.bfloat16],
+          f"attention_mfma splits={n_splits}")
+
+
+def test_attention_finds_one_far_key():
+    """One key among 2,000 matches the query: the output must be that key's value (a skipped page, a wrong
+    split boundary or a wrong table entry would miss it)."""
+    from inferx_amd import ops
+    L, d, heads = 2000, 64, 2
+    for far in (0, 15, 16, 777, 1024, 1999):
+        p = build_paged([L], [1], heads, heads, d, 16, torch.bfloat16, seed=far)
+        k, v = p["dense"][0]
+        q = p["qs"][0]
+        # rewrite the far key in the cache so that q . k is large there
+        page, off = int(p["table"][0, far // 16]), far % 16
+        p["k_cache"][page, :, off, :] = (q[0] * 4.0).to(DEV)
+        k[far] = q[0] * 4.0
+        for n_splits in (1, 5):
+            out = torch.empty_like(p["q"])
+            work = torch.empty(heads * n_splits * (d + 2), dtype=torch.float32, device=DEV)
+            ops.attention_mfma(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for([1]), p["positions"], out,
+                               n_splits, work, d ** -0.5, 0)
+            want = attention_reference(p, [L], [1], heads, heads, d ** -0.5, 0)
+            close(out, want, TOL[torch.bfloat16], f"far key {far}")
+            assert float((out[0].float().cpu() - v[far].float()).abs().max()) < 0.05 * float(v[far].abs().max())
