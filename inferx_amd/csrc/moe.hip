@@ -114,10 +114,16 @@ extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dty
 //   dest[A]         assignment  -> grouped row
 // stable: within an expert, rows keep assignment order
 // (reference: MoeBuildDispatch, moe.cu:452-513; kernels :130-221).
+// Also, for the matrix-core product, a map of row tiles: tile i covers rows
+// [tile_row0[i], min(tile_row0[i] + tile_rows, end of its expert)) of expert
+// tile_expert[i]; tile_info[0] = number of tiles.
 __global__ void __launch_bounds__(1024)
 moe_count_scan_kernel(const int32_t* __restrict__ topk_e, int32_t* __restrict__ offsets, int64_t assignments,
-                      int experts) {
+                      int experts, int tile_rows, int32_t* __restrict__ tile_expert,
+                      int32_t* __restrict__ tile_row0, int32_t* __restrict__ tile_info) {
   __shared__ int32_t counts[IX_MAX_EXPERTS];
+  __shared__ int32_t first_row[IX_MAX_EXPERTS];
+  __shared__ int32_t first_tile[IX_MAX_EXPERTS];
   for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
   __syncthreads();
   for (int64_t a = threadIdx.x; a < assignments; a += blockDim.x) {
@@ -126,12 +132,26 @@ moe_count_scan_kernel(const int32_t* __restrict__ topk_e, int32_t* __restrict__ 
   }
   __syncthreads();
   if (threadIdx.x == 0) {
-    int32_t run = 0;
+    int32_t run = 0, tiles = 0;
     for (int e = 0; e < experts; ++e) {
       offsets[e] = run;
+      first_row[e] = run;
+      first_tile[e] = tiles;
       run += counts[e];
+      if (tile_rows > 0) tiles += (counts[e] + tile_rows - 1) / tile_rows;
     }
     offsets[experts] = run;
+    if (tile_info) tile_info[0] = tiles;
+  }
+  __syncthreads();
+  if (tile_rows > 0 && tile_expert) {
+    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
+      const int n = (counts[e] + tile_rows - 1) / tile_rows;
+      for (int i = 0; i < n; ++i) {
+        tile_expert[first_tile[e] + i] = e;
+        tile_row0[first_tile[e] + i] = first_row[e] + i * tile_rows;
+      }
+    }
   }
 }
 
@@ -164,11 +184,16 @@ moe_scatter_kernel(const int32_t* __restrict__ topk_e, const int32_t* __restrict
   }
 }
 
+// tile_expert / tile_row0 need room for min(A, ceil(A / tile_rows) + E) entries; tile_rows 0 skips the map.
 extern "C" int ix_moe_dispatch(const int32_t* topk_e, int32_t* offsets, int32_t* rows, int32_t* dest,
-                               int64_t assignments, int experts, int k, hipStream_t stream) {
+                               int64_t assignments, int experts, int k, int tile_rows, int32_t* tile_expert,
+                               int32_t* tile_row0, int32_t* tile_info, hipStream_t stream) {
   IX_REQUIRE(assignments >= 0 && k > 0, "sizes must be positive");
   IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
-  hipLaunchKernelGGL(moe_count_scan_kernel, dim3(1), dim3(1024), 0, stream, topk_e, offsets, assignments, experts);
+  IX_REQUIRE(tile_rows >= 0, "tile_rows must not be negative");
+  IX_REQUIRE(tile_rows == 0 || (tile_expert && tile_row0 && tile_info), "tile map buffers needed");
+  hipLaunchKernelGGL(moe_count_scan_kernel, dim3(1), dim3(1024), 0, stream, topk_e, offsets, assignments, experts,
+                     tile_rows, tile_expert, tile_row0, tile_info);
   if (assignments > 0)
     hipLaunchKernelGGL(moe_scatter_kernel, dim3(experts), dim3(256), 0, stream, topk_e, offsets, rows, dest,
                        assignments, k);

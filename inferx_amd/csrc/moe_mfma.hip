@@ -1,0 +1,169 @@
+// Grouped expert products on the matrix cores (bfloat16 in, float32 accumulate).
+//
+//   GATE_UP: act[r, n] = silu(x[rows[r]] . W[e][n]) * (x[rows[r]] . W[e][N + n]),  W [E, 2N, K]
+//   else:    y[r, n]   = a[r] . W[e][n],                                           W [E, N, K]
+// for the rows r of expert e, taken from the row-tile map that the grouping
+// kernel wrote (reference: GroupedGemmBf16Kernel, src/backends/cuda/ops/moe.cu:323-392,
+// which uses scalar FMAs; SwiGLU src/model/moe_ffn.cc:288-291).
+//
+// The product is formed transposed, out^T[n][r] = W[n][:] . x[r][:], so that the
+// big operand, the expert's weight rows, is the A operand and streams from
+// memory straight into registers: v_mfma_f32_16x16x32_bf16, A = 16 weight rows,
+// B = 16 activation rows, lane l of the result holding out-features 4*(l/16)+i
+// of row l%16, i.e. four consecutive numbers of one output row.
+//
+// A wavefront owns 16 out-features x (16 * MT) rows.  Per iteration it covers
+// 128 of K: lane (m, g) reads 64 contiguous bytes of weight row m (k0 + 32 g ..
+// + 32), as four 16-byte pieces j; piece j of all four lane groups forms the 32
+// reduction slots of MFMA j, and the activations are read with the same
+// mapping.  KSPLIT = 4 (decoding: few rows, the weights are the traffic) lets
+// the four wavefronts of a workgroup take a quarter of K each and add up through
+// LDS; KSPLIT = 1 gives each wavefront its own 16 out-features.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+template <int MT, bool GATE_UP, int KSPLIT>
+__global__ void __launch_bounds__(256)
+moe_grouped_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w, __bf16* __restrict__ out,
+                        const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
+                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
+                        const int32_t* __restrict__ tile_info, int n_out, int width) {
+  constexpr int NACC = GATE_UP ? 2 : 1;
+  __shared__ float red[KSPLIT > 1 ? 3 * 64 * MT * NACC * 4 : 1];
+  if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int m = lane & 15, g = lane >> 4;
+  const int e = tile_expert[blockIdx.y];
+  const int row0 = tile_row0[blockIdx.y];
+  const int row_end = offsets[e + 1];
+
+  const int n0 = (KSPLIT > 1 ? blockIdx.x : blockIdx.x * 4 + wave) * 16;
+  if (n0 >= n_out) return;  // whole wavefront (KSPLIT == 1) or whole workgroup
+  const int kper = KSPLIT > 1 ? (((width + KSPLIT - 1) / KSPLIT + 127) & ~127) : width;
+  const int kbegin = KSPLIT > 1 ? wave * kper : 0;
+  const int kend = min(width, kbegin + kper);
+
+  const int64_t w_rows = GATE_UP ? 2 * static_cast<int64_t>(n_out) : n_out;
+  const int wrow = min(n0 + m, n_out - 1);  // rows past the end are computed and not stored
+  const __bf16* wg = w + (static_cast<int64_t>(e) * w_rows + wrow) * width;
+  const __bf16* wu = wg + static_cast<int64_t>(n_out) * width;
+
+  const __bf16* xr[MT];
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int r = min(row0 + 16 * t + m, row_end - 1);
+    xr[t] = a + static_cast<int64_t>(rows ? rows[r] : r) * width;
+  }
+
+  f32x4 acc[NACC][MT];
+#pragma unroll
+  for (int u = 0; u < NACC; ++u)
+#pragma unroll
+    for (int t = 0; t < MT; ++t) acc[u][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
+                       (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+  for (int k0 = kbegin; k0 < kend; k0 += 128) {
+    bf16x8 fw[NACC][4], fx[MT][4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int kk = k0 + 32 * g + 8 * j;
+      const bool ok = kk < kend;
+      fw[0][j] = ok ? *reinterpret_cast<const bf16x8*>(wg + kk) : zero;
+      if (GATE_UP) fw[1][j] = ok ? *reinterpret_cast<const bf16x8*>(wu + kk) : zero;
+#pragma unroll
+      for (int t = 0; t < MT; ++t) fx[t][j] = ok ? *reinterpret_cast<const bf16x8*>(xr[t] + kk) : zero;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int t = 0; t < MT; ++t)
+#pragma unroll
+        for (int u = 0; u < NACC; ++u)
+          acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[u][j], fx[t][j], acc[u][t], 0, 0, 0);
+  }
+
+  if (KSPLIT > 1) {
+    // wavefronts 1..3 hand their partial sums to wavefront 0
+    if (wave > 0) {
+      float* dst = red + ((wave - 1) * 64 + lane) * (MT * NACC * 4);
+#pragma unroll
+      for (int u = 0; u < NACC; ++u)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) dst[(u * MT + t) * 4 + i] = acc[u][t][i];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int s = 0; s < KSPLIT - 1; ++s) {
+      const float* src = red + (s * 64 + lane) * (MT * NACC * 4);
+#pragma unroll
+      for (int u = 0; u < NACC; ++u)
+#pragma unroll
+        for (int t = 0; t < MT; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[u][t][i] += src[(u * MT + t) * 4 + i];
+    }
+  }
+
+  // lane holds out-features n0 + 4 g + i of row row0 + 16 t + m
+  const int nb = n0 + 4 * g;
+#pragma unroll
+  for (int t = 0; t < MT; ++t) {
+    const int r = row0 + 16 * t + m;
+    if (r >= row_end) continue;
+    float v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[i] = acc[0][t][i];
+      if (GATE_UP) v[i] = v[i] / (1.0f + __expf(-v[i])) * acc[1][t][i];
+    }
+    __bf16* dst = out + static_cast<int64_t>(r) * n_out + nb;
+    if (nb + 4 <= n_out && (n_out & 3) == 0) {
+      bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+      *reinterpret_cast<bf16x4*>(dst) = o;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (nb + i < n_out) dst[i] = (__bf16)v[i];
+    }
+  }
+}
+
+// `max_tiles` bounds the number of row tiles (the grid); the kernel reads the true number from tile_info.
+// tile_rows (16, 32 or 64) must be what the grouping kernel was given.
+extern "C" int ix_moe_grouped_mfma(const void* a, const void* w, void* out, const int32_t* offsets,
+                                   const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
+                                   const int32_t* tile_info, int max_tiles, int tile_rows, int64_t n_out,
+                                   int64_t width, int gate_up, int k_split, hipStream_t stream) {
+  IX_REQUIRE(n_out > 0 && width > 0 && max_tiles >= 0, "sizes must be positive");
+  IX_REQUIRE(width % 8 == 0, "the reduction width must be a multiple of 8 for the matrix-core kernel");
+  IX_REQUIRE(n_out < (1 << 30) && width < (1 << 30), "sizes too large");
+  IX_REQUIRE(tile_rows == 16 || tile_rows == 32 || tile_rows == 64, "tile_rows must be 16, 32 or 64");
+  IX_REQUIRE(k_split == 1 || k_split == 4, "k_split must be 1 or 4");
+  IX_REQUIRE(max_tiles <= 65535, "too many row tiles for one launch");
+  if (max_tiles == 0) return 0;
+  const int n_tiles16 = static_cast<int>((n_out + 15) / 16);
+  dim3 grid(k_split > 1 ? n_tiles16 : (n_tiles16 + 3) / 4, max_tiles), block(256);
+#define LAUNCH(MT, GU, KS)                                                                                        \
+  hipLaunchKernelGGL((moe_grouped_mfma_kernel<MT, GU, KS>), grid, block, 0, stream, (const __bf16*)a,             \
+                     (const __bf16*)w, (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, \
+                     (int)width)
+#define PICK(MT)                                       \
+  if (gate_up) {                                       \
+    if (k_split > 1) LAUNCH(MT, true, 4);              \
+    else LAUNCH(MT, true, 1);                          \
+  } else {                                             \
+    if (k_split > 1) LAUNCH(MT, false, 4);             \
+    else LAUNCH(MT, false, 1);                         \
+  }
+  if (tile_rows == 16) { PICK(1) } else if (tile_rows == 32) { PICK(2) } else { PICK(4) }
+#undef PICK
+#undef LAUNCH
+  return ix_check_launch("ix_moe_grouped_mfma");
+}

@@ -226,16 +226,53 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
 
 
 def moe_dispatch(topk_e: torch.Tensor, offsets: torch.Tensor, rows: torch.Tensor, dest: torch.Tensor,
-                 experts: int) -> None:
-    """Group assignments by expert: offsets [E+1], rows [A] (grouped row -> token), dest [A]."""
+                 experts: int, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None) -> None:
+    """Group assignments by expert: offsets [E+1], rows [A] (grouped row -> token), dest [A].
+    With tile_rows > 0 also the row-tile map for the matrix-core product: `tile_map` int32
+    [2 * max_tiles + 1] = tile_expert | tile_row0 | number of tiles, max_tiles = moe_max_tiles(A, E, tile_rows)."""
     T, k = topk_e.shape
     A = T * k
     _is_i32(topk_e)
     _is_i32(offsets, experts + 1)
     _is_i32(rows, A)
     _is_i32(dest, A)
+    te = tr = ti = None
+    if tile_rows > 0:
+        mt = moe_max_tiles(A, experts, tile_rows)
+        _need(tile_map is not None, "tile_map needed")
+        _is_i32(tile_map, 2 * mt + 1)
+        te, tr, ti = tile_map[:mt], tile_map[mt:2 * mt], tile_map[2 * mt:]
     _call("ix_moe_dispatch", _ptr(topk_e), _ptr(offsets), _ptr(rows), _ptr(dest), _i64(A), _i32(experts), _i32(k),
-          _stream())
+          _i32(tile_rows), _ptr(te), _ptr(tr), _ptr(ti), _stream())
+
+
+def moe_max_tiles(assignments: int, experts: int, tile_rows: int) -> int:
+    """Upper bound of the number of row tiles: every expert may end with a partial tile."""
+    return max(1, min(assignments, -(-assignments // tile_rows) + experts))
+
+
+def moe_grouped_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
+                     rows: Optional[torch.Tensor], tile_map: torch.Tensor, tile_rows: int, gate_up: bool,
+                     k_split: int) -> None:
+    """Grouped product on the matrix cores (bfloat16), shapes as `moe_grouped_plain`; `tile_map` from `moe_dispatch`."""
+    E = w.shape[0]
+    A, n_out = out.shape
+    K = a.shape[1]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
+          "the matrix-core grouped product is bfloat16 only")
+    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if gate_up else n_out),
+          "expert weight shape does not fit")
+    _need(K % 8 == 0, "the reduction width must be a multiple of 8")
+    _is_i32(offsets, E + 1)
+    if rows is not None:
+        _is_i32(rows, A)
+    else:
+        _need(a.shape[0] >= A, "a has fewer rows than out")
+    mt = moe_max_tiles(A, E, tile_rows)
+    _is_i32(tile_map, 2 * mt + 1)
+    _call("ix_moe_grouped_mfma", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
+          _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i32(tile_rows), _i64(n_out), _i64(K),
+          _i32(1 if gate_up else 0), _i32(k_split), _stream())
 
 
 def moe_grouped_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,

@@ -74,20 +74,37 @@ class MoeFeedForward(FeedForward):
         ops.moe_route(x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate, self.renormalize, self.routed_scale)
         return topk_w, topk_e, gate
 
-    def dispatch(self, ctx, topk_e):
+    def _tile_rows(self, x) -> int:
+        """Rows per tile of the matrix-core product, or 0 where it does not take the shapes (then the plain one runs)."""
+        ok = (x.dtype == torch.bfloat16 and self.w13.dtype == torch.bfloat16 and self.w2.dtype == torch.bfloat16
+              and self.hidden_size % 8 == 0 and self.expert_width % 8 == 0)
+        if not ok:
+            return 0
+        per_expert = x.shape[0] * self.top_k / self.num_experts
+        return 16 if per_expert <= 16 else (32 if per_expert <= 32 else 64)
+
+    def dispatch(self, ctx, topk_e, tile_rows: int = 0):
         rt, A = ctx.rt, topk_e.numel()
         offsets = rt.empty((self.num_experts + 1,), torch.int32)
         rows = rt.empty((A,), torch.int32)
         dest = rt.empty((A,), torch.int32)
-        ops.moe_dispatch(topk_e, offsets, rows, dest, self.num_experts)
-        return offsets, rows, dest
+        tile_map = None
+        if tile_rows:
+            tile_map = rt.empty((2 * ops.moe_max_tiles(A, self.num_experts, tile_rows) + 1,), torch.int32)
+        ops.moe_dispatch(topk_e, offsets, rows, dest, self.num_experts, tile_rows, tile_map)
+        return offsets, rows, dest, tile_map
 
-    def experts(self, ctx, x, offsets, rows):
+    def experts(self, ctx, x, offsets, rows, tile_map=None, tile_rows: int = 0):
         rt, A = ctx.rt, rows.numel()
         act = rt.empty((A, self.expert_width))
-        ops.moe_grouped_plain(x, self.w13, act, offsets, rows, gate_up=True)
         y = rt.empty((A, self.hidden_size))
-        ops.moe_grouped_plain(act, self.w2, y, offsets, None, gate_up=False)
+        if tile_rows:
+            k_split = 4 if A <= 1024 else 1  # few rows: the weights are the traffic, split the reduction
+            ops.moe_grouped_mfma(x, self.w13, act, offsets, rows, tile_map, tile_rows, True, k_split)
+            ops.moe_grouped_mfma(act, self.w2, y, offsets, None, tile_map, tile_rows, False, k_split)
+        else:
+            ops.moe_grouped_plain(x, self.w13, act, offsets, rows, gate_up=True)
+            ops.moe_grouped_plain(act, self.w2, y, offsets, None, gate_up=False)
         return y
 
     def shared(self, ctx, x):
@@ -99,8 +116,9 @@ class MoeFeedForward(FeedForward):
 
     def forward(self, ctx, x):
         topk_w, topk_e, gate = self.route(ctx, x)
-        offsets, rows, dest = self.dispatch(ctx, topk_e)
-        y = self.experts(ctx, x, offsets, rows)
+        tile_rows = self._tile_rows(x)
+        offsets, rows, dest, tile_map = self.dispatch(ctx, topk_e, tile_rows)
+        y = self.experts(ctx, x, offsets, rows, tile_map, tile_rows)
         shared = self.shared(ctx, x) if self.shared_width > 0 else None
         out = ctx.rt.empty((x.shape[0], self.hidden_size))
         ops.moe_combine(y, dest, topk_w, shared, gate, out)

@@ -1,0 +1,199 @@
+"""The mixture-of-experts kernels alone against PyTorch references: router, grouping,
+grouped products (plain and matrix-core), combine.  Properties follow the reference's
+tests/kernel/moe_test.cc (lines cited per test)."""
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def rel_err(got, want):
+    want = want.double().cpu()
+    return float((got.double().cpu() - want).abs().max()) / max(float(want.abs().max()), 1e-30)
+
+
+def route_reference(x, wr, k, renorm, scale=1.0):
+    p = torch.softmax(x.double().cpu() @ wr.double().cpu().T, -1)
+    w, e = torch.topk(p, k, dim=-1)
+    if renorm:
+        w = w / w.sum(-1, keepdim=True)
+    return w * scale, e
+
+
+@pytest.mark.parametrize("T,H,E,k,renorm", [(24, 64, 8, 2, False), (7, 200, 60, 4, True), (130, 72, 5, 1, False),
+                                            (3, 2048, 64, 8, True), (50, 96, 32, 32, True)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_route(T, H, E, k, renorm, dtype):
+    # reference: moe_test.cc:170-246 (router equals host to 1e-5, renormalised sums to 1, un-normalised below)
+    from inferx_amd import ops
+    x, wr, wsg = rnd(T, H, dtype=dtype), rnd(E, H, seed=1, dtype=dtype, scale=0.3), rnd(1, H, seed=2, dtype=dtype, scale=0.1)
+    topk_w = torch.empty(T, k, dtype=torch.float32, device=DEV)
+    topk_e = torch.empty(T, k, dtype=torch.int32, device=DEV)
+    gate = torch.empty(T, dtype=torch.float32, device=DEV)
+    ops.moe_route(x, wr, wsg, topk_w, topk_e, gate, renorm, 1.0)
+    want_w, want_e = route_reference(x, wr, k, renorm)
+    assert torch.equal(topk_e.cpu().long(), want_e)
+    assert rel_err(topk_w, want_w) < 1e-5
+    assert rel_err(gate, torch.sigmoid(x.double().cpu() @ wsg.double().cpu().T)[:, 0]) < 1e-5
+    sums = topk_w.sum(-1).cpu()
+    if renorm:
+        assert torch.allclose(sums, torch.ones(T), atol=1e-5)
+    elif k < E:
+        assert (sums < 0.9999).all()
+
+
+def test_route_refuses_what_it_cannot_do():
+    from inferx_amd import ops
+    x, wr = rnd(4, 96), rnd(40, 96, seed=1)
+    with pytest.raises(ops.KernelError, match="top_k"):
+        ops.moe_route(x, wr, None, torch.empty(4, 33, device=DEV), torch.empty(4, 33, dtype=torch.int32, device=DEV),
+                      None, False, 1.0)
+
+
+def test_route_equal_logits_take_the_lowest_indices():
+    # reference vector: moe_test.cc:248-273
+    from inferx_amd import ops
+    T, H, E, k = 5, 16, 32, 2
+    x = torch.ones(T, H, device=DEV)
+    wr = torch.full((E, H), 0.25 / H, device=DEV)
+    topk_w = torch.empty(T, k, device=DEV)
+    topk_e = torch.empty(T, k, dtype=torch.int32, device=DEV)
+    ops.moe_route(x, wr, None, topk_w, topk_e, None, False, 1.0)
+    assert topk_e.cpu().tolist() == [[0, 1]] * T
+    assert torch.allclose(topk_w.cpu(), torch.full((T, k), 1 / 32))
+
+
+def dispatch(topk_e, E, tile_rows=0):
+    from inferx_amd import ops
+    T, k = topk_e.shape
+    A = T * k
+    offsets = torch.empty(E + 1, dtype=torch.int32, device=DEV)
+    rows = torch.empty(A, dtype=torch.int32, device=DEV)
+    dest = torch.empty(A, dtype=torch.int32, device=DEV)
+    tile_map = None
+    if tile_rows:
+        tile_map = torch.full((2 * ops.moe_max_tiles(A, E, tile_rows) + 1,), -7, dtype=torch.int32, device=DEV)
+    ops.moe_dispatch(topk_e, offsets, rows, dest, E, tile_rows, tile_map)
+    return offsets, rows, dest, tile_map
+
+
+@pytest.mark.parametrize("T,E,k,tile_rows", [(24, 8, 2, 16), (300, 60, 4, 32), (1, 4, 2, 16), (1000, 7, 3, 64),
+                                             (40, 64, 1, 0)])
+def test_dispatch_is_a_stable_bijection(T, E, k, tile_rows):
+    # reference: moe_test.cc:277-350
+    g = torch.Generator().manual_seed(T)
+    topk_e = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    if E > 3:
+        topk_e[topk_e == 2] = 3  # expert 2 stays empty (an assignment may then repeat expert 3; fine for grouping)
+    offsets, rows, dest, tile_map = dispatch(topk_e.to(DEV), E, tile_rows)
+    offsets, rows, dest = offsets.cpu(), rows.cpu(), dest.cpu()
+    flat = topk_e.flatten()
+    A = T * k
+    assert offsets[0] == 0 and offsets[E] == A
+    assert sorted(dest.tolist()) == list(range(A))  # every assignment exactly once
+    for a in range(A):
+        e = int(flat[a])
+        assert offsets[e] <= dest[a] < offsets[e + 1]      # in its expert's range
+        assert rows[dest[a]] == a // k                      # rows and dest are inverse
+    if E > 3:
+        assert offsets[2] == offsets[3]                     # an empty expert has an empty range
+    for e in range(E):
+        mine = [int(dest[a]) for a in range(A) if int(flat[a]) == e]
+        assert mine == sorted(mine)                         # stable: assignment order is kept
+    if tile_rows:
+        mt = (tile_map.numel() - 1) // 2
+        n = int(tile_map[2 * mt])
+        te, tr = tile_map[:n].cpu().tolist(), tile_map[mt:mt + n].cpu().tolist()
+        covered = []
+        for e_, r0 in zip(te, tr):
+            assert offsets[e_] <= r0 < offsets[e_ + 1]
+            covered += list(range(r0, min(r0 + tile_rows, int(offsets[e_ + 1]))))
+        assert covered == list(range(A))  # tiles cover every row once, in order
+
+
+def grouped_reference(a, w, offsets, rows, gate_up):
+    a, w = a.double().cpu(), w.double().cpu()
+    E = w.shape[0]
+    A = int(offsets[E])
+    n = w.shape[1] // 2 if gate_up else w.shape[1]
+    out = torch.zeros(A, n, dtype=torch.float64)
+    for e in range(E):
+        for r in range(int(offsets[e]), int(offsets[e + 1])):
+            x = a[int(rows[r])] if rows is not None else a[r]
+            z = w[e] @ x
+            out[r] = torch.nn.functional.silu(z[:n]) * z[n:] if gate_up else z
+    return out
+
+
+GROUPED = [(24, 64, 8, 2, 32), (300, 96, 8, 3, 48), (9, 72, 5, 1, 40), (700, 256, 60, 4, 176), (3, 2048, 60, 4, 1408)]
+
+
+@pytest.mark.parametrize("T,H,E,k,mi", GROUPED)
+@pytest.mark.parametrize("dtype,wdtype", [(torch.float32, torch.float32), (torch.bfloat16, torch.bfloat16),
+                                          (torch.bfloat16, torch.float32)])
+def test_grouped_plain(T, H, E, k, mi, dtype, wdtype):
+    from inferx_amd import ops
+    if T * mi * H > 300 * 96 * 48 * 40:
+        pytest.skip("large for the plain kernel's test")
+    g = torch.Generator().manual_seed(1)
+    topk_e = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    offsets, rows, dest, _ = dispatch(topk_e, E)
+    x = rnd(T, H, dtype=dtype)
+    w13, w2 = rnd(E, 2 * mi, H, seed=2, dtype=wdtype, scale=H ** -0.5), rnd(E, H, mi, seed=3, dtype=wdtype, scale=mi ** -0.5)
+    act = torch.empty(T * k, mi, dtype=dtype, device=DEV)
+    ops.moe_grouped_plain(x, w13, act, offsets, rows, True)
+    tol = 1e-5 if dtype == torch.float32 else 1.5e-2
+    assert rel_err(act, grouped_reference(x, w13, offsets.cpu(), rows.cpu(), True)) < tol
+    y = torch.empty(T * k, H, dtype=dtype, device=DEV)
+    ops.moe_grouped_plain(act, w2, y, offsets, None, False)
+    assert rel_err(y, grouped_reference(act, w2, offsets.cpu(), None, False)) < tol
+
+
+@pytest.mark.parametrize("T,H,E,k,mi", GROUPED)
+@pytest.mark.parametrize("tile_rows", [16, 32, 64])
+@pytest.mark.parametrize("k_split", [1, 4])
+def test_grouped_mfma(T, H, E, k, mi, tile_rows, k_split):
+    from inferx_amd import ops
+    g = torch.Generator().manual_seed(1)
+    topk_e = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    offsets, rows, dest, tile_map = dispatch(topk_e, E, tile_rows)
+    x = rnd(T, H, dtype=torch.bfloat16)
+    w13 = rnd(E, 2 * mi, H, seed=2, dtype=torch.bfloat16, scale=H ** -0.5)
+    w2 = rnd(E, H, mi, seed=3, dtype=torch.bfloat16, scale=mi ** -0.5)
+    act = torch.full((T * k, mi), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.moe_grouped_mfma(x, w13, act, offsets, rows, tile_map, tile_rows, True, k_split)
+    assert rel_err(act, grouped_reference(x, w13, offsets.cpu(), rows.cpu(), True)) < 1.5e-2
+    y = torch.full((T * k, H), float("nan"), dtype=torch.bfloat16, device=DEV)
+    ops.moe_grouped_mfma(act, w2, y, offsets, None, tile_map, tile_rows, False, k_split)
+    assert rel_err(y, grouped_reference(act, w2, offsets.cpu(), None, False)) < 1.5e-2
+    # bitwise repeatable (reference: moe_test.cc:972-1046)
+    y2 = torch.empty_like(y)
+    ops.moe_grouped_mfma(act, w2, y2, offsets, None, tile_map, tile_rows, False, k_split)
+    assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gather_then_combine_is_the_identity(dtype):
+    # reference: moe_test.cc:352-411 (weights 0.25 / 0.75)
+    from inferx_amd import ops
+    T, H, E, k = 24, 64, 8, 2
+    g = torch.Generator().manual_seed(2)
+    topk_e = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    offsets, rows, dest, _ = dispatch(topk_e, E)
+    x = rnd(T, H, dtype=dtype)
+    y = x[rows.long()]  # what an identity expert would produce
+    topk_w = torch.tensor([[0.25, 0.75]] * T, device=DEV)
+    out = torch.empty_like(x)
+    ops.moe_combine(y, dest, topk_w, None, None, out)
+    assert rel_err(out, x) < (1e-6 if dtype == torch.float32 else 1e-2)
+    shared, gate = rnd(T, H, seed=5, dtype=dtype), torch.rand(T, device=DEV)
+    ops.moe_combine(y, dest, topk_w, shared, gate, out)
+    assert rel_err(out, x.double() + gate.double()[:, None] * shared.double()) < (1e-6 if dtype == torch.float32 else 1e-2)
+    ops.moe_combine(y, dest, topk_w, shared, None, out)  # an ungated shared expert adds exactly its output
+    assert rel_err(out, x.double() + shared.double()) < (1e-6 if dtype == torch.float32 else 1e-2)
