@@ -24,7 +24,7 @@ moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dt
                  const void* __restrict__ shared_gate_w, int sg_dtype, float* __restrict__ topk_w,
                  int32_t* __restrict__ topk_e, float* __restrict__ shared_gate, int64_t width, int experts, int k,
                  int renormalize, float scale) {
-  extern __shared__ float smem[];
+  extern __shared__ __align__(16) float smem[];
   float* xs = smem;            // [width]
   float* z = smem + width;     // [experts + 1]
   __shared__ float red[16];
@@ -38,7 +38,28 @@ moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dt
     const int dt = e < experts ? wr_dtype : sg_dtype;
     const int64_t base = e < experts ? static_cast<int64_t>(e) * width : 0;
     float dot = 0.f;
-    for (int64_t i = lane; i < width; i += 64) dot += xs[i] * ix_load_rt(w, dt, base + i);
+    if (dt == IX_BF16 && (width & 7) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+      // eight weights per lane and load (16 bytes); the order of additions is fixed by the lane layout
+      const uint16_t* wrow = static_cast<const uint16_t*>(w) + base;
+      for (int64_t i = lane * 8; i < width; i += 512) {
+        const uint4 v = *reinterpret_cast<const uint4*>(wrow + i);
+        const float4 x0 = *reinterpret_cast<const float4*>(xs + i);
+        const float4 x1 = *reinterpret_cast<const float4*>(xs + i + 4);
+        dot += x0.x * __uint_as_float(v.x << 16) + x0.y * __uint_as_float(v.x & 0xffff0000u) +
+               x0.z * __uint_as_float(v.y << 16) + x0.w * __uint_as_float(v.y & 0xffff0000u) +
+               x1.x * __uint_as_float(v.z << 16) + x1.y * __uint_as_float(v.z & 0xffff0000u) +
+               x1.z * __uint_as_float(v.w << 16) + x1.w * __uint_as_float(v.w & 0xffff0000u);
+      }
+    } else if (dt == IX_F32 && (width & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+      const float* wrow = static_cast<const float*>(w) + base;
+      for (int64_t i = lane * 4; i < width; i += 256) {
+        const float4 v = *reinterpret_cast<const float4*>(wrow + i);
+        const float4 x0 = *reinterpret_cast<const float4*>(xs + i);
+        dot += x0.x * v.x + x0.y * v.y + x0.z * v.z + x0.w * v.w;
+      }
+    } else {
+      for (int64_t i = lane; i < width; i += 64) dot += xs[i] * ix_load_rt(w, dt, base + i);
+    }
     dot = ix_wave_sum(dot);
     if (lane == 0) z[e] = dot;
   }

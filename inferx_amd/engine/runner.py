@@ -7,10 +7,16 @@ batch, against the cache that earlier steps left, and returns float32 logits
 at the wanted rows (reference: Qwen2Model::Step, src/model/qwen2.cc:2246-2277;
 PrepareBatchInputs :564-817).  It holds no policy: who runs, in which portions,
 and what happens when pages run out is decided above it (scheduler, replay).
+
+Steps in which every request brings one token are launch-bound, so they are
+captured once per (batch size, context bucket) into a HIP graph and replayed
+(reference: CaptureDecodeGraph, src/model/qwen2.cc:1588-1712).  The graph reads
+its indices from one static device buffer that each step refills with a single
+copy; kernels, buffers and results are those of the eager path.
 """
 from __future__ import annotations
 
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -22,10 +28,22 @@ from ..weights import load_weights
 from .batch import Entry, StepBatch, build_step_batch
 from .runtime import CacheBinding, Runtime, StepContext
 
+N_FIXED = 7  # token_ids, positions, seq_of_token, q_start, seq_lens, state_slots, logits_rows
+
+
+def _pack(batch: StepBatch) -> Tuple[List[int], np.ndarray]:
+    parts = [batch.token_ids, batch.positions, batch.seq_of_token, batch.q_start, batch.seq_lens,
+             batch.state_slots, batch.logits_rows] + list(batch.slots) + [t.reshape(-1) for t in batch.block_tables]
+    sizes = [int(p.size) for p in parts]
+    if not sum(sizes):
+        return sizes, np.zeros(0, np.int32)
+    return sizes, np.concatenate([np.ascontiguousarray(p, dtype=np.int32).reshape(-1) for p in parts])
+
 
 class ModelRunner:
     def __init__(self, config, weights: Dict[str, torch.Tensor], rt: Runtime, *, page_size: int = 16,
-                 num_pages: int = 256, max_requests: int = 8, max_seq_len: Optional[int] = None, model=None):
+                 num_pages: int = 256, max_requests: int = 8, max_seq_len: Optional[int] = None, model=None,
+                 use_graphs: bool = True):
         self.config = config
         self.rt = rt
         self.spec = config.model_spec()
@@ -36,6 +54,7 @@ class ModelRunner:
             max_seq_len = self.spec.max_positions if self.spec.max_positions > 0 else num_pages * page_size
         self.max_seq_len = int(max_seq_len)
         self.max_requests = int(max_requests)
+        self.use_graphs = bool(use_graphs) and self.model.graph_safe()
         self._lay_out_cache(int(num_pages))
 
     @classmethod
@@ -73,16 +92,17 @@ class ModelRunner:
                     raise ValueError(f"schedule entry {i} reads the cache of entry {src}, whose layout differs")
                 g = needs.index(need)
                 j = owners[g].index(src)
-                n_ = needs[g]
                 b.group, b.k, b.writes = g, self.kv[g][j, 0], cache_from is None
                 # values are kept transposed within a page: [pages, kv_heads, head_dim, page_size]
-                b.v = self.kv[g][j, 1].view(-1, n_.kv_heads, n_.head_dim, self.page_size)
+                b.v = self.kv[g][j, 1].view(-1, need.kv_heads, need.head_dim, self.page_size)
             if state is not None:
                 b.state = torch.zeros((self.max_requests,) + tuple(state.shape), dtype=torch.float32,
                                       device=rt.device)
             self.bindings.append(b)
         self.cache = CacheManager([GroupLayout(n.window) for n in needs], [num_pages] * len(needs), self.page_size,
                                   self.max_requests, self.max_seq_len)
+        self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
+        self._graph_pool = None
 
     def kv_bytes_per_token(self) -> int:
         size = torch.empty((), dtype=self.rt.dtype).element_size()
@@ -92,32 +112,50 @@ class ModelRunner:
     def step(self, batch: StepBatch) -> torch.Tensor:
         """Run the batch; float32 logits [len(batch.logits_rows), vocab] on the device."""
         batch.validate(self.spec.vocab_size, [p.num_pages for p in self.cache.pools], self.page_size)
-        ctx = self._upload(batch)
-        for b in self.bindings:
-            if b.state is not None:
-                fresh = [int(batch.state_slots[s]) for s in range(batch.num_requests)
-                         if batch.q_start[s + 1] > batch.q_start[s] and batch.positions[batch.q_start[s]] == 0]
-                if fresh:
-                    b.state[fresh] = 0
-        return self.model.forward(ctx, self.bindings)
+        if batch.num_tokens == 0:
+            return self.rt.empty((0, self.spec.vocab_size), torch.float32)
+        self._zero_fresh_state(batch)
+        if self.use_graphs and batch.num_tokens == batch.num_requests:
+            return self._graph_step(batch)
+        return self.model.forward(self._upload(batch), self.bindings)
 
-    def _upload(self, batch: StepBatch) -> StepContext:
-        T, S = batch.num_tokens, batch.num_requests
-        parts = [batch.token_ids, batch.positions, batch.seq_of_token, batch.q_start, batch.seq_lens,
-                 batch.state_slots, batch.logits_rows] + list(batch.slots) + [t.reshape(-1) for t in batch.block_tables]
-        sizes = [p.size for p in parts]
-        flat = np.concatenate([np.ascontiguousarray(p, dtype=np.int32).reshape(-1) for p in parts]) \
-            if sum(sizes) else np.zeros(0, np.int32)
-        dev = torch.from_numpy(flat).to(self.rt.device)
+    def _zero_fresh_state(self, batch: StepBatch) -> None:
+        """State slots of requests that start at position 0 in this step are cleared."""
+        if not any(b.state is not None for b in self.bindings):
+            return
+        fresh = [int(batch.state_slots[s]) for s in range(batch.num_requests)
+                 if batch.q_start[s + 1] > batch.q_start[s] and batch.positions[batch.q_start[s]] == 0]
+        if fresh:
+            for b in self.bindings:
+                if b.state is not None:
+                    b.state[fresh] = 0
+
+    def _context(self, dev: torch.Tensor, sizes: List[int], batch: StepBatch) -> StepContext:
         views, at = [], 0
         for n in sizes:
             views.append(dev[at:at + n])
             at += n
+        T, S = batch.num_tokens, batch.num_requests
         G = len(batch.slots)
-        tables = [views[7 + G + g].view(S, -1) for g in range(G)]
+        tables = [views[N_FIXED + G + g].view(S, -1) for g in range(G)]
         return StepContext(rt=self.rt, num_tokens=T, num_requests=S, token_ids=views[0], positions=views[1],
                            seq_of_token=views[2], q_start=views[3], seq_lens=views[4], state_slots=views[5],
-                           logits_rows=views[6], slots=views[7:7 + G], block_tables=tables, host=batch)
+                           logits_rows=views[6], slots=views[N_FIXED:N_FIXED + G], block_tables=tables, host=batch)
+
+    def _upload(self, batch: StepBatch) -> StepContext:
+        sizes, flat = _pack(batch)
+        return self._context(torch.from_numpy(flat).to(self.rt.device), sizes, batch)
+
+    # ---- graphs for one-token-per-request steps ---------------------------------
+    def _graph_step(self, batch: StepBatch) -> torch.Tensor:
+        S = batch.num_requests
+        longest = int(batch.seq_lens.max())
+        bucket = 1 << max(longest - 1, 0).bit_length()  # context rounded up to a power of two
+        key = (S, bucket)
+        graph = self._graphs.get(key)
+        if graph is None:
+            graph = self._graphs[key] = _DecodeGraph(self, batch, bucket)
+        return graph.run(batch)
 
     # ---- convenience over the cache manager -----------------------------------
     def add_request(self, rid: Hashable) -> None:
@@ -133,3 +171,60 @@ class ModelRunner:
         for rid, tokens, _ in entries:
             self.cache.commit(rid, len(tokens))
         return logits
+
+
+class _DecodeGraph:
+    """One captured step for `S` requests of one token each, contexts up to `bucket`."""
+
+    def __init__(self, runner: ModelRunner, batch: StepBatch, bucket: int):
+        rt = runner.rt
+        S = batch.num_requests
+        all_rows = self._with_all_rows(batch)
+        sizes, flat = _pack(all_rows)
+        self.sizes = sizes
+        self.host = torch.empty(flat.size, dtype=torch.int32).pin_memory()
+        self.host_np = self.host.numpy()
+        self.dev = torch.empty(flat.size, dtype=torch.int32, device=rt.device)
+        self.copied = torch.cuda.Event()
+        self._fill(flat)
+        ctx = runner._context(self.dev, sizes, all_rows)
+        # the attention plan of a one-token-per-request step never changes: tile i = request i, row i, one query
+        tiles = torch.tensor([list(range(S)), list(range(S)), [1] * S], dtype=torch.int32, device=rt.device)
+        ctx.memo["attention_tiles_host"] = (tiles, S, bucket)
+        ctx.host = None  # nothing may plan from host data inside the capture
+        self.ctx = ctx
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            runner.model.forward(ctx, runner.bindings)  # warm-up: library plans, allocator
+            ctx.memo = {"attention_tiles_host": (tiles, S, bucket)}
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph, pool=runner._graph_pool):
+            self.logits = runner.model.forward(ctx, runner.bindings)
+        if runner._graph_pool is None:
+            runner._graph_pool = self.graph.pool()
+
+    @staticmethod
+    def _with_all_rows(batch: StepBatch) -> StepBatch:
+        return StepBatch(batch.token_ids, batch.positions, batch.seq_of_token, batch.q_start, batch.seq_lens,
+                         batch.state_slots, np.arange(batch.num_tokens, dtype=np.int32), batch.slots,
+                         batch.block_tables, batch.request_ids)
+
+    def _fill(self, flat: np.ndarray) -> None:
+        self.copied.synchronize()  # the pinned buffer is free again
+        self.host_np[:] = flat
+        self.dev.copy_(self.host, non_blocking=True)
+        self.copied.record()
+
+    def run(self, batch: StepBatch) -> torch.Tensor:
+        sizes, flat = _pack(self._with_all_rows(batch))
+        if sizes != self.sizes:
+            raise RuntimeError("a captured step was given a batch of another shape")
+        self._fill(flat)
+        self.graph.replay()
+        rows = batch.logits_rows
+        if len(rows) == batch.num_tokens and np.array_equal(rows, np.arange(batch.num_tokens)):
+            return self.logits.clone()
+        return self.logits[torch.from_numpy(rows.astype(np.int64)).to(self.logits.device)]

@@ -21,6 +21,8 @@ from .dense_mlp import stack_rows
 
 
 class PagedAttention(Mixer):
+    graph_safe = True  # the query tiles are planned on the host, but outside a captured step (see query_tiles)
+
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, qkv_bias: bool = True,
                  out_bias: bool = False, window: int = 0, scale: Optional[float] = None,
                  position: Optional[PartSpec] = None, init_std: float = 0.02):
@@ -123,6 +125,7 @@ def query_tiles(ctx, window: int, heads: int):
     tiles_dev, n_tiles, longest = base
     span = min(longest, window + QUERY_TILE + 32) if window > 0 else longest
     n_splits = max(1, min(-(-WAVES_WANTED // max(1, n_tiles * heads)), -(-span // MIN_KEYS_PER_SPLIT), 64))
+    n_splits = 1 << (n_splits.bit_length() - 1)  # a power of two: few distinct values, few captured graphs
     ctx.memo[key] = (tiles_dev, n_splits)
     return ctx.memo[key]
 

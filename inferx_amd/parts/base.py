@@ -55,6 +55,10 @@ class StateNeed:
 
 
 class Part:
+    # True if `forward` only launches work on the current stream (no host reads of device data, no host-side
+    # planning from the batch), so that a step can be captured into a HIP graph
+    graph_safe = False
+
     def param_specs(self) -> List[ParamSpec]:
         return []
 
@@ -89,6 +93,8 @@ class FeedForward(Part):
 
 
 class Block:
+    graph_safe = False
+
     def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
         self.mixer, self.feed_forward = mixer, feed_forward
         self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm

@@ -12,6 +12,8 @@ from .base import Block, register_part
 
 
 class PreNormBlock(Block):
+    graph_safe = True
+
     def forward(self, ctx, h, pending, cache):
         x = self.mixer_norm.forward(ctx, h, pending)
         a = self.mixer.forward(ctx, x, cache)

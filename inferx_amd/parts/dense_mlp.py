@@ -22,6 +22,8 @@ def stack_rows(tensors):
 
 
 class DenseMlp(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, width: int, init_std: float = 0.02):
         self.hidden_size, self.width, self.init_std = int(hidden_size), int(width), float(init_std)
         self.w_gate_up = self.w_down = None

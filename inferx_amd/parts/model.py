@@ -62,6 +62,14 @@ class DecoderModel:
             part.bind(local, rt)
         weights.clear()
 
+    def graph_safe(self) -> bool:
+        """True if every part may run inside a captured HIP graph."""
+        parts = [self.final_norm]
+        for b in self.blocks:
+            parts += [b, b.mixer, b.feed_forward, b.mixer_norm, b.feed_forward_norm]
+            parts.append(getattr(b.mixer, "position", None))
+        return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
+
     # ---- what the cache manager must provide -------------------------------
     def cache_plan(self):
         """Per schedule entry: (CacheNeed or None, StateNeed or None, cache_from)."""

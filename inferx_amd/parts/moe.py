@@ -20,6 +20,8 @@ from .dense_mlp import stack_rows
 
 
 class MoeFeedForward(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, num_experts: int, top_k: int, expert_width: int, shared_width: int = 0,
                  shared_gated: bool = True, renormalize: bool = False, routed_scale: float = 1.0,
                  init_std: float = 0.02):

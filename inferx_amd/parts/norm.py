@@ -12,6 +12,8 @@ from .base import Norm, ParamSpec, register_part
 
 
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, width: int, eps: float):
         self.width, self.eps = int(width), float(eps)
         self.weight = None

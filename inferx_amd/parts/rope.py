@@ -18,6 +18,8 @@ from .base import PositionEncoding, register_part
 
 
 class Rotary(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, theta: float, rotary_dim: int):
         if rotary_dim <= 0 or rotary_dim % 2:
             raise ValueError(f"rotary_dim {rotary_dim} must be positive and even")
