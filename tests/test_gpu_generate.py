@@ -1,0 +1,215 @@
+"""Generation through the entry points: the Python engine, the command line and the replay
+program, against the plain implementation; long decoding; the first tokens of a sequence;
+what happens when pages run out."""
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+import replay_util as ru
+import tiny
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def plain_greedy(cfg, weights, prompt, steps):
+    seq, margins = list(prompt), []
+    for _ in range(steps):
+        logits = pm.forward(cfg, weights, seq)[-1]
+        top2 = torch.topk(logits, 2).values
+        margins.append(float(top2[0] - top2[1]) / float(logits.abs().max()))
+        seq.append(pm.greedy(logits))
+    return seq[len(prompt):], margins
+
+
+def check_greedy(got, want, margins, exact):
+    for i, (g, w, m) in enumerate(zip(got, want, margins)):
+        if g != w:
+            assert not exact and m < 2e-2, f"token {i}: got {g}, plain implementation {w} (margin {m:.2e})"
+            return  # after a near-tie the two continuations legitimately differ
+    assert len(got) == len(want)
+
+
+@pytest.mark.parametrize("name,dtype,lengths,steps", [("A", "float32", (5, 9, 17), 8), ("B", "float32", (7, 23, 40), 12),
+                                                      ("A", "bfloat16", (5, 9, 17), 8), ("B", "bfloat16", (7, 23, 40), 12)])
+def test_greedy_generation_through_the_python_entry_point(tmp_path, name, dtype, lengths, steps):
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIGS[name], 31, str(tmp_path), dtype)
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 40 + n) for n in lengths]
+    # portions of 8 tokens (the second configuration's workload), three requests at a time
+    engine = LLMEngine(str(tmp_path), dtype, max_num_seqs=3, max_model_len=128, max_num_batched_tokens=8,
+                       num_gpu_blocks_override=24)
+    got = engine.generate(prompts, SamplingParams(max_tokens=steps))
+    for p, g in zip(prompts, got):
+        want, margins = plain_greedy(cfg, weights, p, steps)
+        check_greedy(g, want, margins, exact=dtype == "float32")
+    assert engine.stats.tokens_out == steps * len(prompts)
+    assert all(pool.used_pages == 0 for pool in engine.runner.cache.pools)
+
+
+def test_temperature_sampling_is_seeded_and_in_the_support(tmp_path):
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_B, 32, str(tmp_path), "float32", std_scale=6.0)  # peaked enough for small supports
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 50 + n) for n in (7, 23, 40)]
+    params = SamplingParams(max_tokens=12, temperature=0.7, top_k=6, seed=99)
+    runs = []
+    for _ in range(2):
+        engine = LLMEngine(str(tmp_path), "float32", max_num_seqs=3, max_model_len=128, max_num_batched_tokens=8,
+                           num_gpu_blocks_override=24)
+        runs.append(engine.generate(prompts, params))
+    assert runs[0] == runs[1]  # a pinned seed reproduces
+    for p, out in zip(prompts, runs[0]):
+        seq = list(p)
+        for tok in out:
+            logits = pm.forward(cfg, weights, seq)[-1]
+            assert tok in pm.sampling_support(logits, 0.7, top_k=6)
+            seq.append(tok)
+    other = LLMEngine(str(tmp_path), "float32", max_num_seqs=3, max_model_len=128, num_gpu_blocks_override=24)
+    assert other.generate(prompts, SamplingParams(max_tokens=12, temperature=0.7, top_k=6, seed=100)) != runs[0]
+
+
+def test_preempted_generation_equals_unpreempted(tmp_path):
+    """So few pages that running requests are preempted and recomputed: same tokens (reference:
+    tests/unit/scheduler_test.cc:742-812)."""
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_A, 33, str(tmp_path), "float32")
+    cfg, _ = tiny.read_folder(str(tmp_path))
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 60 + n) for n in (20, 25, 30)]
+    params = [SamplingParams(max_tokens=40, temperature=0.8, seed=i) for i in range(3)]
+    roomy = LLMEngine(str(tmp_path), "float32", max_num_seqs=3, max_model_len=128, num_gpu_blocks_override=24)
+    tight = LLMEngine(str(tmp_path), "float32", max_num_seqs=3, max_model_len=128, num_gpu_blocks_override=9)
+    a, b = roomy.generate(prompts, params), tight.generate(prompts, params)
+    assert roomy.stats.preemptions == 0 and tight.stats.preemptions > 0
+    assert a == b
+
+
+def test_stop_token_and_context_limit(tmp_path):
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_A, 34, str(tmp_path), "float32")
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    prompt = tiny.random_tokens(6, cfg["vocab_size"], 70)
+    want, _ = plain_greedy(cfg, weights, prompt, 6)
+    engine = LLMEngine(str(tmp_path), "float32", max_num_seqs=2, max_model_len=32, num_gpu_blocks_override=8)
+    out = engine.generate([prompt], SamplingParams(max_tokens=20, stop_tokens=[want[3]]), with_reasons=True)
+    first_stop = want.index(want[3])
+    assert out[0] == (want[:first_stop + 1], "stop_token")
+    out = engine.generate([prompt], SamplingParams(max_tokens=100), with_reasons=True)
+    assert out[0][1] == "context_limit" and len(out[0][0]) == 32 - 6 + 1
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_and_first_tokens(tmp_path, dtype):
+    """300 tokens one by one after a two-token start (graphs, page edges, the window), and every
+    first position of a sequence, against the plain implementation."""
+    from inferx_amd.engine.runner import ModelRunner
+    tiny.make_folder(tiny.CONFIG_B, 35, str(tmp_path), dtype)
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    toks = tiny.random_tokens(250, cfg["vocab_size"], 80)
+    expected = {"r": pm.forward(cfg, weights, toks)}
+    runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=16, num_pages=16, max_requests=2,
+                                        max_seq_len=256)
+    steps = [{"entries": [("r", toks[:2], [0, 1])], "end": []}]
+    steps += [{"entries": [("r", toks[i:i + 1], [0])], "end": []} for i in range(2, 250)]
+    got = ru.replay(runner, steps)
+    ru.compare(got, expected, ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL, f"long decode {dtype}")
+    assert runner.use_graphs and len(runner._graphs) >= 2  # captured steps were replayed, over several buckets
+
+
+def test_far_key_and_window_edge_show_in_the_logits(tmp_path):
+    """Random weights attend almost uniformly and would hide a lost key.  With attention weights scaled up the
+    scores are peaked, so a key lost at a page edge, a split boundary or the window's edge changes the logits."""
+    from inferx_amd.engine.runner import ModelRunner
+    raw = dict(tiny.CONFIG_B, max_position_embeddings=512)
+    tiny.make_folder(raw, 36, str(tmp_path), "float32")
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    from safetensors.torch import save_file
+    for k in weights:
+        if "q_proj.weight" in k or "k_proj.weight" in k:
+            weights[k] = weights[k] * 12.0
+    save_file(weights, os.path.join(str(tmp_path), "model.safetensors"))
+    toks = tiny.random_tokens(300, cfg["vocab_size"], 81)
+    whole = pm.forward(cfg, weights, toks)
+    # the plain implementation itself is sensitive here: dropping the oldest key of the window changes the result
+    assert float((pm.forward(dict(cfg, sliding_window=15), weights, toks)[-1] - whole[-1]).abs().max()) > \
+        1e-3 * float(whole.abs().max())
+    runner = ModelRunner.from_directory(str(tmp_path), dtype="float32", page_size=16, num_pages=24, max_requests=2,
+                                        max_seq_len=384)
+    prompts = {"r": toks}
+    for steps in (ru.whole(prompts), ru.chunked(prompts, sizes=(33, 2, 64, 17, 100)), ru.tail_decoded(prompts, 40)):
+        ru.compare(ru.replay(runner, steps), {"r": whole}, ru.FP32_TOL, "peaked attention")
+
+
+def test_command_line(tmp_path):
+    tiny.make_folder(tiny.CONFIG_A, 37, str(tmp_path), "float32")
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    prompt = tiny.random_tokens(9, cfg["vocab_size"], 90)
+    want, _ = plain_greedy(cfg, weights, prompt, 5)
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "inferx-generate"), "--model", str(tmp_path), "--dtype", "float32",
+           "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "5", "--max-model-len", "64",
+           "--num-gpu-blocks-override", "8", "--max-num-seqs", "2"]
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    rec = json.loads(out.stdout.strip().splitlines()[-1])
+    assert rec["output_token_ids"] == want and rec["finish_reason"] == "max_tokens"
+    bad = subprocess.run(cmd[:2] + ["--no-such-flag"], capture_output=True, text=True, timeout=60)
+    assert bad.returncode == 2
+    missing = subprocess.run(cmd[:2] + ["--model", os.path.join(str(tmp_path), "nothing"), "--prompt-ids", "1"],
+                             capture_output=True, text=True, timeout=120)
+    assert missing.returncode == 1 and "config.json" in missing.stderr
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(tmp_path, dtype):
+    """bin/trace_run as a user calls it: steps on standard input, logits in files, `done <step>` per step."""
+    model = tmp_path / "model"
+    out_dir = tmp_path / "out"
+    tiny.make_folder(tiny.CONFIG_B, 38, str(model), dtype)
+    cfg, weights = tiny.read_folder(str(model))
+    prompts = {f"r{i}": tiny.random_tokens(n, cfg["vocab_size"], 95 + i) for i, n in enumerate((40, 70, 23, 55, 64))}
+    steps = ru.mixed(prompts, seed=9, max_live=4, max_tokens=256)
+    lines, wanted = [], []
+    fed = {rid: 0 for rid in prompts}
+    for i, st in enumerate(steps):
+        entries = []
+        for rid, toks, want in st["entries"]:
+            want = want if (i + len(toks)) % 3 else want[::2]  # not every place is asked for
+            entries.append({"id": rid, "tokens": toks, "want": want})
+            wanted.append((i, [(rid, fed[rid] + w) for w in want]))
+            fed[rid] += len(toks)
+        lines.append(json.dumps({"step": i, "entries": entries, "end": st["end"]}))
+    proc = subprocess.run([os.path.join(ROOT, "bin", "trace_run"), "--model", str(model), "--dtype", dtype, "--out",
+                           str(out_dir), "--max-tokens", "256"], input="\n".join(lines) + "\n", capture_output=True,
+                          text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert proc.stdout.split() == [w for i in range(len(steps)) for w in ("done", str(i))]
+    got = {}
+    by_step = {}
+    for i, keys in wanted:
+        by_step.setdefault(i, []).extend(keys)
+    for i, keys in by_step.items():
+        path = out_dir / f"{i}.f32"
+        if not keys:
+            assert not path.exists()
+            continue
+        rows = np.fromfile(path, dtype="<f4").reshape(len(keys), cfg["vocab_size"])
+        for key, row in zip(keys, rows):
+            got[key] = torch.from_numpy(row.copy())
+    expected = ru.expected_logits(cfg, weights, prompts)
+    tol = ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL
+    scale = max(float(e.abs().max()) for e in expected.values())
+    assert len(got) > 100
+    for (rid, pos), row in got.items():
+        err = float((row.double() - expected[rid][pos]).abs().max()) / scale
+        assert err <= tol, f"request {rid} position {pos}: error {err:.2e}"

@@ -1,0 +1,199 @@
+"""Embedding, norm, SwiGLU product, rotary table, bias + rotation + cache append, greedy and
+temperature sampling, penalties: each kernel alone against a PyTorch reference."""
+import math
+
+import pytest
+import torch
+
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def rnd(*shape, seed=0, dtype=torch.float32, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype).to(DEV)
+
+
+def rel_err(got, want):
+    want = want.double().cpu()
+    return float((got.double().cpu() - want).abs().max()) / max(float(want.abs().max()), 1e-30)
+
+
+def tol(dtype):
+    return 2e-6 if dtype == torch.float32 else 8e-3
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(dtype):
+    from inferx_amd import ops
+    table = rnd(301, 72, dtype=dtype)
+    ids = torch.tensor([0, 300, 7, 7, 150], dtype=torch.int32, device=DEV)
+    h = torch.empty(5, 72, device=DEV)
+    ops.embed(h, table, ids)
+    assert torch.equal(h.cpu(), table.float().cpu()[ids.long().cpu()])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("wdtype", DTYPES)
+@pytest.mark.parametrize("T,H,eps", [(5, 72, 1e-5), (3, 2048, 1e-6), (2, 5000, 1e-6)])
+def test_add_rmsnorm(dtype, wdtype, T, H, eps):
+    from inferx_amd import ops
+    h0, delta, w = rnd(T, H), rnd(T, H, seed=1, dtype=dtype), rnd(H, seed=2, dtype=wdtype)
+    h = h0.clone()
+    out = torch.empty(T, H, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(h, delta, w, out, eps)
+    v = h0.double().cpu() + delta.double().cpu()
+    assert rel_err(h, v) < 1e-6  # the residual stream carries the sum, in float32
+    assert rel_err(out, pm.rms_norm(v, w.double().cpu(), eps)) < tol(dtype)
+    # no delta; and picked rows (a row may be asked for twice; h is then left alone)
+    h = h0.clone()
+    ops.add_rmsnorm(h, None, w, out, eps)
+    assert torch.equal(h, h0) and rel_err(out, pm.rms_norm(h0.double().cpu(), w.double().cpu(), eps)) < tol(dtype)
+    rows = torch.tensor([T - 1, 0, T - 1], dtype=torch.int32, device=DEV)
+    picked = torch.empty(3, H, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(h, delta, w, picked, eps, rows)
+    assert torch.equal(h, h0)
+    assert rel_err(picked, pm.rms_norm(v, w.double().cpu(), eps)[rows.long().cpu()]) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul(dtype):
+    from inferx_amd import ops
+    gu = rnd(7, 2 * 104, dtype=dtype, scale=3.0)
+    out = torch.empty(7, 104, dtype=dtype, device=DEV)
+    ops.silu_mul(gu, out)
+    g, u = gu.double().cpu()[:, :104], gu.double().cpu()[:, 104:]
+    assert rel_err(out, pm.silu(g) * u) < tol(dtype)
+
+
+@pytest.mark.parametrize("theta,d", [(10000.0, 16), (1e6, 128), (50000.0, 48)])
+def test_rope_table(theta, d):
+    from inferx_amd import ops
+    from inferx_amd.parts.rope import Rotary
+    pos = torch.tensor([0, 1, 2, 17, 255, 4095, 32767], dtype=torch.int32, device=DEV)
+    inv = Rotary(theta, d).frequencies().to(DEV)
+    assert torch.equal(inv.cpu().double(), pm.rope_frequencies(theta, d))
+    table = torch.empty(len(pos), d // 2, 2, device=DEV)
+    ops.rope_table(table, pos, inv)
+    angle = (pos.cpu().float()[:, None] * inv.cpu()[None, :]).double()
+    assert float((table[..., 0].cpu().double() - torch.cos(angle)).abs().max()) < 2e-6
+    assert float((table[..., 1].cpu().double() - torch.sin(angle)).abs().max()) < 2e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv,d,page,bias", [(4, 2, 16, 16, True), (3, 1, 32, 16, True), (6, 3, 48, 32, False),
+                                                  (16, 16, 128, 16, True)])
+def test_qkv_rope_append(dtype, heads, kv, d, page, bias):
+    from inferx_amd import ops
+    from inferx_amd.parts.rope import Rotary
+    T, pages, theta = 9, 5, 10000.0
+    width = (heads + 2 * kv) * d
+    qkv = rnd(T, width, dtype=dtype)
+    b = rnd(width, seed=1, dtype=dtype) if bias else None
+    pos = torch.tensor([3, 4, 5, 6, 0, 1, 40, 41, 42], dtype=torch.int32, device=DEV)
+    slots = torch.tensor([page * 2 + 3, page * 2 + 4, page * 2 + 5, page * 2 + 6, 0, 1, page * 4 + 8, page * 4 + 9,
+                          page * 1 + 0], dtype=torch.int32, device=DEV)
+    table = torch.empty(T, d // 2, 2, device=DEV)
+    ops.rope_table(table, pos, Rotary(theta, d).frequencies().to(DEV))
+    q = torch.empty(T, heads, d, dtype=dtype, device=DEV)
+    kc = torch.zeros(pages, kv, page, d, dtype=dtype, device=DEV)
+    vc = torch.zeros(pages, kv, d, page, dtype=dtype, device=DEV)
+    ops.qkv_rope_append(qkv, b, table, slots, q, kc, vc, heads, kv, d)
+    x = qkv.double().cpu() + (b.double().cpu() if bias else 0)
+    wq = pm.apply_rope(x[:, :heads * d].view(T, heads, d), pos.cpu(), theta)
+    wk = pm.apply_rope(x[:, heads * d:(heads + kv) * d].view(T, kv, d), pos.cpu(), theta)
+    wv = x[:, (heads + kv) * d:].view(T, kv, d)
+    assert rel_err(q, wq) < tol(dtype)
+    for t in range(T):
+        pg, off = int(slots[t]) // page, int(slots[t]) % page
+        assert rel_err(kc[pg, :, off, :], wk[t]) < tol(dtype)
+        assert rel_err(vc[pg, :, :, off], wv[t]) < tol(dtype)
+    written = torch.zeros(pages, page, dtype=torch.bool)
+    for t in range(T):
+        written[int(slots[t]) // page, int(slots[t]) % page] = True
+    assert float(kc.float().abs().sum(dim=(1, 3)).cpu()[~written].sum()) == 0  # nothing else was touched
+    # no rotation table: q and k pass through; no caches: only q is written
+    q2 = torch.empty_like(q)
+    ops.qkv_rope_append(qkv, b, None, None, q2, None, None, heads, kv, d)
+    assert rel_err(q2, x[:, :heads * d].view(T, heads, d)) < tol(dtype)
+
+
+def test_argmax_first_maximum():
+    # reference vector: tests/unit/host_sampling_test.cc:12-17 ({1, 4, 2} -> 1); ties go to the lowest index
+    from inferx_amd import ops
+    logits = torch.tensor([[1.0, 4.0, 2.0], [3.0, 3.0, 1.0], [-1.0, -5.0, -1.0]], device=DEV)
+    out = torch.empty(3, dtype=torch.int32, device=DEV)
+    ops.argmax(logits, out)
+    assert out.tolist() == [1, 0, 0]
+    big = rnd(4, 151936, seed=3)
+    big[2, 77777] = 50.0
+    big[2, 150000] = 50.0
+    out = torch.empty(4, dtype=torch.int32, device=DEV)
+    ops.argmax(big, out)
+    assert out.tolist() == [int(r.argmax()) for r in big.cpu()[:2]] + [77777, int(big[3].argmax())]
+
+
+def draw(logits, temperature, top_k=0, top_p=1.0, min_p=0.0, seed=0, counter=0):
+    from inferx_amd import ops
+    R = logits.shape[0]
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    f = lambda v, dt: torch.full((R,), v, dtype=dt, device=DEV)
+    ops.sample(logits, out, f(temperature, torch.float32), f(top_p, torch.float32), f(top_k, torch.int32),
+               f(min_p, torch.float32), f(seed, torch.int64), f(counter, torch.int64))
+    return out.tolist()
+
+
+def test_deterministic_settings_equal_argmax():
+    # reference: tests/kernel/sampling_test.cc:213-364 (t = 0, top_k = 1, min_p = 1, a dominant nucleus)
+    logits = rnd(6, 1000, seed=5, scale=2.0)
+    want = logits.argmax(-1).tolist()
+    assert draw(logits, 0.0) == want
+    assert draw(logits, 0.7, top_k=1) == want
+    assert draw(logits, 0.7, min_p=1.0) == want
+    peaked = logits.clone()
+    peaked[torch.arange(6), torch.tensor(want)] += 30.0
+    assert draw(peaked, 1.0, top_p=0.5) == want
+
+
+@pytest.mark.parametrize("settings", [dict(top_k=5), dict(top_p=0.6), dict(min_p=0.2), dict(top_k=8, top_p=0.8),
+                                      dict()])
+def test_random_settings_stay_in_the_support_and_repeat(settings):
+    # reference: sampling_test.cc:265-291, 366-438; tests/unit/host_sampling_test.cc:34-53
+    logits = rnd(1, 300, seed=6, scale=2.5)
+    support = set(pm.sampling_support(logits[0].cpu(), 0.8, **settings))
+    seen = set()
+    for seed in range(40):
+        a = draw(logits, 0.8, seed=seed, counter=3, **settings)
+        assert a == draw(logits, 0.8, seed=seed, counter=3, **settings)  # a pinned seed reproduces
+        assert a[0] in support
+        seen.add(a[0])
+    assert len(seen) > 1 or len(support) == 1
+    assert len({draw(logits, 0.8, seed=1, counter=c, **settings)[0] for c in range(40)}) > 1 or len(support) == 1
+
+
+def test_sampling_follows_the_distribution():
+    logits = torch.tensor([[2.0, 1.0, 0.0, -1.0]], device=DEV)
+    p = torch.softmax(logits[0].cpu().double() / 0.9, -1)
+    n = 4000
+    counts = torch.zeros(4)
+    for seed in range(n):
+        counts[draw(logits, 0.9, seed=seed)[0]] += 1
+    assert float((counts / n - p).abs().max()) < 0.03
+
+
+def test_penalties_and_masks():
+    # reference vector: tests/unit/host_sampling_test.cc:19-32 ({5, 4, 3}, presence 3 on id 0, mask on id 1 -> 2)
+    from inferx_amd import ops
+    logits = torch.tensor([[5.0, 4.0, 3.0], [2.0, -2.0, 1.0]], device=DEV)
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    f32 = lambda v: torch.tensor(v, dtype=torch.float32, device=DEV)
+    ops.apply_penalties(logits, i32([0, 1, 3]), i32([0, 0, 1]), i32([1, 2, 1]), f32([3.0, 0.5]), f32([0.0, 0.25]),
+                        f32([1.0, 2.0]), i32([0, 1, 1]), i32([1]))
+    want = [[5.0 - 3.0, -math.inf, 3.0], [2.0 / 2 - 0.5 - 0.5, -2.0 * 2 - 0.5 - 0.25, 1.0]]
+    assert logits.cpu().tolist() == want
+    out = torch.empty(2, dtype=torch.int32, device=DEV)
+    ops.argmax(logits, out)
+    assert out.tolist()[0] == 2

@@ -1,0 +1,176 @@
+"""Each part of a layer alone (norm, attention with its position encoding, dense and
+expert feed-forward, the block) against the plain implementation's function for it."""
+import numpy as np
+import pytest
+import torch
+
+import plain_model as pm
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+PARAMS = [("float32", 2e-5), ("bfloat16", 2e-2)]
+
+
+def make_ctx(rt, q_lens, seq_lens, page_size, pages, groups=1):
+    """A step context for requests with the given new and total lengths (pages handed out in order)."""
+    from inferx_amd.cache.manager import CacheManager, GroupLayout
+    from inferx_amd.engine.batch import build_step_batch
+    from inferx_amd.engine.runner import _pack
+    from inferx_amd.engine.runtime import StepContext
+    cache = CacheManager([GroupLayout(0)] * groups, [pages] * groups, page_size, len(q_lens), pages * page_size)
+    entries = []
+    for i, (n, L) in enumerate(zip(q_lens, seq_lens)):
+        cache.add(i)
+        if L > n:
+            cache.reserve(i, L - n)
+            cache.commit(i, L - n)
+        entries.append((i, [0] * n, list(range(n))))
+    batch = build_step_batch(cache, entries)
+    sizes, flat = _pack(batch)
+    dev = torch.from_numpy(flat).to(DEV)
+    views, at = [], 0
+    for n in sizes:
+        views.append(dev[at:at + n])
+        at += n
+    S, G = len(q_lens), groups
+    return StepContext(rt=rt, num_tokens=batch.num_tokens, num_requests=S, token_ids=views[0], positions=views[1],
+                       seq_of_token=views[2], q_start=views[3], seq_lens=views[4], state_slots=views[5],
+                       logits_rows=views[6], slots=views[7:7 + G],
+                       block_tables=[views[7 + G + g].view(S, -1) for g in range(G)], host=batch), batch
+
+
+def tensors_for(part, rt, seed=0, std=None):
+    out = {}
+    for i, p in enumerate(part.param_specs()):
+        g = torch.Generator().manual_seed(seed * 1000 + i)
+        t = torch.ones(p.shape) if p.init == "ones" else torch.randn(p.shape, generator=g) * (std or p.std)
+        out[p.name] = t.to(rt.dtype)
+    return out
+
+
+def err(got, want):
+    want = want.double().cpu()
+    return float((got.double().cpu() - want).abs().max()) / float(want.abs().max())
+
+
+@pytest.mark.parametrize("dtype,tol", PARAMS)
+def test_rmsnorm_part(dtype, tol):
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_part
+    from inferx_amd.config import PartSpec
+    rt = Runtime(dtype)
+    part = build_part("norm", PartSpec("rmsnorm", {"width": 72, "eps": 1e-5}))
+    w = {"weight": (torch.randn(72, generator=torch.Generator().manual_seed(1)) * 0.5 + 1).to(rt.dtype)}
+    part.bind({k: v.to(DEV) for k, v in w.items()}, rt)
+    ctx, _ = make_ctx(rt, [5], [5], 16, 4)
+    h = torch.randn(5, 72, generator=torch.Generator().manual_seed(2)).to(DEV)
+    delta = torch.randn(5, 72, generator=torch.Generator().manual_seed(3)).to(rt.dtype).to(DEV)
+    want_h = h.double().cpu() + delta.double().cpu()
+    out = part.forward(ctx, h, delta)
+    assert err(out, pm.rms_norm(want_h, w["weight"].double(), 1e-5)) < tol
+    assert err(h, want_h) < 1e-6
+
+
+@pytest.mark.parametrize("dtype,tol", PARAMS)
+@pytest.mark.parametrize("heads,kv,d,window,bias", [(4, 2, 16, 0, True), (3, 1, 32, 7, True), (6, 3, 48, 0, False)])
+def test_attention_part_whole_and_in_two_steps(dtype, tol, heads, kv, d, window, bias):
+    from inferx_amd.config import PartSpec
+    from inferx_amd.engine.runtime import CacheBinding, Runtime
+    from inferx_amd.parts import build_part
+    rt = Runtime(dtype)
+    H, theta, T = 40, 10000.0, 37
+    spec = PartSpec("attention", {"hidden_size": H, "num_heads": heads, "num_kv_heads": kv, "head_dim": d,
+                                  "qkv_bias": bias, "window": window,
+                                  "position": PartSpec("rope", {"theta": theta, "rotary_dim": d}), "init_std": 0.2})
+    part = build_part("mixer", spec)
+    w = tensors_for(part, rt, seed=4)
+    part.bind({k: v.to(DEV) for k, v in w.items()}, rt)
+    x = (torch.randn(T, H, generator=torch.Generator().manual_seed(5))).to(rt.dtype)
+    # plain: projections, bias, rotation, attention, output projection (tests/plain_model.py forward())
+    wd = {k: v.double() for k, v in w.items()}
+    xd = x.double()
+    q, k, v = xd @ wd["q_proj.weight"].T, xd @ wd["k_proj.weight"].T, xd @ wd["v_proj.weight"].T
+    if bias:
+        q, k, v = q + wd["q_proj.bias"], k + wd["k_proj.bias"], v + wd["v_proj.bias"]
+    pos = torch.arange(T)
+    att = pm.attention(pm.apply_rope(q.view(T, heads, d), pos, theta), pm.apply_rope(k.view(T, kv, d), pos, theta),
+                       v.view(T, kv, d), pos, d ** -0.5, window)
+    want = att.reshape(T, heads * d) @ wd["o_proj.weight"].T
+
+    def run(splits):
+        pages, page = 4, 16
+        cache = CacheBinding(group=0, k=torch.zeros(pages, kv, page, d, dtype=rt.dtype, device=DEV),
+                             v=torch.zeros(pages, kv, d, page, dtype=rt.dtype, device=DEV))
+        outs, done = [], 0
+        for n in splits:
+            ctx, _ = make_ctx(rt, [n], [done + n], page, pages)
+            outs.append(part.forward(ctx, x[done:done + n].to(DEV), cache))
+            done += n
+        return torch.cat(outs)
+
+    assert err(run([T]), want) < tol
+    assert err(run([20, 2, 14, 1]), want) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", PARAMS)
+def test_dense_mlp_part(dtype, tol):
+    from inferx_amd.config import PartSpec
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_part
+    rt = Runtime(dtype)
+    part = build_part("feed_forward", PartSpec("dense_mlp", {"hidden_size": 72, "width": 104, "init_std": 0.2}))
+    w = tensors_for(part, rt, seed=6)
+    part.bind({k: v.to(DEV) for k, v in w.items()}, rt)
+    ctx, _ = make_ctx(rt, [9], [9], 16, 4)
+    x = torch.randn(9, 72, generator=torch.Generator().manual_seed(7)).to(rt.dtype)
+    want = pm.gated_mlp(x.double(), w["gate_proj.weight"].double(), w["up_proj.weight"].double(),
+                        w["down_proj.weight"].double())
+    assert err(part.forward(ctx, x.to(DEV)), want) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", PARAMS)
+@pytest.mark.parametrize("H,E,k,mi,si,renorm,gated", [(64, 4, 2, 32, 64, False, True), (96, 8, 3, 48, 80, True, True),
+                                                      (72, 5, 1, 40, 0, False, True), (64, 6, 6, 32, 48, True, False),
+                                                      (64, 1, 1, 32, 0, False, True)])
+def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated):
+    from inferx_amd.config import PartSpec
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_part
+    rt = Runtime(dtype)
+    part = build_part("feed_forward", PartSpec("moe", {
+        "hidden_size": H, "num_experts": E, "top_k": k, "expert_width": mi, "shared_width": si,
+        "shared_gated": gated, "renormalize": renorm, "init_std": 0.15}))
+    w = tensors_for(part, rt, seed=8)
+    part.bind({n: v.to(DEV) for n, v in w.items()}, rt)
+    T = 29
+    ctx, _ = make_ctx(rt, [T], [T], 16, 4)
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(9)).to(rt.dtype)
+    wd = {"m." + n: v.double() for n, v in w.items()}
+    if si and not gated:  # an ungated shared expert adds exactly its output: sigmoid(+inf) = 1
+        wd["m.shared_expert_gate.weight"] = torch.full((1, H), 1e4, dtype=torch.float64) * torch.sign(x.double().sum(0))
+        want = pm.moe_block(x.double(), {n: v for n, v in wd.items() if "shared" not in n}, "m.", E, k, renorm, 0) + \
+            pm.gated_mlp(x.double(), wd["m.shared_expert.gate_proj.weight"], wd["m.shared_expert.up_proj.weight"],
+                         wd["m.shared_expert.down_proj.weight"])
+    else:
+        want = pm.moe_block(x.double(), wd, "m.", E, k, renorm, si)
+    got = part.forward(ctx, x.to(DEV))
+    assert err(got, want) < tol
+    # the routing itself, exactly (float32 scores): experts and weights per slot
+    topk_w, topk_e, _ = part.route(ctx, x.to(DEV))
+    want_w, want_e = pm.route(x.double(), wd["m.gate.weight"], k, renorm)
+    assert torch.equal(topk_e.cpu().long(), want_e)
+    assert err(topk_w, want_w) < 1e-5
+    # repeat runs are bitwise equal (reference: tests/kernel/moe_test.cc:972-1046)
+    again = part.forward(ctx, x.to(DEV))
+    assert torch.equal(got.view(torch.int16 if dtype == "bfloat16" else torch.int32),
+                       again.view(torch.int16 if dtype == "bfloat16" else torch.int32))
+
+
+def test_registry_errors():
+    from inferx_amd.config import PartSpec
+    from inferx_amd.parts import build_part
+    with pytest.raises(KeyError, match="no mixer registered as 'nonesuch'"):
+        build_part("mixer", PartSpec("nonesuch"))
+    with pytest.raises(ValueError, match="rotary_dim must equal head_dim"):
+        build_part("mixer", PartSpec("attention", {"hidden_size": 32, "num_heads": 2, "num_kv_heads": 2, "head_dim": 16,
+                                                   "position": PartSpec("rope", {"theta": 1e4, "rotary_dim": 8})}))

@@ -1,0 +1,177 @@
+"""Generality of the parts: a toy mixer that keeps a state of its own per request, defined
+HERE, is registered, built into a model beside attention layers, loaded from a folder and
+stepped (whole, in portions, mixed with another request) without any change to the
+framework's files.  Also a layer order that names a layer twice and lets an execution
+read another one's cache."""
+import json
+import os
+
+import pytest
+import torch
+
+import plain_model as pm
+import replay_util as ru
+import tiny
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ---- the toy mixer: a leaky running sum over the request's tokens -----------------------------
+#   s_t = decay * s_{t-1} + W_in x_t ;  y_t = W_out s_t          (s carried across steps in a state slot)
+def define_toy():
+    from inferx_amd.config import ModelSpec, PartSpec, ScheduleEntry, register_architecture
+    from inferx_amd.config.spec import LayerSpec
+    from inferx_amd.parts import Mixer, ParamSpec, StateNeed, register_part
+
+    class RunningSumMixer(Mixer):
+        def __init__(self, hidden_size, state_size, decay):
+            self.hidden_size, self.state_size, self.decay = hidden_size, state_size, decay
+
+        def state_need(self):
+            return StateNeed((self.state_size,))
+
+        def param_specs(self):
+            return [ParamSpec("in.weight", (self.state_size, self.hidden_size), std=0.3),
+                    ParamSpec("out.weight", (self.hidden_size, self.state_size), std=0.3)]
+
+        def bind(self, tensors, rt):
+            self.w_in, self.w_out = tensors["in.weight"].float(), tensors["out.weight"].float()
+
+        def forward(self, ctx, x, cache):
+            batch = ctx.host  # host arrays of the step: which rows belong to which request, and its state slot
+            u = x.float() @ self.w_in.T
+            s_all = torch.empty_like(u)
+            for r in range(batch.num_requests):
+                b, e, slot = int(batch.q_start[r]), int(batch.q_start[r + 1]), int(batch.state_slots[r])
+                s = cache.state[slot]
+                for t in range(b, e):  # tokens of a request in order
+                    s = self.decay * s + u[t]
+                    s_all[t] = s
+                cache.state[slot] = s
+            return (s_all @ self.w_out.T).to(x.dtype)
+
+    register_part("mixer", "toy_running_sum", RunningSumMixer)
+
+    class ToyConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def validate(self):
+            pass
+
+        def model_spec(self):
+            r = self.raw
+            H = r["hidden_size"]
+            norm = lambda p: PartSpec("rmsnorm", {"width": H, "eps": r["eps"]}, prefix=p)
+            layers = []
+            for l, kind in enumerate(r["mixers"]):
+                p = f"layers.{l}."
+                if kind == "toy":
+                    mixer = PartSpec("toy_running_sum", {"hidden_size": H, "state_size": r["state_size"],
+                                                         "decay": r["decay"]}, prefix=p + "mix.")
+                else:
+                    mixer = PartSpec("attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
+                                                   "qkv_bias": False, "init_std": 0.2,
+                                                   "position": PartSpec("rope", {"theta": 1e4, "rotary_dim": 16})},
+                                     prefix=p + "attn.")
+                ffn = PartSpec("dense_mlp", {"hidden_size": H, "width": r["width"], "init_std": 0.2}, prefix=p + "mlp.")
+                layers.append(LayerSpec("prenorm", mixer, ffn, norm(p + "norm1."), norm(p + "norm2.")))
+            return ModelSpec("ToyStateForCausalLM", H, r["vocab_size"], 0, layers,
+                             [ScheduleEntry(l) for l in range(len(layers))], "embed.weight", norm("final_norm."),
+                             None, init_std=0.5)
+
+    register_architecture("ToyStateForCausalLM", ToyConfig)
+    return ToyConfig
+
+
+TOY = {"architectures": ["ToyStateForCausalLM"], "hidden_size": 24, "state_size": 10, "decay": 0.8, "eps": 1e-5,
+       "width": 40, "vocab_size": 50, "mixers": ["toy", "attention", "toy"]}
+
+
+def toy_reference(w, tokens):
+    """The toy model, whole sequence, float64."""
+    w = {k: v.double() for k, v in w.items()}
+    T = len(tokens)
+    h = w["embed.weight"][torch.tensor(tokens)]
+    pos = torch.arange(T)
+    for l, kind in enumerate(TOY["mixers"]):
+        p = f"layers.{l}."
+        x = pm.rms_norm(h, w[p + "norm1.weight"], TOY["eps"])
+        if kind == "toy":
+            u = x @ w[p + "mix.in.weight"].T
+            s, rows = torch.zeros(TOY["state_size"], dtype=torch.float64), []
+            for t in range(T):
+                s = TOY["decay"] * s + u[t]
+                rows.append(s)
+            a = torch.stack(rows) @ w[p + "mix.out.weight"].T
+        else:
+            q = pm.apply_rope((x @ w[p + "attn.q_proj.weight"].T).view(T, 2, 16), pos, 1e4)
+            k = pm.apply_rope((x @ w[p + "attn.k_proj.weight"].T).view(T, 1, 16), pos, 1e4)
+            v = (x @ w[p + "attn.v_proj.weight"].T).view(T, 1, 16)
+            a = pm.attention(q, k, v, pos, 0.25).reshape(T, 32) @ w[p + "attn.o_proj.weight"].T
+        h = h + a
+        x = pm.rms_norm(h, w[p + "norm2.weight"], TOY["eps"])
+        h = h + pm.gated_mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return pm.rms_norm(h, w["final_norm.weight"], TOY["eps"]) @ w["embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", ru.FP32_TOL), ("bfloat16", ru.BF16_TOL)])
+def test_a_mixer_with_state_of_its_own(tmp_path, dtype, tol):
+    ToyConfig = define_toy()
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.parts import build_model
+    from inferx_amd.weights import random_tensors, write_safetensors
+    model = build_model(ToyConfig(TOY).model_spec())
+    assert [type(b.mixer).__name__ for b in model.blocks] == ["RunningSumMixer", "PagedAttention", "RunningSumMixer"]
+    weights = random_tensors(model, 3, dtype)
+    write_safetensors(os.path.join(str(tmp_path), "model.safetensors"), weights)
+    with open(os.path.join(str(tmp_path), "config.json"), "w") as f:
+        json.dump(TOY, f)
+    prompts = {"a": tiny.random_tokens(45, 50, 1), "b": tiny.random_tokens(20, 50, 2), "c": tiny.random_tokens(33, 50, 3)}
+    expected = {rid: toy_reference(weights, toks) for rid, toks in prompts.items()}
+    for name, steps in [("whole", ru.whole(prompts)), ("tail", ru.tail_decoded(prompts, 8)),
+                        ("chunked", ru.chunked(prompts)), ("mixed", ru.mixed(prompts, seed=2, max_live=2))]:
+        runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=16, num_pages=8, max_requests=2,
+                                            max_seq_len=128)
+        assert not runner.use_graphs  # the toy mixer plans on the host: it does not claim to be graph-safe
+        assert sum(b.state is not None for b in runner.bindings) == 2 and len(runner.kv) == 1
+        got = ru.replay(runner, steps)
+        ru.compare(got, expected, tol, f"toy {name} {dtype}")
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", ru.FP32_TOL), ("bfloat16", ru.BF16_TOL)])
+def test_layer_order_is_data(tmp_path, dtype, tol):
+    """Layer 1 runs twice (shared weights, caches of its own) and the last execution reads the cache of the first."""
+    from inferx_amd.config import ScheduleEntry, config_from_dict
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_model
+    from inferx_amd.weights import load_weights
+    import dataclasses
+    tiny.make_folder(tiny.CONFIG_A, 21, str(tmp_path), dtype)
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    schedule = [(0, None), (1, None), (1, None), (0, 0)]
+
+    class Reordered:  # the same configuration with another order of execution
+        def __init__(self, inner):
+            self.inner = inner
+
+        def model_spec(self):
+            spec = self.inner.model_spec()
+            return dataclasses.replace(spec, schedule=[ScheduleEntry(l, c) for l, c in schedule])
+
+    config = Reordered(config_from_dict(tiny.CONFIG_A))
+    rt = Runtime(dtype)
+    model = build_model(config.model_spec())
+    runner = ModelRunner(config, load_weights(model, str(tmp_path), rt), rt, page_size=16, num_pages=16,
+                         max_requests=2, max_seq_len=128, model=model)
+    assert runner.kv[0].shape[0] == 3  # three executions own a cache; the fourth reads the first one's
+    prompts = {"a": tiny.random_tokens(40, 256, 7), "b": tiny.random_tokens(9, 256, 8)}
+    expected = {rid: pm.forward(cfg, weights, toks, schedule=schedule) for rid, toks in prompts.items()}
+    for steps in (ru.whole(prompts), ru.chunked(prompts), ru.tail_decoded(prompts, 12)):
+        ru.compare(ru.replay(runner, steps), expected, tol, f"schedule {dtype}")
