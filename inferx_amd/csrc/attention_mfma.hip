@@ -171,22 +171,36 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
 }
 
 // out[t, h, :] = sum_s o_s 2^(m_s - M) / sum_s l_s 2^(m_s - M),  M = max_s m_s
-__global__ void attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                    __bf16* __restrict__ out, int n_splits, int head_dim) {
+// One workgroup per (token, head); the slices' weights are worked out once, then every thread
+// sums its columns with independent loads.
+__global__ void __launch_bounds__(128)
+attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ part_ml, __bf16* __restrict__ out,
+                    int n_splits, int head_dim) {
+  __shared__ float wgt[256];
+  __shared__ float inv_l;
   const int64_t th = blockIdx.x;  // token * heads + head
   const float* ml = part_ml + th * n_splits * 2;
-  float M = -INFINITY;
-  for (int s = 0; s < n_splits; ++s) M = fmaxf(M, ml[2 * s]);
-  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
-    float acc = 0.f, l = 0.f;
-    for (int s = 0; s < n_splits; ++s) {
+  if (threadIdx.x < 64) {
+    float mloc = -INFINITY;
+    for (int s = threadIdx.x; s < n_splits; s += 64) mloc = fmaxf(mloc, ml[2 * s]);
+    const float M = ix_wave_max(mloc);
+    float lloc = 0.f;
+    for (int s = threadIdx.x; s < n_splits; s += 64) {
       const float m_s = ml[2 * s];
-      if (m_s == -INFINITY) continue;
-      const float w = exp2f(m_s - M);
-      acc += w * part_o[(th * n_splits + s) * head_dim + d];
-      l += w * ml[2 * s + 1];
+      const float w = (m_s == -INFINITY) ? 0.f : exp2f(m_s - M);
+      wgt[s] = w;
+      lloc += w * ml[2 * s + 1];
     }
-    out[th * head_dim + d] = (__bf16)(acc / l);
+    const float L = ix_wave_sum(lloc);
+    if (threadIdx.x == 0) inv_l = 1.0f / L;
+  }
+  __syncthreads();
+  const float* po = part_o + th * n_splits * head_dim;
+  for (int d = threadIdx.x; d < head_dim; d += blockDim.x) {
+    float acc = 0.f;
+#pragma unroll 8
+    for (int s = 0; s < n_splits; ++s) acc += wgt[s] * po[s * head_dim + d];
+    out[th * head_dim + d] = (__bf16)(acc * inv_l);
   }
 }
 
@@ -232,7 +246,7 @@ extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void*
 #undef CASE
   if (ix_check_launch("ix_attention_mfma")) return 1;
   if (n_splits > 1) {
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(static_cast<unsigned>(tokens * heads)), dim3(64), 0, stream, part_o,
+    hipLaunchKernelGGL(attn_combine_kernel, dim3(static_cast<unsigned>(tokens * heads)), dim3(128), 0, stream, part_o,
                        part_ml, (__bf16*)out, n_splits, head_dim);
     return ix_check_launch("ix_attention_combine");
   }

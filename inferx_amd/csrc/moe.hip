@@ -18,58 +18,45 @@
 // (reference: RouteTopKKernel, moe.cu:36-127).  Output order: descending score.
 // If `shared_gate_w` is given, sigmoid(x . shared_gate_w) is written too
 // (reference: AddSharedExpertKernel, moe.cu:275-287).
-template <typename T>
-__global__ void __launch_bounds__(ROUTE_THREADS)
-moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dtype,
-                 const void* __restrict__ shared_gate_w, int sg_dtype, float* __restrict__ topk_w,
-                 int32_t* __restrict__ topk_e, float* __restrict__ shared_gate, int64_t width, int experts, int k,
-                 int renormalize, float scale) {
-  extern __shared__ __align__(16) float smem[];
-  float* xs = smem;            // [width]
-  float* z = smem + width;     // [experts + 1]
-  __shared__ float red[16];
-  const int64_t t = blockIdx.x;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int64_t i = tid; i < width; i += ROUTE_THREADS) xs[i] = ix_load(x + t * width + i);
-  __syncthreads();
-  const int rows = experts + (shared_gate_w ? 1 : 0);
-  for (int e = wave; e < rows; e += ROUTE_THREADS / 64) {
-    const void* w = e < experts ? wr : shared_gate_w;
-    const int dt = e < experts ? wr_dtype : sg_dtype;
-    const int64_t base = e < experts ? static_cast<int64_t>(e) * width : 0;
-    float dot = 0.f;
-    if (dt == IX_BF16 && (width & 7) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
-      // eight weights per lane and load (16 bytes); the order of additions is fixed by the lane layout
-      const uint16_t* wrow = static_cast<const uint16_t*>(w) + base;
-      for (int64_t i = lane * 8; i < width; i += 512) {
-        const uint4 v = *reinterpret_cast<const uint4*>(wrow + i);
-        const float4 x0 = *reinterpret_cast<const float4*>(xs + i);
-        const float4 x1 = *reinterpret_cast<const float4*>(xs + i + 4);
-        dot += x0.x * __uint_as_float(v.x << 16) + x0.y * __uint_as_float(v.x & 0xffff0000u) +
-               x0.z * __uint_as_float(v.y << 16) + x0.w * __uint_as_float(v.y & 0xffff0000u) +
-               x1.x * __uint_as_float(v.z << 16) + x1.y * __uint_as_float(v.z & 0xffff0000u) +
-               x1.z * __uint_as_float(v.w << 16) + x1.w * __uint_as_float(v.w & 0xffff0000u);
-      }
-    } else if (dt == IX_F32 && (width & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
-      const float* wrow = static_cast<const float*>(w) + base;
-      for (int64_t i = lane * 4; i < width; i += 256) {
-        const float4 v = *reinterpret_cast<const float4*>(wrow + i);
-        const float4 x0 = *reinterpret_cast<const float4*>(xs + i);
-        dot += x0.x * v.x + x0.y * v.y + x0.z * v.z + x0.w * v.w;
-      }
-    } else {
-      for (int64_t i = lane; i < width; i += 64) dot += xs[i] * ix_load_rt(w, dt, base + i);
+// x . w[row] over `width`, one wavefront, x as float32 at `xs` (LDS or global)
+__device__ __forceinline__ float route_row_dot(const float* __restrict__ xs, const void* __restrict__ w, int dt,
+                                               int64_t base, int64_t width, int lane) {
+  float dot = 0.f;
+  if (dt == IX_BF16 && (width & 7) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+    // eight weights per lane and load (16 bytes); the order of additions is fixed by the lane layout
+    const uint16_t* wrow = static_cast<const uint16_t*>(w) + base;
+    for (int64_t i = lane * 8; i < width; i += 512) {
+      const uint4 v = *reinterpret_cast<const uint4*>(wrow + i);
+      const float4 x0 = *reinterpret_cast<const float4*>(xs + i);
+      const float4 x1 = *reinterpret_cast<const float4*>(xs + i + 4);
+      dot += x0.x * __uint_as_float(v.x << 16) + x0.y * __uint_as_float(v.x & 0xffff0000u) +
+             x0.z * __uint_as_float(v.y << 16) + x0.w * __uint_as_float(v.y & 0xffff0000u) +
+             x1.x * __uint_as_float(v.z << 16) + x1.y * __uint_as_float(v.z & 0xffff0000u) +
+             x1.z * __uint_as_float(v.w << 16) + x1.w * __uint_as_float(v.w & 0xffff0000u);
     }
-    dot = ix_wave_sum(dot);
-    if (lane == 0) z[e] = dot;
+  } else if (dt == IX_F32 && (width & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
+    const float* wrow = static_cast<const float*>(w) + base;
+    for (int64_t i = lane * 4; i < width; i += 256) {
+      const float4 v = *reinterpret_cast<const float4*>(wrow + i);
+      const float4 x0 = *reinterpret_cast<const float4*>(xs + i);
+      dot += x0.x * v.x + x0.y * v.y + x0.z * v.z + x0.w * v.w;
+    }
+  } else {
+    for (int64_t i = lane; i < width; i += 64) dot += xs[i] * ix_load_rt(w, dt, base + i);
   }
-  __syncthreads();
-  if (shared_gate_w && tid == 0) shared_gate[t] = 1.0f / (1.0f + expf(-z[experts]));
+  return ix_wave_sum(dot);
+}
+
+// softmax over z[0..experts) (LDS, overwritten) and k rounds of argmax, by the whole workgroup
+__device__ __forceinline__ void route_select(float* z, float* red, float* __restrict__ topk_w,
+                                             int32_t* __restrict__ topk_e, int64_t t, int experts, int k,
+                                             int renormalize, float scale) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   float mx = -INFINITY;
-  for (int e = tid; e < experts; e += ROUTE_THREADS) mx = fmaxf(mx, z[e]);
+  for (int e = tid; e < experts; e += blockDim.x) mx = fmaxf(mx, z[e]);
   mx = ix_block_max(mx, red);
   float sum = 0.f;
-  for (int e = tid; e < experts; e += ROUTE_THREADS) {
+  for (int e = tid; e < experts; e += blockDim.x) {
     const float p = expf(z[e] - mx);
     z[e] = p;
     sum += p;
@@ -107,24 +94,101 @@ moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dt
   if (lane < k) topk_w[t * k + lane] = chosen * f;
 }
 
+// One workgroup per token: x row in LDS, every router row against it (many tokens: prompt portions).
+template <typename T>
+__global__ void __launch_bounds__(ROUTE_THREADS)
+moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dtype,
+                 const void* __restrict__ shared_gate_w, int sg_dtype, float* __restrict__ topk_w,
+                 int32_t* __restrict__ topk_e, float* __restrict__ shared_gate, int64_t width, int experts, int k,
+                 int renormalize, float scale) {
+  extern __shared__ __align__(16) float smem[];
+  float* xs = smem;                        // [width rounded up to 4]
+  float* z = smem + ((width + 3) & ~3);    // [experts + 1]
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int64_t i = tid; i < width; i += ROUTE_THREADS) xs[i] = ix_load(x + t * width + i);
+  __syncthreads();
+  const int rows = experts + (shared_gate_w ? 1 : 0);
+  for (int e = wave; e < rows; e += ROUTE_THREADS / 64) {
+    const bool routed = e < experts;
+    const float dot = route_row_dot(xs, routed ? wr : shared_gate_w, routed ? wr_dtype : sg_dtype,
+                                    routed ? static_cast<int64_t>(e) * width : 0, width, lane);
+    if (lane == 0) z[e] = dot;
+  }
+  __syncthreads();
+  if (shared_gate_w && tid == 0) shared_gate[t] = 1.0f / (1.0f + expf(-z[experts]));
+  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale);
+}
+
+// Few tokens (decoding): the router rows are spread over many workgroups, one row per wavefront,
+// scores go to `logits` [tokens, experts + 1]; a second small kernel selects.
+template <typename T>
+__global__ void __launch_bounds__(ROUTE_THREADS)
+moe_route_logits_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dtype,
+                        const void* __restrict__ shared_gate_w, int sg_dtype, float* __restrict__ logits,
+                        int64_t width, int experts) {
+  extern __shared__ __align__(16) float xs[];  // [width]
+  const int64_t t = blockIdx.x;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int64_t i = tid; i < width; i += ROUTE_THREADS) xs[i] = ix_load(x + t * width + i);
+  __syncthreads();
+  const int rows = experts + (shared_gate_w ? 1 : 0);
+  const int e = blockIdx.y * (ROUTE_THREADS / 64) + wave;
+  if (e >= rows) return;
+  const bool routed = e < experts;
+  const float dot = route_row_dot(xs, routed ? wr : shared_gate_w, routed ? wr_dtype : sg_dtype,
+                                  routed ? static_cast<int64_t>(e) * width : 0, width, lane);
+  if (lane == 0) logits[t * (experts + 1) + e] = dot;
+}
+
+__global__ void __launch_bounds__(64)
+moe_route_select_kernel(const float* __restrict__ logits, float* __restrict__ topk_w, int32_t* __restrict__ topk_e,
+                        float* __restrict__ shared_gate, int experts, int k, int renormalize, float scale) {
+  extern __shared__ __align__(16) float z[];  // [experts]
+  __shared__ float red[16];
+  const int64_t t = blockIdx.x;
+  for (int e = threadIdx.x; e < experts; e += 64) z[e] = logits[t * (experts + 1) + e];
+  if (shared_gate && threadIdx.x == 0) shared_gate[t] = 1.0f / (1.0f + expf(-logits[t * (experts + 1) + experts]));
+  __syncthreads();
+  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale);
+}
+
+// `logits_scratch`: float32 [tokens, experts + 1], used when tokens <= ROUTE_SMALL_TOKENS (may be null otherwise).
+#define ROUTE_SMALL_TOKENS 128
 extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dtype, const void* shared_gate_w,
-                            int sg_dtype, float* topk_w, int32_t* topk_e, float* shared_gate, int64_t tokens,
-                            int64_t width, int experts, int k, int renormalize, float scale, hipStream_t stream) {
+                            int sg_dtype, float* topk_w, int32_t* topk_e, float* shared_gate, float* logits_scratch,
+                            int64_t tokens, int64_t width, int experts, int k, int renormalize, float scale,
+                            hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
   IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
   IX_REQUIRE(k > 0 && k <= experts && k <= IX_MAX_TOP_K, "top_k must be between 1 and min(experts, 32)");
-  const size_t smem = (width + experts + 1) * sizeof(float);
+  IX_REQUIRE(dtype == IX_F32 || dtype == IX_BF16, "dtype must be float32 or bfloat16");
+  const size_t smem = (((width + 3) & ~3) + experts + 1) * sizeof(float);
   IX_REQUIRE(smem <= 60 * 1024, "hidden width too large for the router kernel (limit about 15000)");
   if (tokens == 0) return 0;
+  if (tokens <= ROUTE_SMALL_TOKENS && logits_scratch != nullptr) {
+    const int rows = experts + (shared_gate_w ? 1 : 0);
+    dim3 grid(tokens, (rows + ROUTE_THREADS / 64 - 1) / (ROUTE_THREADS / 64)), block(ROUTE_THREADS);
+    const size_t xs_bytes = ((width + 3) & ~3) * sizeof(float);
+    if (dtype == IX_F32)
+      hipLaunchKernelGGL(moe_route_logits_kernel<float>, grid, block, xs_bytes, stream, (const float*)x, wr, wr_dtype,
+                         shared_gate_w, sg_dtype, logits_scratch, width, experts);
+    else
+      hipLaunchKernelGGL(moe_route_logits_kernel<bf16_t>, grid, block, xs_bytes, stream, (const bf16_t*)x, wr,
+                         wr_dtype, shared_gate_w, sg_dtype, logits_scratch, width, experts);
+    hipLaunchKernelGGL(moe_route_select_kernel, dim3(tokens), dim3(64), experts * sizeof(float), stream,
+                       logits_scratch, topk_w, topk_e, shared_gate_w ? shared_gate : nullptr, experts, k, renormalize,
+                       scale);
+    return ix_check_launch("ix_moe_route");
+  }
   dim3 grid(tokens), block(ROUTE_THREADS);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, smem, stream, (const float*)x, wr, wr_dtype,
                        shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale);
-  else if (dtype == IX_BF16)
+  else
     hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, smem, stream, (const bf16_t*)x, wr, wr_dtype,
                        shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale);
-  else
-    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_moe_route");
 }
 
@@ -205,6 +269,58 @@ moe_scatter_kernel(const int32_t* __restrict__ topk_e, const int32_t* __restrict
   }
 }
 
+// Few assignments (decoding): one workgroup does counts, offsets, the stable placement and the tile map.
+// rank of assignment a within its expert = number of earlier assignments of the same expert.
+#define DISPATCH_SMALL_MAX 1024
+__global__ void __launch_bounds__(1024)
+moe_dispatch_small_kernel(const int32_t* __restrict__ topk_e, int32_t* __restrict__ offsets,
+                          int32_t* __restrict__ rows, int32_t* __restrict__ dest, int assignments, int experts, int k,
+                          int tile_rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
+                          int32_t* __restrict__ tile_info) {
+  __shared__ int32_t chosen[DISPATCH_SMALL_MAX];
+  __shared__ int32_t counts[IX_MAX_EXPERTS];
+  __shared__ int32_t first_row[IX_MAX_EXPERTS];
+  __shared__ int32_t first_tile[IX_MAX_EXPERTS];
+  const int tid = threadIdx.x;
+  for (int e = tid; e < experts; e += blockDim.x) counts[e] = 0;
+  if (tid < assignments) chosen[tid] = topk_e[tid];
+  __syncthreads();
+  int mine = -1, rank = 0;
+  if (tid < assignments) {
+    mine = chosen[tid];
+    for (int b = 0; b < tid; ++b) rank += (chosen[b] == mine) ? 1 : 0;
+    if (mine >= 0 && mine < experts) atomicAdd(&counts[mine], 1);  // integer counts: order does not matter
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int32_t run = 0, tiles = 0;
+    for (int e = 0; e < experts; ++e) {
+      offsets[e] = run;
+      first_row[e] = run;
+      first_tile[e] = tiles;
+      run += counts[e];
+      if (tile_rows > 0) tiles += (counts[e] + tile_rows - 1) / tile_rows;
+    }
+    offsets[experts] = run;
+    if (tile_info) tile_info[0] = tiles;
+  }
+  __syncthreads();
+  if (tid < assignments && mine >= 0 && mine < experts) {
+    const int32_t r = first_row[mine] + rank;
+    rows[r] = tid / k;
+    dest[tid] = r;
+  }
+  if (tile_rows > 0 && tile_expert) {
+    for (int e = tid; e < experts; e += blockDim.x) {
+      const int n = (counts[e] + tile_rows - 1) / tile_rows;
+      for (int i = 0; i < n; ++i) {
+        tile_expert[first_tile[e] + i] = e;
+        tile_row0[first_tile[e] + i] = first_row[e] + i * tile_rows;
+      }
+    }
+  }
+}
+
 // tile_expert / tile_row0 need room for min(A, ceil(A / tile_rows) + E) entries; tile_rows 0 skips the map.
 extern "C" int ix_moe_dispatch(const int32_t* topk_e, int32_t* offsets, int32_t* rows, int32_t* dest,
                                int64_t assignments, int experts, int k, int tile_rows, int32_t* tile_expert,
@@ -213,6 +329,11 @@ extern "C" int ix_moe_dispatch(const int32_t* topk_e, int32_t* offsets, int32_t*
   IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
   IX_REQUIRE(tile_rows >= 0, "tile_rows must not be negative");
   IX_REQUIRE(tile_rows == 0 || (tile_expert && tile_row0 && tile_info), "tile map buffers needed");
+  if (assignments > 0 && assignments <= DISPATCH_SMALL_MAX) {
+    hipLaunchKernelGGL(moe_dispatch_small_kernel, dim3(1), dim3(1024), 0, stream, topk_e, offsets, rows, dest,
+                       (int)assignments, experts, k, tile_rows, tile_expert, tile_row0, tile_info);
+    return ix_check_launch("ix_moe_dispatch");
+  }
   hipLaunchKernelGGL(moe_count_scan_kernel, dim3(1), dim3(1024), 0, stream, topk_e, offsets, assignments, experts,
                      tile_rows, tile_expert, tile_row0, tile_info);
   if (assignments > 0)

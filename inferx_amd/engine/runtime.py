@@ -41,6 +41,7 @@ class Runtime:
         from .. import ops
         ops.lib()  # fail now, loudly, if the HIP library cannot be had
         self._mm_out_dtype_ok: Optional[bool] = None
+        self._skinny_plans: Dict[int, Any] = {}
 
     @property
     def is_fp32(self) -> bool:
@@ -59,12 +60,48 @@ class Runtime:
             return t.to(self.device, torch.float32)
         return t.to(self.device, torch.bfloat16)
 
+    # ---- few rows (decoding): the weights are the traffic, so they are streamed by the matrix-core kernel
+    # that also serves the experts (one "expert", one row tile), instead of a library product tuned for tiles
+    SKINNY_ROWS = 64
+
+    def _skinny_ok(self, x: torch.Tensor, w: torch.Tensor) -> bool:
+        return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < x.shape[0] <= self.SKINNY_ROWS
+                and x.shape[1] % 8 == 0 and x.is_contiguous() and w.is_contiguous())
+
+    def _skinny(self, x: torch.Tensor, w: torch.Tensor, gate_up: bool) -> torch.Tensor:
+        from .. import ops
+        T = x.shape[0]
+        plan = self._skinny_plans.get(T)
+        if plan is None:
+            tile_rows = 16 if T <= 16 else (32 if T <= 32 else 64)
+            mt = ops.moe_max_tiles(T, 1, tile_rows)
+            tile_map = torch.tensor([0] * (2 * mt) + [1], dtype=torch.int32, device=self.device)
+            offsets = torch.tensor([0, T], dtype=torch.int32, device=self.device)
+            plan = self._skinny_plans[T] = (offsets, tile_map, tile_rows)
+        offsets, tile_map, tile_rows = plan
+        n_out = w.shape[0] // 2 if gate_up else w.shape[0]
+        out = self.empty((T, n_out))
+        ops.moe_grouped_mfma(x, w.unsqueeze(0), out, offsets, None, tile_map, tile_rows, gate_up, 4)
+        return out
+
     def linear(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         """x [T, in] . w[out, in]^T -> [T, out] in the run's type, float32 accumulation.
         A weight kept in float32 during a bfloat16 run is multiplied in float32."""
         if w.dtype == x.dtype:
+            if self._skinny_ok(x, w):
+                return self._skinny(x, w, False)
             return torch.matmul(x, w.t())
         return torch.matmul(x.to(torch.float32), w.to(torch.float32).t()).to(self.dtype)
+
+    def gated_linear(self, x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+        """silu(x . Wg^T) * (x . Wu^T) for w_gate_up = [Wg; Wu] of shape [2 n, in] -> [T, n]."""
+        from .. import ops
+        if self._skinny_ok(x, w_gate_up):
+            return self._skinny(x, w_gate_up, True)
+        gate_up = self.linear(x, w_gate_up)
+        act = self.empty((x.shape[0], w_gate_up.shape[0] // 2))
+        ops.silu_mul(gate_up, act)
+        return act
 
     def linear_f32(self, x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         """As `linear`, result float32 (the logits)."""

@@ -206,6 +206,9 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
           _i32(block_table.shape[1]), _f32(scale), _i32(window), _stream())
 
 
+ROUTE_SMALL_TOKENS = 128
+
+
 def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor], topk_w: torch.Tensor,
               topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor], renormalize: bool, scale: float) -> None:
     """Router product, softmax and top-k in float32; optional sigmoid gate of the shared expert."""
@@ -219,9 +222,12 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
         _need(shared_gate_w.numel() == H, "shared gate weight must hold `hidden` numbers")
         _need(shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= T,
               "shared_gate must be float32 [T]")
+    scratch = None
+    if T <= ROUTE_SMALL_TOKENS:  # few tokens: scores go through a scratch so that many workgroups share the rows
+        scratch = torch.empty((T, E + 1), dtype=torch.float32, device=x.device)
     _call("ix_moe_route", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
           _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(topk_w), _ptr(topk_e),
-          _ptr(shared_gate if shared_gate_w is not None else None), _i64(T), _i64(H), _i32(E), _i32(k),
+          _ptr(shared_gate if shared_gate_w is not None else None), _ptr(scratch), _i64(T), _i64(H), _i32(E), _i32(k),
           _i32(1 if renormalize else 0), _f32(scale), _stream())
 
 

@@ -39,10 +39,7 @@ class DenseMlp(FeedForward):
 
     def forward(self, ctx, x):
         rt = ctx.rt
-        gate_up = rt.linear(x, self.w_gate_up)
-        act = rt.empty((x.shape[0], self.width))
-        ops.silu_mul(gate_up, act)
-        return rt.linear(act, self.w_down)
+        return rt.linear(rt.gated_linear(x, self.w_gate_up), self.w_down)
 
 
 register_part("feed_forward", "dense_mlp", DenseMlp)

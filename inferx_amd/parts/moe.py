@@ -111,10 +111,7 @@ class MoeFeedForward(FeedForward):
 
     def shared(self, ctx, x):
         rt = ctx.rt
-        gate_up = rt.linear(x, self.w_shared_gate_up)
-        act = rt.empty((x.shape[0], self.shared_width))
-        ops.silu_mul(gate_up, act)
-        return rt.linear(act, self.w_shared_down)
+        return rt.linear(rt.gated_linear(x, self.w_shared_gate_up), self.w_shared_down)
 
     def forward(self, ctx, x):
         topk_w, topk_e, gate = self.route(ctx, x)
