@@ -62,7 +62,7 @@ class Runtime:
 
     # ---- few rows (decoding): the weights are the traffic, so they are streamed by the matrix-core kernel
     # that also serves the experts (one "expert", one row tile), instead of a library product tuned for tiles
-    SKINNY_ROWS = 64
+    SKINNY_ROWS = 16  # beyond one 16-row tile the activations' re-reads outweigh the gain
 
     def _skinny_ok(self, x: torch.Tensor, w: torch.Tensor) -> bool:
         return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and 0 < x.shape[0] <= self.SKINNY_ROWS

@@ -281,6 +281,29 @@ def moe_grouped_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
           _i32(1 if gate_up else 0), _i32(k_split), _stream())
 
 
+def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
+                      rows: Optional[torch.Tensor], tile_map: torch.Tensor, gate_up: bool) -> None:
+    """Grouped product staged through LDS (bfloat16, many rows per expert); `tile_map` made for tiles of 64 rows."""
+    E = w.shape[0]
+    A, n_out = out.shape
+    K = a.shape[1]
+    _need(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.bfloat16,
+          "the matrix-core grouped product is bfloat16 only")
+    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if gate_up else n_out),
+          "expert weight shape does not fit")
+    _need(K % 8 == 0, "the reduction width must be a multiple of 8")
+    _is_i32(offsets, E + 1)
+    if rows is not None:
+        _is_i32(rows, A)
+    else:
+        _need(a.shape[0] >= A, "a has fewer rows than out")
+    mt = moe_max_tiles(A, E, 64)
+    _is_i32(tile_map, 2 * mt + 1)
+    _call("ix_moe_grouped_tiled", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
+          _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i64(n_out), _i64(K),
+          _i32(1 if gate_up else 0), _stream())
+
+
 def moe_grouped_plain(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
                       rows: Optional[torch.Tensor], gate_up: bool) -> None:
     """Grouped product over device offsets.  gate_up: a [T, H] gathered through `rows`,

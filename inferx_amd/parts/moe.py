@@ -100,7 +100,10 @@ class MoeFeedForward(FeedForward):
         rt, A = ctx.rt, rows.numel()
         act = rt.empty((A, self.expert_width))
         y = rt.empty((A, self.hidden_size))
-        if tile_rows:
+        if tile_rows == 64:  # many rows per expert: operands staged through LDS
+            ops.moe_grouped_tiled(x, self.w13, act, offsets, rows, tile_map, True)
+            ops.moe_grouped_tiled(act, self.w2, y, offsets, None, tile_map, False)
+        elif tile_rows:
             k_split = 4 if A <= 1024 else 1  # few rows: the weights are the traffic, split the reduction
             ops.moe_grouped_mfma(x, self.w13, act, offsets, rows, tile_map, tile_rows, True, k_split)
             ops.moe_grouped_mfma(act, self.w2, y, offsets, None, tile_map, tile_rows, False, k_split)
