@@ -204,6 +204,88 @@ __global__ void qkv_rope_append_kernel(const T* __restrict__ qkv, const void* __
   }
 }
 
+// The same for bfloat16 with head_dim a multiple of 16: a thread takes eight consecutive elements of the
+// low half of a head and the eight of the high half that pair with them (16-byte loads and stores).
+__global__ void __launch_bounds__(256)
+qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
+                            const float2* __restrict__ cs, const int32_t* __restrict__ slots,
+                            uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache,
+                            uint16_t* __restrict__ v_cache, int heads, int kv_heads, int head_dim, int page_size,
+                            int64_t total_slots) {
+  const int64_t t = blockIdx.x;
+  const int half = head_dim / 2, per_head = half / 8;
+  const int items = (heads + 2 * kv_heads) * per_head;
+  const int64_t in_width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
+  const uint16_t* in = qkv + t * in_width;
+  const int64_t slot = slots ? slots[t] : -1;
+  const bool cache_ok = k_cache != nullptr && slot >= 0 && slot < total_slots;
+  const int64_t page = cache_ok ? slot / page_size : 0;
+  const int off = cache_ok ? static_cast<int>(slot % page_size) : 0;
+  for (int p = blockIdx.y * blockDim.x + threadIdx.x; p < items; p += gridDim.y * blockDim.x) {
+    const int head = p / per_head, j = (p - head * per_head) * 8;
+    const int col = head * head_dim + j;
+    const uint4 lo4 = *reinterpret_cast<const uint4*>(in + col);
+    const uint4 hi4 = *reinterpret_cast<const uint4*>(in + col + half);
+    const uint32_t lw[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, hw[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
+    float lo[8], hi[8];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo[2 * i] = __uint_as_float(lw[i] << 16);
+      lo[2 * i + 1] = __uint_as_float(lw[i] & 0xffff0000u);
+      hi[2 * i] = __uint_as_float(hw[i] << 16);
+      hi[2 * i + 1] = __uint_as_float(hw[i] & 0xffff0000u);
+    }
+    if (bias) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        lo[i] += ix_load_rt(bias, bias_dtype, col + i);
+        hi[i] += ix_load_rt(bias, bias_dtype, col + half + i);
+      }
+    }
+    const bool is_v = head >= heads + kv_heads;
+    if (!is_v && cs) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float2 c = cs[t * half + j + i];
+        const float rlo = lo[i] * c.x - hi[i] * c.y;
+        const float rhi = hi[i] * c.x + lo[i] * c.y;
+        lo[i] = rlo;
+        hi[i] = rhi;
+      }
+    }
+    uint16_t lb[8], hb[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      lb[i] = ix_f32_to_bf16(lo[i]);
+      hb[i] = ix_f32_to_bf16(hi[i]);
+    }
+    if (is_v) {
+      if (cache_ok) {
+        const int g = head - heads - kv_heads;
+        uint16_t* dst = v_cache + ((page * kv_heads + g) * head_dim + j) * page_size + off;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+          dst[static_cast<int64_t>(i) * page_size] = lb[i];
+          dst[static_cast<int64_t>(half + i) * page_size] = hb[i];
+        }
+      }
+    } else {
+      uint16_t* dst = nullptr;
+      if (head < heads) dst = q_out + (t * heads + head) * head_dim + j;
+      else if (cache_ok) dst = k_cache + ((page * kv_heads + (head - heads)) * page_size + off) * head_dim + j;
+      if (dst) {
+        uint4 a, b;
+        a.x = lb[0] | (uint32_t)lb[1] << 16; a.y = lb[2] | (uint32_t)lb[3] << 16;
+        a.z = lb[4] | (uint32_t)lb[5] << 16; a.w = lb[6] | (uint32_t)lb[7] << 16;
+        b.x = hb[0] | (uint32_t)hb[1] << 16; b.y = hb[2] | (uint32_t)hb[3] << 16;
+        b.z = hb[4] | (uint32_t)hb[5] << 16; b.w = hb[6] | (uint32_t)hb[7] << 16;
+        *reinterpret_cast<uint4*>(dst) = a;
+        *reinterpret_cast<uint4*>(dst + half) = b;
+      }
+    }
+  }
+}
+
 extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const void* cs,
                                   const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int64_t tokens,
                                   int heads, int kv_heads, int head_dim, int page_size, int64_t total_slots,
@@ -218,7 +300,13 @@ extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, 
     hipLaunchKernelGGL(qkv_rope_append_kernel<float>, grid, block, 0, stream, (const float*)qkv, bias, bias_dtype,
                        (const float2*)cs, slots, (float*)q_out, (float*)k_cache, (float*)v_cache, heads, kv_heads,
                        head_dim, page_size, total_slots);
-  else if (dtype == IX_BF16)
+  else if (dtype == IX_BF16 && head_dim % 16 == 0) {
+    const int items8 = (heads + 2 * kv_heads) * (head_dim / 16);
+    dim3 grid8(tokens, std::min((items8 + 255) / 256, 8));
+    hipLaunchKernelGGL(qkv_rope_append_vec8_kernel, grid8, block, 0, stream, (const uint16_t*)qkv, bias, bias_dtype,
+                       (const float2*)cs, slots, (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, heads,
+                       kv_heads, head_dim, page_size, total_slots);
+  } else if (dtype == IX_BF16)
     hipLaunchKernelGGL(qkv_rope_append_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)qkv, bias, bias_dtype,
                        (const float2*)cs, slots, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads,
                        head_dim, page_size, total_slots);

@@ -337,6 +337,28 @@ def moe_combine(y: torch.Tensor, dest: torch.Tensor, topk_w: torch.Tensor, share
           _ptr(shared_gate if shared is not None else None), _ptr(out), _i64(T), _i64(H), _i32(k), _stream())
 
 
+def moe_combine_add_rmsnorm(h: torch.Tensor, y: torch.Tensor, dest: torch.Tensor, topk_w: torch.Tensor,
+                            shared: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor], weight: torch.Tensor,
+                            out: torch.Tensor, eps: float, rows: Optional[torch.Tensor] = None) -> None:
+    """`moe_combine` followed by `add_rmsnorm` in one pass: h += sum; out = rmsnorm(h) * weight."""
+    T, k = topk_w.shape
+    H = h.shape[1]
+    _need(h.dtype == torch.float32 and h.shape[0] == T, "the residual stream is float32 [T, H]")
+    _need(y.shape[1] == H and y.shape[0] >= T * k and out.dtype == y.dtype and out.shape[1] == H, "shape mismatch")
+    _need(weight.numel() == H, "norm weight length differs")
+    _is_i32(dest, T * k)
+    n_out = out.shape[0]
+    if rows is None:
+        _need(n_out == T, "out must have a row per token")
+    else:
+        _is_i32(rows, n_out)
+    if shared is not None:
+        _need(shared.shape == (T, H) and shared.dtype == y.dtype, "shared mismatch")
+    _call("ix_moe_combine_add_rmsnorm", _ptr(h), _ptr(y), _i32(_dt(y)), _ptr(dest), _ptr(topk_w), _ptr(shared),
+          _ptr(shared_gate if shared is not None else None), _ptr(weight), _i32(_dt(weight)), _ptr(out), _ptr(rows),
+          _i64(n_out), _i64(H), _i32(k), _f32(eps), _stream())
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     R, V = logits.shape
     _need(logits.dtype == torch.float32, "logits must be float32")

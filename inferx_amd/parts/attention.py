@@ -124,7 +124,7 @@ def query_tiles(ctx, window: int, heads: int):
         base = ctx.memo["attention_tiles_host"] = (tiles_dev, tiles_host.shape[1], longest)
     tiles_dev, n_tiles, longest = base
     span = min(longest, window + QUERY_TILE + 32) if window > 0 else longest
-    n_splits = max(1, min(-(-WAVES_WANTED // max(1, n_tiles * heads)), -(-span // MIN_KEYS_PER_SPLIT), 64))
+    n_splits = max(1, min(WAVES_WANTED // max(1, n_tiles * heads), -(-span // MIN_KEYS_PER_SPLIT), 64))
     n_splits = 1 << (n_splits.bit_length() - 1)  # a power of two: few distinct values, few captured graphs
     ctx.memo[key] = (tiles_dev, n_splits)
     return ctx.memo[key]

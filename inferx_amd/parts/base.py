@@ -54,6 +54,24 @@ class StateNeed:
     shape: Tuple[int, ...]
 
 
+class LazyDelta:
+    """What a mixer or feed-forward may return instead of a tensor: a delta that is not formed yet, so that the
+    norm that consumes it can form it, add it to the residual stream and normalise in one kernel.
+    A norm that cannot do that calls `materialize` and goes on with the tensor."""
+
+    def materialize(self, ctx):
+        raise NotImplementedError
+
+    def add_rmsnorm(self, ctx, h, weight, eps, rows, out) -> bool:
+        """h += delta; out = rmsnorm(h) * weight.  Returns False if this case is not fused (then nothing was done)."""
+        return False
+
+
+def resolve_delta(ctx, delta):
+    """A tensor (or None) whatever `delta` is."""
+    return delta.materialize(ctx) if isinstance(delta, LazyDelta) else delta
+
+
 class Part:
     # True if `forward` only launches work on the current stream (no host reads of device data, no host-side
     # planning from the batch), so that a step can be captured into a HIP graph

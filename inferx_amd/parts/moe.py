@@ -15,7 +15,7 @@ from typing import List
 import torch
 
 from .. import ops
-from .base import FeedForward, ParamSpec, register_part
+from .base import FeedForward, LazyDelta, ParamSpec, register_part
 from .dense_mlp import stack_rows
 
 
@@ -122,9 +122,25 @@ class MoeFeedForward(FeedForward):
         offsets, rows, dest, tile_map = self.dispatch(ctx, topk_e, tile_rows)
         y = self.experts(ctx, x, offsets, rows, tile_map, tile_rows)
         shared = self.shared(ctx, x) if self.shared_width > 0 else None
-        out = ctx.rt.empty((x.shape[0], self.hidden_size))
-        ops.moe_combine(y, dest, topk_w, shared, gate, out)
+        return MoeSum(y, dest, topk_w, shared, gate, self.hidden_size)
+
+
+class MoeSum(LazyDelta):
+    """sum_s topk_w[t, s] * y[dest[t, s]] + gate[t] * shared[t], formed by whoever consumes it."""
+
+    def __init__(self, y, dest, topk_w, shared, gate, width):
+        self.y, self.dest, self.topk_w, self.shared, self.gate, self.width = y, dest, topk_w, shared, gate, width
+
+    def materialize(self, ctx):
+        out = ctx.rt.empty((self.topk_w.shape[0], self.width))
+        ops.moe_combine(self.y, self.dest, self.topk_w, self.shared, self.gate, out)
         return out
+
+    def add_rmsnorm(self, ctx, h, weight, eps, rows, out) -> bool:
+        if self.width * 4 > 60 * 1024:
+            return False
+        ops.moe_combine_add_rmsnorm(h, self.y, self.dest, self.topk_w, self.shared, self.gate, weight, out, eps, rows)
+        return True
 
 
 register_part("feed_forward", "moe", MoeFeedForward)

@@ -8,7 +8,7 @@ from __future__ import annotations
 from typing import List
 
 from .. import ops
-from .base import Norm, ParamSpec, register_part
+from .base import LazyDelta, Norm, ParamSpec, register_part
 
 
 class RMSNorm(Norm):
@@ -29,6 +29,10 @@ class RMSNorm(Norm):
         picks rows out); returns the normalised rows in the run's type."""
         n = h.shape[0] if rows is None else rows.numel()
         out = ctx.rt.empty((n, self.width))
+        if isinstance(delta, LazyDelta):
+            if delta.add_rmsnorm(ctx, h, self.weight, self.eps, rows, out):
+                return out
+            delta = delta.materialize(ctx)
         ops.add_rmsnorm(h, delta, self.weight, out, self.eps, rows)
         return out
 

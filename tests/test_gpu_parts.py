@@ -153,7 +153,9 @@ def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated):
                          wd["m.shared_expert.down_proj.weight"])
     else:
         want = pm.moe_block(x.double(), wd, "m.", E, k, renorm, si)
-    got = part.forward(ctx, x.to(DEV))
+    from inferx_amd.parts import resolve_delta
+    lazy = part.forward(ctx, x.to(DEV))
+    got = resolve_delta(ctx, lazy)
     assert err(got, want) < tol
     # the routing itself, exactly (float32 scores): experts and weights per slot
     topk_w, topk_e, _ = part.route(ctx, x.to(DEV))
@@ -161,9 +163,38 @@ def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated):
     assert torch.equal(topk_e.cpu().long(), want_e)
     assert err(topk_w, want_w) < 1e-5
     # repeat runs are bitwise equal (reference: tests/kernel/moe_test.cc:972-1046)
-    again = part.forward(ctx, x.to(DEV))
+    again = resolve_delta(ctx, part.forward(ctx, x.to(DEV)))
     assert torch.equal(got.view(torch.int16 if dtype == "bfloat16" else torch.int32),
                        again.view(torch.int16 if dtype == "bfloat16" else torch.int32))
+
+
+@pytest.mark.parametrize("dtype,tol", PARAMS)
+def test_norm_fuses_the_expert_sum(dtype, tol):
+    """The norm forms a lazy expert sum itself: same stream and same output as sum, add, norm one after the other."""
+    from inferx_amd.config import PartSpec
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import LazyDelta, build_part, resolve_delta
+    rt = Runtime(dtype)
+    H, T = 96, 21
+    moe = build_part("feed_forward", PartSpec("moe", {"hidden_size": H, "num_experts": 8, "top_k": 3,
+                                                      "expert_width": 48, "shared_width": 80, "init_std": 0.15}))
+    moe.bind({n: v.to(DEV) for n, v in tensors_for(moe, rt, seed=11).items()}, rt)
+    norm = build_part("norm", PartSpec("rmsnorm", {"width": H, "eps": 1e-5}))
+    norm.bind({"weight": (torch.rand(H) + 0.5).to(rt.dtype).to(DEV)}, rt)
+    ctx, _ = make_ctx(rt, [T], [T], 16, 4)
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(12)).to(rt.dtype).to(DEV)
+    h0 = torch.randn(T, H, generator=torch.Generator().manual_seed(13)).to(DEV)
+    lazy = moe.forward(ctx, x)
+    assert isinstance(lazy, LazyDelta)
+    h1, h2 = h0.clone(), h0.clone()
+    fused = norm.forward(ctx, h1, lazy)
+    plain = norm.forward(ctx, h2, resolve_delta(ctx, lazy))
+    assert err(h1, h2) < (1e-6 if dtype == "float32" else 1e-2)
+    assert err(fused, plain) < (1e-5 if dtype == "float32" else 1e-2)
+    rows = torch.tensor([T - 1, 0, 5, 5], dtype=torch.int32, device=DEV)
+    h3 = h0.clone()
+    picked = norm.forward(ctx, h3, lazy, rows=rows)
+    assert torch.equal(h3, h0) and err(picked, plain[rows.long()]) < (1e-5 if dtype == "float32" else 1e-2)
 
 
 def test_registry_errors():
