@@ -27,7 +27,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define ATTN_KEYS_PER_ITER 32
 
-template <int NB>  // head_dim = 16 * NB
+// head_dim = 16 * NB; a tile holds up to 16 * QT queries; PF: request the next iteration's keys and values
+// before this iteration's are multiplied (pays when few wavefronts are resident: decoding)
+template <int NB, int QT, bool PF>
 __global__ void __launch_bounds__(256)
 attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                  const int32_t* __restrict__ block_table, const int32_t* __restrict__ tile_seq,
@@ -58,29 +60,33 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
   const int ks = lo_al + split * per;
   const int ke = min(hi, ks + per);
 
-  const int my_pos = pos0 + n;  // this lane's query (column n)
-  const bool my_row = n < rows;
-  const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
-
-  // Q as B operand: lane (n, g) holds Q[query n][32 c + 8 g .. +8]
-  bf16x8 qf[NC];
+  // Q as B operand: lane (n, g) holds Q[query 16 t + n][32 c + 8 g .. +8]
+  bf16x8 qf[QT][NC];
 #pragma unroll
-  for (int c = 0; c < NC; ++c) {
-    const int d0 = 32 * c + 8 * g;
-    if (my_row && d0 < D)
-      qf[c] = *reinterpret_cast<const bf16x8*>(q + (static_cast<int64_t>(tq0 + n) * heads + head) * D + d0);
-    else
-      for (int j = 0; j < 8; ++j) qf[c][j] = (__bf16)0.f;
+  for (int t = 0; t < QT; ++t)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int d0 = 32 * c + 8 * g;
+      if (16 * t + n < rows && d0 < D)
+        qf[t][c] =
+            *reinterpret_cast<const bf16x8*>(q + (static_cast<int64_t>(tq0 + 16 * t + n) * heads + head) * D + d0);
+      else
+        for (int j = 0; j < 8; ++j) qf[t][c][j] = (__bf16)0.f;
+    }
+
+  f32x4 o[QT][NB];
+  float m[QT], lsum[QT];
+#pragma unroll
+  for (int t = 0; t < QT; ++t) {
+    m[t] = -INFINITY;
+    lsum[t] = 0.f;
+#pragma unroll
+    for (int b = 0; b < NB; ++b) o[t][b] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
-  f32x4 o[NB];
-#pragma unroll
-  for (int b = 0; b < NB; ++b) o[b] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, lsum = 0.f;
-
-  for (int kb = ks; kb < ke; kb += ATTN_KEYS_PER_ITER) {
-    // ---- S^T for 32 keys: two blocks of 16 rows ----
-    f32x4 s[2];
+  // K fragments for the 32 keys from kb on (two blocks of 16 rows) and V^T fragments
+  // (lane (dd = n, g) holds V^T[16 blk + dd][kb + 8 g .. +8])
+  auto load_kv = [&](int kb, bf16x8 (&kf)[2][NC], bf16x8 (&vf)[NB]) {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       int key = kb + 8 * (n >> 2) + 4 * b + (n & 3);  // A row n of block b
@@ -89,83 +95,115 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
       page = max(page, 0);                             // a page the window has passed: masked below
       const __bf16* kr =
           k_cache + ((static_cast<int64_t>(page) * kv_heads + kvh) * page_size + key % page_size) * D;
-      s[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const int d0 = 32 * c + 8 * g;
-        bf16x8 kf;
         if (d0 < D)
-          kf = *reinterpret_cast<const bf16x8*>(kr + d0);
+          kf[b][c] = *reinterpret_cast<const bf16x8*>(kr + d0);
         else
-          for (int j = 0; j < 8; ++j) kf[j] = (__bf16)0.f;
-        s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[c], s[b], 0, 0, 0);
+          for (int j = 0; j < 8; ++j) kf[b][c][j] = (__bf16)0.f;
       }
     }
-    // ---- V^T fragments: lane (dd = n, g) holds V^T[16 blk + dd][kb + 8 g .. +8] ----
-    bf16x8 vf[NB];
-    {
-      int key = min(kb + 8 * g, hi - 1) & ~7;
-      int page = max(table[key / page_size], 0);
-      const __bf16* vr = v_cache + (static_cast<int64_t>(page) * kv_heads + kvh) * D * page_size + key % page_size;
+    int key = min(kb + 8 * g, hi - 1) & ~7;
+    int page = max(table[key / page_size], 0);
+    const __bf16* vr = v_cache + (static_cast<int64_t>(page) * kv_heads + kvh) * D * page_size + key % page_size;
 #pragma unroll
-      for (int b = 0; b < NB; ++b)
-        vf[b] = *reinterpret_cast<const bf16x8*>(vr + static_cast<int64_t>(16 * b + n) * page_size);
+    for (int b = 0; b < NB; ++b)
+      vf[b] = *reinterpret_cast<const bf16x8*>(vr + static_cast<int64_t>(16 * b + n) * page_size);
+  };
+
+  bf16x8 kf_next[PF ? 2 : 1][PF ? NC : 1], vf_next[PF ? NB : 1];
+  if constexpr (PF) {
+    if (ks < ke) load_kv(ks, kf_next, vf_next);
+  }
+  for (int kb = ks; kb < ke; kb += ATTN_KEYS_PER_ITER) {
+    bf16x8 kf[2][NC], vf[NB];
+    if constexpr (PF) {
+#pragma unroll
+      for (int b = 0; b < 2; ++b)
+#pragma unroll
+        for (int c = 0; c < NC; ++c) kf[b][c] = kf_next[b][c];
+#pragma unroll
+      for (int b = 0; b < NB; ++b) vf[b] = vf_next[b];
+      if (kb + ATTN_KEYS_PER_ITER < ke) load_kv(kb + ATTN_KEYS_PER_ITER, kf_next, vf_next);
+    } else {
+      load_kv(kb, kf, vf);
     }
-    // ---- mask, online softmax for this lane's query over its 8 keys ----
-    float sv[8];
-    float mx = -INFINITY;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int key = kb + 8 * g + j;
-      const bool ok = my_row && key >= my_lo && key <= my_pos && key < ke;
-      sv[j] = ok ? s[j >> 2][j & 3] * scale_log2 : -INFINITY;
-      mx = fmaxf(mx, sv[j]);
-    }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-    const float m_new = fmaxf(m, mx);
-    const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-    const float alpha = exp2f(m - m_safe);
-    float psum = 0.f;
-    bf16x8 pf;
+    for (int t = 0; t < QT; ++t) {
+      if (QT > 1 && (16 * t >= rows || kb > pos0 + 16 * t + 15)) continue;  // no query of this block reads these keys
+      // ---- S^T = K Q^T ----
+      f32x4 s[2];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float p = exp2f(sv[j] - m_safe);
-      psum += p;
-      pf[j] = (__bf16)p;
-    }
-    lsum = lsum * alpha + psum;
-    m = m_new;
-    // ---- O^T += V^T P^T ----
+      for (int b = 0; b < 2; ++b) {
+        s[b] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      o[b] *= alpha;
-      o[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf, o[b], 0, 0, 0);
+        for (int c = 0; c < NC; ++c) s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b][c], qf[t][c], s[b], 0, 0, 0);
+      }
+      // ---- mask, online softmax for this lane's query over its 8 keys ----
+      const int my_pos = pos0 + 16 * t + n;
+      const bool my_row = 16 * t + n < rows;
+      const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
+      float sv[8];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = kb + 8 * g + j;
+        const bool ok = my_row && key >= my_lo && key <= my_pos && key < ke;
+        sv[j] = ok ? s[j >> 2][j & 3] * scale_log2 : -INFINITY;
+        mx = fmaxf(mx, sv[j]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m[t], mx);
+      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
+      const float alpha = exp2f(m[t] - m_safe);
+      float psum = 0.f;
+      bf16x8 pf;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float p = exp2f(sv[j] - m_safe);
+        psum += p;
+        pf[j] = (__bf16)p;
+      }
+      lsum[t] = lsum[t] * alpha + psum;
+      m[t] = m_new;
+      // ---- O^T += V^T P^T ----
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        o[t][b] *= alpha;
+        o[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf, o[t][b], 0, 0, 0);
+      }
     }
   }
-  lsum += __shfl_xor(lsum, 16, 64);
-  lsum += __shfl_xor(lsum, 32, 64);
-  if (!my_row) return;
 
-  // lane holds O^T rows d = 16 b + 4 g + i of column n
-  if (n_splits == 1) {
-    const float inv = 1.0f / lsum;
-    __bf16* dst = out + (static_cast<int64_t>(tq0 + n) * heads + head) * D + 4 * g;
 #pragma unroll
-    for (int b = 0; b < NB; ++b) {
-      bf16x4 v;
+  for (int t = 0; t < QT; ++t) {
+    float l = lsum[t];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    if (16 * t + n >= rows) continue;
+    // lane holds O^T rows d = 16 b + 4 g + i of column n
+    const int64_t token = tq0 + 16 * t + n;
+    if (n_splits == 1) {
+      const float inv = 1.0f / l;
+      __bf16* dst = out + (token * heads + head) * D + 4 * g;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) v[i] = (__bf16)(o[b][i] * inv);
-      *reinterpret_cast<bf16x4*>(dst + 16 * b) = v;
-    }
-  } else {
-    const int64_t p = (static_cast<int64_t>(tq0 + n) * heads + head) * n_splits + split;
-    float* dst = part_o + p * D + 4 * g;
+      for (int b = 0; b < NB; ++b) {
+        bf16x4 v;
 #pragma unroll
-    for (int b = 0; b < NB; ++b) *reinterpret_cast<f32x4*>(dst + 16 * b) = o[b];
-    if (g == 0) {
-      part_ml[2 * p] = m;
-      part_ml[2 * p + 1] = lsum;
+        for (int i = 0; i < 4; ++i) v[i] = (__bf16)(o[t][b][i] * inv);
+        *reinterpret_cast<bf16x4*>(dst + 16 * b) = v;
+      }
+    } else {
+      const int64_t p = (token * heads + head) * n_splits + split;
+      float* dst = part_o + p * D + 4 * g;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) *reinterpret_cast<f32x4*>(dst + 16 * b) = o[t][b];
+      if (g == 0) {
+        part_ml[2 * p] = m[t];
+        part_ml[2 * p + 1] = l;
+      }
     }
   }
 }
@@ -204,13 +242,13 @@ attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ 
   }
 }
 
-template <int NB>
+template <int NB, int QT, bool PF>
 static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void* k, const void* v,
                         const int32_t* table, const int32_t* tile_seq, const int32_t* tile_q0,
                         const int32_t* tile_rows, const int32_t* positions, void* out, float* part_o, float* part_ml,
                         int n_tiles, int n_splits, int heads, int kv_heads, int page_size, int max_blocks,
                         float scale_log2, int window) {
-  hipLaunchKernelGGL(attn_mfma_kernel<NB>, grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
+  hipLaunchKernelGGL((attn_mfma_kernel<NB, QT, PF>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, positions, (__bf16*)out, part_o, part_ml,
                      n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window);
 }
@@ -220,8 +258,11 @@ static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void
 extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                                  const int32_t* tile_seq, const int32_t* tile_q0, const int32_t* tile_rows,
                                  const int32_t* positions, void* out, float* part_o, float* part_ml, int64_t tokens,
-                                 int n_tiles, int n_splits, int heads, int kv_heads, int head_dim, int page_size,
-                                 int max_blocks, float scale, int window, hipStream_t stream) {
+                                 int n_tiles, int tile_queries, int n_splits, int heads, int kv_heads, int head_dim,
+                                 int page_size, int max_blocks, float scale, int window, int prefetch,
+                                 hipStream_t stream) {
+  IX_REQUIRE(tile_queries == 16 || tile_queries == 32, "a query tile holds up to 16 or 32 queries");
+  IX_REQUIRE(tile_queries == 16 || head_dim <= 128, "tiles of 32 queries need head_dim <= 128");
   IX_REQUIRE(tokens >= 0 && n_tiles >= 0 && heads > 0 && kv_heads > 0 && max_blocks > 0, "sizes must be positive");
   IX_REQUIRE(heads % kv_heads == 0, "heads must be a multiple of kv_heads");
   IX_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 256, "head_dim must be a multiple of 16 up to 256");
@@ -234,16 +275,31 @@ extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void*
   const int64_t units = static_cast<int64_t>(n_tiles) * n_splits;
   dim3 grid(static_cast<unsigned>((units + 3) / 4), heads);
   const float scale_log2 = scale * 1.4426950408889634f;
-#define CASE(NB)                                                                                                   \
-  case NB:                                                                                                         \
-    launch_attn<NB>(grid, stream, q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, positions, out,  \
-                    part_o, part_ml, n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window); \
+#define ARGS                                                                                                    \
+  grid, stream, q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, positions, out, part_o, part_ml, \
+      n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window
+#define CASE(NB)                                   \
+  case NB:                                         \
+    if (prefetch) launch_attn<NB, 1, true>(ARGS);  \
+    else launch_attn<NB, 1, false>(ARGS);          \
     break;
-  switch (head_dim / 16) {
-    CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
-    CASE(9) CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
+#define CASE4(NB)                        \
+  case NB:                               \
+    launch_attn<NB, 2, false>(ARGS);     \
+    break;
+  if (tile_queries == 16) {
+    switch (head_dim / 16) {
+      CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8)
+      CASE(9) CASE(10) CASE(11) CASE(12) CASE(13) CASE(14) CASE(15) CASE(16)
+    }
+  } else {
+    switch (head_dim / 16) {
+      CASE4(1) CASE4(2) CASE4(3) CASE4(4) CASE4(5) CASE4(6) CASE4(7) CASE4(8)
+    }
   }
 #undef CASE
+#undef CASE4
+#undef ARGS
   if (ix_check_launch("ix_attention_mfma")) return 1;
   if (n_splits > 1) {
     hipLaunchKernelGGL(attn_combine_kernel, dim3(static_cast<unsigned>(tokens * heads)), dim3(128), 0, stream, part_o,

@@ -190,14 +190,14 @@ class _DecodeGraph:
         ctx = runner._context(self.dev, sizes, all_rows)
         # the attention plan of a one-token-per-request step never changes: tile i = request i, row i, one query
         tiles = torch.tensor([list(range(S)), list(range(S)), [1] * S], dtype=torch.int32, device=rt.device)
-        ctx.memo["attention_tiles_host"] = (tiles, S, bucket)
+        ctx.memo[("attention_tiles_host", 16)] = (tiles, S, bucket)
         ctx.host = None  # nothing may plan from host data inside the capture
         self.ctx = ctx
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             runner.model.forward(ctx, runner.bindings)  # warm-up: library plans, allocator
-            ctx.memo = {"attention_tiles_host": (tiles, S, bucket)}
+            ctx.memo = {("attention_tiles_host", 16): (tiles, S, bucket)}
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()

@@ -178,9 +178,10 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 
 def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, n_splits: int,
-                   workspace: Optional[torch.Tensor], scale: float, window: int) -> None:
+                   workspace: Optional[torch.Tensor], scale: float, window: int, tile_queries: int = 16,
+                   prefetch: bool = False) -> None:
     """Paged attention on the matrix cores (bfloat16).  `tiles` int32 [3, n_tiles]: request, first token row and
-    number of rows (<= 16) of each query tile.  `workspace` float32 with T * heads * n_splits * (d + 2) entries
+    number of rows (<= tile_queries, which is 16 or 32) of each query tile.  `workspace` float32 with T * heads * n_splits * (d + 2) entries
     when n_splits > 1."""
     T, heads, d = q.shape
     _need(q.dtype == torch.bfloat16, "the matrix-core attention kernel is bfloat16 only")
@@ -202,8 +203,8 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
         part_ml = workspace[T * heads * n_splits * d:]
     _call("ix_attention_mfma", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
           _ptr(tiles[1]), _ptr(tiles[2]), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), _i64(T),
-          _i32(n_tiles), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(page_size),
-          _i32(block_table.shape[1]), _f32(scale), _i32(window), _stream())
+          _i32(n_tiles), _i32(tile_queries), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(page_size),
+          _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(1 if prefetch else 0), _stream())
 
 
 ROUTE_SMALL_TOKENS = 128

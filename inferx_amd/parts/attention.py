@@ -86,47 +86,52 @@ class PagedAttention(Mixer):
         """bfloat16 with pages and heads in multiples of 16: the matrix-core kernel; else the plain one."""
         page_size = cache.k.shape[2]
         if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0:
-            tiles, n_splits = query_tiles(ctx, self.window, self.num_heads)
+            tiles, tile, n_splits = query_tiles(ctx, self.window, self.num_heads, self.head_dim)
             work = None
             if n_splits > 1:
                 work = ctx.rt.empty((q.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),), torch.float32)
             ops.attention_mfma(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, out,
-                               n_splits, work, self.scale, self.window)
+                               n_splits, work, self.scale, self.window, tile,
+                               prefetch=ctx.num_tokens == ctx.num_requests)
         else:
             ops.attention_plain(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.seq_of_token, ctx.positions,
                                 out, self.scale, self.window)
 
 
-QUERY_TILE = 16          # queries of one request per wavefront
+QUERY_TILE = 16          # queries of one request per wavefront ...
+LARGE_QUERY_TILE = 32    # ... or 32 when the step brings many tokens (keys and values are then read once per 32)
+LARGE_TILE_TOKENS = 1 << 30  # measured: no faster than tiles of 16 on MI355X, so off
 WAVES_WANTED = 4096      # enough wavefronts to fill 256 compute units
 MIN_KEYS_PER_SPLIT = 128
 
 
-def query_tiles(ctx, window: int, heads: int):
-    """Tiles of up to 16 consecutive queries per request (int32 [3, n]: request, first row, rows) on the device,
-    and into how many slices each tile's keys are cut.  Planned on the host from the step's batch, once per step."""
-    key = ("attention_tiles", window, heads)
+def query_tiles(ctx, window: int, heads: int, head_dim: int = 128):
+    """Tiles of consecutive queries per request (int32 [3, n]: request, first row, rows) on the device, the tile
+    size (16 or 32) and into how many slices each tile's keys are cut.  Planned on the host from the step's
+    batch, once per step; a captured step finds its (static) plan already in `ctx.memo`."""
+    tile = LARGE_QUERY_TILE if (ctx.num_tokens >= LARGE_TILE_TOKENS and head_dim <= 128) else QUERY_TILE
+    key = ("attention_tiles", window, heads, tile)
     hit = ctx.memo.get(key)
     if hit is not None:
         return hit
-    base = ctx.memo.get("attention_tiles_host")
+    base = ctx.memo.get(("attention_tiles_host", tile))
     if base is None:
         b = ctx.host
         n = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
-        counts = -(-n // QUERY_TILE)
+        counts = -(-n // tile)
         seq = np.repeat(np.arange(len(n)), counts)
         first = np.cumsum(counts) - counts
-        off = (np.arange(int(counts.sum())) - np.repeat(first, counts)) * QUERY_TILE
-        rows = np.minimum(QUERY_TILE, n[seq] - off)
+        off = (np.arange(int(counts.sum())) - np.repeat(first, counts)) * tile
+        rows = np.minimum(tile, n[seq] - off)
         tiles_host = np.stack([seq, b.q_start[:-1][seq] + off, rows]).astype(np.int32)
         tiles_dev = torch.from_numpy(np.ascontiguousarray(tiles_host)).to(ctx.rt.device)
         longest = int(b.seq_lens.max()) if len(b.seq_lens) else 0
-        base = ctx.memo["attention_tiles_host"] = (tiles_dev, tiles_host.shape[1], longest)
+        base = ctx.memo[("attention_tiles_host", tile)] = (tiles_dev, tiles_host.shape[1], longest)
     tiles_dev, n_tiles, longest = base
-    span = min(longest, window + QUERY_TILE + 32) if window > 0 else longest
+    span = min(longest, window + tile + 32) if window > 0 else longest
     n_splits = max(1, min(WAVES_WANTED // max(1, n_tiles * heads), -(-span // MIN_KEYS_PER_SPLIT), 64))
     n_splits = 1 << (n_splits.bit_length() - 1)  # a power of two: few distinct values, few captured graphs
-    ctx.memo[key] = (tiles_dev, n_splits)
+    ctx.memo[key] = (tiles_dev, tile, n_splits)
     return ctx.memo[key]
 
 

@@ -103,29 +103,31 @@ def test_attention_plain(case, dtype):
     close(out, attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window), TOL[dtype], "attention_plain")
 
 
-def tiles_for(q_lens):
+def tiles_for(q_lens, tile=16):
     rows, at = [], 0
     for s, n in enumerate(q_lens):
-        for q0 in range(0, n, 16):
-            rows.append((s, at + q0, min(16, n - q0)))
+        for q0 in range(0, n, tile):
+            rows.append((s, at + q0, min(tile, n - q0)))
         at += n
     return torch.tensor(rows, dtype=torch.int32).t().contiguous().to(DEV)
 
 
+@pytest.mark.parametrize("tile", [16, 32, -16])  # -16: tiles of 16 with prefetch
 @pytest.mark.parametrize("n_splits", [1, 3, 8])
 @pytest.mark.parametrize("case", ATTN_CASES)
-def test_attention_mfma(case, n_splits):
+def test_attention_mfma(case, n_splits, tile):
     from inferx_amd import ops
     seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    prefetch, tile = tile < 0, abs(tile)
     p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, torch.bfloat16, seed=4)
     out = torch.full_like(p["q"], float("nan"))
     T = p["q"].shape[0]
     work = torch.empty(T * heads * n_splits * (d + 2), dtype=torch.float32, device=DEV) if n_splits > 1 else None
     scale = d ** -0.5
-    ops.attention_mfma(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for(q_lens), p["positions"], out,
-                       n_splits, work, scale, window)
+    ops.attention_mfma(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for(q_lens, tile), p["positions"], out,
+                       n_splits, work, scale, window, tile, prefetch)
     close(out, attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window), TOL[torch.bfloat16],
-          f"attention_mfma splits={n_splits}")
+          f"attention_mfma splits={n_splits} tile={tile}")
 
 
 def test_attention_finds_one_far_key():
