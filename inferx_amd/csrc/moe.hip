@@ -507,3 +507,26 @@ extern "C" int ix_moe_combine(const void* y, int dtype, const int32_t* dest, con
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_moe_combine");
 }
+
+// Router scores only: logits float32 [tokens, experts + 1] (the last column is the shared expert's gate score,
+// written when shared_gate_w is given).  For few tokens; selection and grouping then happen in
+// ix_moe_select_dispatch (moe_route_small.hip).
+extern "C" int ix_moe_route_logits(const void* x, int dtype, const void* wr, int wr_dtype, const void* shared_gate_w,
+                                   int sg_dtype, float* logits, int64_t tokens, int64_t width, int experts,
+                                   hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
+  IX_REQUIRE(dtype == IX_F32 || dtype == IX_BF16, "dtype must be float32 or bfloat16");
+  const size_t xs_bytes = ((width + 3) & ~3) * sizeof(float);
+  IX_REQUIRE(xs_bytes <= 60 * 1024, "hidden width too large for the router kernel (limit about 15000)");
+  if (tokens == 0) return 0;
+  const int rows = experts + (shared_gate_w ? 1 : 0);
+  dim3 grid(tokens, (rows + ROUTE_THREADS / 64 - 1) / (ROUTE_THREADS / 64)), block(ROUTE_THREADS);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(moe_route_logits_kernel<float>, grid, block, xs_bytes, stream, (const float*)x, wr, wr_dtype,
+                       shared_gate_w, sg_dtype, logits, width, experts);
+  else
+    hipLaunchKernelGGL(moe_route_logits_kernel<bf16_t>, grid, block, xs_bytes, stream, (const bf16_t*)x, wr,
+                       wr_dtype, shared_gate_w, sg_dtype, logits, width, experts);
+  return ix_check_launch("ix_moe_route_logits");
+}

@@ -25,23 +25,15 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// The work of one wavefront (KSPLIT == 1) or workgroup (KSPLIT == 4): rows [row0, row_end) x out-features
+// [n0, n0 + 16) of expert e.  `red`: LDS for the partial sums of a split reduction.
 template <int MT, bool GATE_UP, int KSPLIT>
-__global__ void __launch_bounds__(256)
-moe_grouped_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w, __bf16* __restrict__ out,
-                        const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
-                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
-                        const int32_t* __restrict__ tile_info, int n_out, int width) {
+__device__ __forceinline__ void grouped_body(const __bf16* __restrict__ a, const __bf16* __restrict__ w,
+                                             __bf16* __restrict__ out, const int32_t* __restrict__ rows, int e,
+                                             int row0, int row_end, int n0, int n_out, int width, float* red) {
   constexpr int NACC = GATE_UP ? 2 : 1;
-  __shared__ float red[KSPLIT > 1 ? 3 * 64 * MT * NACC * 4 : 1];
-  if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m = lane & 15, g = lane >> 4;
-  const int e = tile_expert[blockIdx.y];
-  const int row0 = tile_row0[blockIdx.y];
-  const int row_end = offsets[e + 1];
-
-  const int n0 = (KSPLIT > 1 ? blockIdx.x : blockIdx.x * 4 + wave) * 16;
-  if (n0 >= n_out) return;  // whole wavefront (KSPLIT == 1) or whole workgroup
   const int kper = KSPLIT > 1 ? (((width + KSPLIT - 1) / KSPLIT + 127) & ~127) : width;
   const int kbegin = KSPLIT > 1 ? wave * kper : 0;
   const int kend = min(width, kbegin + kper);
@@ -135,6 +127,49 @@ moe_grouped_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__
   }
 }
 
+template <int MT, bool GATE_UP, int KSPLIT>
+__global__ void __launch_bounds__(256)
+moe_grouped_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w, __bf16* __restrict__ out,
+                        const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
+                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
+                        const int32_t* __restrict__ tile_info, int n_out, int width) {
+  __shared__ float red[KSPLIT > 1 ? 3 * 64 * MT * (GATE_UP ? 2 : 1) * 4 : 1];
+  if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
+  const int e = tile_expert[blockIdx.y];
+  const int n0 = (KSPLIT > 1 ? blockIdx.x : blockIdx.x * 4 + (threadIdx.x >> 6)) * 16;
+  if (n0 >= n_out) return;  // whole wavefront (KSPLIT == 1) or whole workgroup
+  grouped_body<MT, GATE_UP, KSPLIT>(a, w, out, rows, e, tile_row0[blockIdx.y], offsets[e + 1], n0, n_out, width, red);
+}
+
+// Routed experts and the shared expert in one launch (decoding: every launch saved counts).  Workgroups
+// [0, n16_e * max_tiles) serve the routed experts' row tiles, the rest the shared expert, which is one more
+// "expert" over all `shared_rows` tokens with weights and sizes of its own.
+template <int MT, bool GATE_UP>
+__global__ void __launch_bounds__(256)
+moe_grouped_dual_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w, __bf16* __restrict__ out,
+                        const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
+                        const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
+                        const int32_t* __restrict__ tile_info, int max_tiles, int n_out, int width,
+                        const __bf16* __restrict__ a_s, const __bf16* __restrict__ w_s, __bf16* __restrict__ out_s,
+                        int shared_rows, int n_out_s, int width_s) {
+  __shared__ float red[3 * 64 * MT * (GATE_UP ? 2 : 1) * 4];
+  const int n16_e = (n_out + 15) / 16;
+  int idx = blockIdx.x;
+  if (idx < n16_e * max_tiles) {
+    const int tile = idx / n16_e;
+    if (tile >= tile_info[0]) return;
+    const int e = tile_expert[tile];
+    grouped_body<MT, GATE_UP, 4>(a, w, out, rows, e, tile_row0[tile], offsets[e + 1], (idx - tile * n16_e) * 16, n_out,
+                                 width, red);
+  } else {
+    idx -= n16_e * max_tiles;
+    const int n16_s = (n_out_s + 15) / 16;
+    const int tile = idx / n16_s;
+    grouped_body<MT, GATE_UP, 4>(a_s, w_s, out_s, nullptr, 0, tile * 16 * MT, shared_rows, (idx - tile * n16_s) * 16,
+                                 n_out_s, width_s, red);
+  }
+}
+
 // `max_tiles` bounds the number of row tiles (the grid); the kernel reads the true number from tile_info.
 // tile_rows (16, 32 or 64) must be what the grouping kernel was given.
 extern "C" int ix_moe_grouped_mfma(const void* a, const void* w, void* out, const int32_t* offsets,
@@ -166,4 +201,35 @@ extern "C" int ix_moe_grouped_mfma(const void* a, const void* w, void* out, cons
 #undef PICK
 #undef LAUNCH
   return ix_check_launch("ix_moe_grouped_mfma");
+}
+
+// One launch for the routed experts (as ix_moe_grouped_mfma with k_split 4) and the shared expert
+// (a_s [shared_rows, width_s] . w_s[(2) n_out_s, width_s]^T -> out_s [shared_rows, n_out_s]).
+extern "C" int ix_moe_grouped_dual(const void* a, const void* w, void* out, const int32_t* offsets,
+                                   const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
+                                   const int32_t* tile_info, int max_tiles, int tile_rows, int64_t n_out,
+                                   int64_t width, const void* a_s, const void* w_s, void* out_s, int shared_rows,
+                                   int64_t n_out_s, int64_t width_s, int gate_up, hipStream_t stream) {
+  IX_REQUIRE(n_out > 0 && width > 0 && n_out_s > 0 && width_s > 0 && max_tiles >= 0 && shared_rows > 0,
+             "sizes must be positive");
+  IX_REQUIRE(width % 8 == 0 && width_s % 8 == 0, "the reduction widths must be multiples of 8");
+  IX_REQUIRE(n_out < (1 << 24) && width < (1 << 30) && n_out_s < (1 << 24) && width_s < (1 << 30), "sizes too large");
+  IX_REQUIRE(tile_rows == 16 || tile_rows == 32 || tile_rows == 64, "tile_rows must be 16, 32 or 64");
+  const int64_t n16_e = (n_out + 15) / 16, n16_s = (n_out_s + 15) / 16;
+  const int64_t shared_tiles = (shared_rows + tile_rows - 1) / tile_rows;
+  const int64_t blocks = n16_e * max_tiles + n16_s * shared_tiles;
+  IX_REQUIRE(blocks < (1ll << 31), "too many workgroups");
+  dim3 grid(static_cast<unsigned>(blocks)), block(256);
+#define LAUNCH(MT, GU)                                                                                            \
+  hipLaunchKernelGGL((moe_grouped_dual_kernel<MT, GU>), grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w, \
+                     (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, max_tiles, (int)n_out,        \
+                     (int)width, (const __bf16*)a_s, (const __bf16*)w_s, (__bf16*)out_s, shared_rows, (int)n_out_s, \
+                     (int)width_s)
+#define PICK(MT)               \
+  if (gate_up) LAUNCH(MT, true); \
+  else LAUNCH(MT, false);
+  if (tile_rows == 16) { PICK(1) } else if (tile_rows == 32) { PICK(2) } else { PICK(4) }
+#undef PICK
+#undef LAUNCH
+  return ix_check_launch("ix_moe_grouped_dual");
 }

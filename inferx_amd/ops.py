@@ -232,6 +232,47 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
           _i32(1 if renormalize else 0), _f32(scale), _stream())
 
 
+SELECT_DISPATCH_MAX_ASSIGNMENTS, SELECT_DISPATCH_MAX_EXPERTS = 1024, 256
+
+
+def moe_route_dispatch(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor],
+                       topk_w: torch.Tensor, topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor],
+                       renormalize: bool, scale: float, offsets: torch.Tensor, rows: torch.Tensor,
+                       dest: torch.Tensor, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None) -> None:
+    """`moe_route` and `moe_dispatch` for few tokens in two launches: router scores spread over many workgroups,
+    then selection and grouping in one workgroup.  Needs T * k <= 1024 and at most 256 experts."""
+    T, H = x.shape
+    E = router_w.shape[0]
+    k = topk_w.shape[1]
+    A = T * k
+    _need(A <= SELECT_DISPATCH_MAX_ASSIGNMENTS and E <= SELECT_DISPATCH_MAX_EXPERTS and T > 0,
+          "too many assignments or experts for the fused selection")
+    _need(router_w.shape == (E, H), "router weight must be [experts, hidden]")
+    _need(topk_w.shape == (T, k) and topk_w.dtype == torch.float32, "topk_w must be float32 [T, k]")
+    _need(topk_e.shape == (T, k) and topk_e.dtype == torch.int32, "topk_e must be int32 [T, k]")
+    if shared_gate_w is not None:
+        _need(shared_gate_w.numel() == H, "shared gate weight must hold `hidden` numbers")
+        _need(shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= T,
+              "shared_gate must be float32 [T]")
+    _is_i32(offsets, E + 1)
+    _is_i32(rows, A)
+    _is_i32(dest, A)
+    te = tr = ti = None
+    if tile_rows > 0:
+        mt = moe_max_tiles(A, E, tile_rows)
+        _need(tile_map is not None, "tile_map needed")
+        _is_i32(tile_map, 2 * mt + 1)
+        te, tr, ti = tile_map[:mt], tile_map[mt:2 * mt], tile_map[2 * mt:]
+    logits = torch.empty((T, E + 1), dtype=torch.float32, device=x.device)
+    _call("ix_moe_route_logits", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
+          _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits), _i64(T), _i64(H), _i32(E),
+          _stream())
+    _call("ix_moe_select_dispatch", _ptr(logits), _ptr(topk_w), _ptr(topk_e),
+          _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest), _i32(T),
+          _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(tile_rows), _ptr(te), _ptr(tr), _ptr(ti),
+          _stream())
+
+
 def moe_dispatch(topk_e: torch.Tensor, offsets: torch.Tensor, rows: torch.Tensor, dest: torch.Tensor,
                  experts: int, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None) -> None:
     """Group assignments by expert: offsets [E+1], rows [A] (grouped row -> token), dest [A].
@@ -280,6 +321,35 @@ def moe_grouped_mfma(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
     _call("ix_moe_grouped_mfma", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
           _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i32(tile_rows), _i64(n_out), _i64(K),
           _i32(1 if gate_up else 0), _i32(k_split), _stream())
+
+
+def moe_grouped_dual(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
+                     rows: Optional[torch.Tensor], tile_map: torch.Tensor, tile_rows: int, a_s: torch.Tensor,
+                     w_s: torch.Tensor, out_s: torch.Tensor, gate_up: bool) -> None:
+    """`moe_grouped_mfma` (split reduction) for the routed experts and, in the same launch, the shared expert:
+    out_s = a_s . w_s^T (with SwiGLU when gate_up)."""
+    E = w.shape[0]
+    A, n_out = out.shape
+    K = a.shape[1]
+    T, n_out_s = out_s.shape
+    K_s = a_s.shape[1]
+    for t in (a, w, out, a_s, w_s, out_s):
+        _need(t.dtype == torch.bfloat16, "the matrix-core grouped product is bfloat16 only")
+    _need(w.dim() == 3 and w.shape[2] == K and w.shape[1] == (2 * n_out if gate_up else n_out),
+          "expert weight shape does not fit")
+    _need(w_s.shape == ((2 * n_out_s if gate_up else n_out_s), K_s) and a_s.shape[0] == T,
+          "shared weight shape does not fit")
+    _need(K % 8 == 0 and K_s % 8 == 0, "the reduction widths must be multiples of 8")
+    _is_i32(offsets, E + 1)
+    if rows is not None:
+        _is_i32(rows, A)
+    else:
+        _need(a.shape[0] >= A, "a has fewer rows than out")
+    mt = moe_max_tiles(A, E, tile_rows)
+    _is_i32(tile_map, 2 * mt + 1)
+    _call("ix_moe_grouped_dual", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
+          _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i32(tile_rows), _i64(n_out), _i64(K),
+          _ptr(a_s), _ptr(w_s), _ptr(out_s), _i32(T), _i64(n_out_s), _i64(K_s), _i32(1 if gate_up else 0), _stream())
 
 
 def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,

@@ -112,16 +112,49 @@ class MoeFeedForward(FeedForward):
             ops.moe_grouped_plain(act, self.w2, y, offsets, None, gate_up=False)
         return y
 
+    def _one_launch(self, ctx, x, tile_rows: int) -> bool:
+        """Few tokens (decoding): routed and shared experts go into one launch per product."""
+        return (tile_rows in (16, 32) and self.shared_width > 0 and self.shared_width % 8 == 0
+                and x.shape[0] <= ctx.rt.SKINNY_ROWS and self.w_shared_gate_up.dtype == torch.bfloat16
+                and self.w_shared_down.dtype == torch.bfloat16)
+
+    def experts_and_shared(self, ctx, x, offsets, rows, tile_map, tile_rows):
+        rt, A, T = ctx.rt, rows.numel(), x.shape[0]
+        act, sact = rt.empty((A, self.expert_width)), rt.empty((T, self.shared_width))
+        ops.moe_grouped_dual(x, self.w13, act, offsets, rows, tile_map, tile_rows, x, self.w_shared_gate_up, sact, True)
+        y, sout = rt.empty((A, self.hidden_size)), rt.empty((T, self.hidden_size))
+        ops.moe_grouped_dual(act, self.w2, y, offsets, None, tile_map, tile_rows, sact, self.w_shared_down, sout, False)
+        return y, sout
+
     def shared(self, ctx, x):
         rt = ctx.rt
         return rt.linear(rt.gated_linear(x, self.w_shared_gate_up), self.w_shared_down)
 
+    def route_and_dispatch(self, ctx, x, tile_rows: int):
+        """`route` then `dispatch`; for few tokens the selection and the grouping share one launch."""
+        rt, T, k, E = ctx.rt, x.shape[0], self.top_k, self.num_experts
+        if T * k > ops.SELECT_DISPATCH_MAX_ASSIGNMENTS or E > ops.SELECT_DISPATCH_MAX_EXPERTS:
+            topk_w, topk_e, gate = self.route(ctx, x)
+            return (topk_w, topk_e, gate) + self.dispatch(ctx, topk_e, tile_rows)
+        topk_w = rt.empty((T, k), torch.float32)
+        topk_e = rt.empty((T, k), torch.int32)
+        gate = rt.empty((T,), torch.float32) if self.w_shared_gate is not None else None
+        offsets = rt.empty((E + 1,), torch.int32)
+        rows = rt.empty((T * k,), torch.int32)
+        dest = rt.empty((T * k,), torch.int32)
+        tile_map = rt.empty((2 * ops.moe_max_tiles(T * k, E, tile_rows) + 1,), torch.int32) if tile_rows else None
+        ops.moe_route_dispatch(x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate, self.renormalize,
+                               self.routed_scale, offsets, rows, dest, tile_rows, tile_map)
+        return topk_w, topk_e, gate, offsets, rows, dest, tile_map
+
     def forward(self, ctx, x):
-        topk_w, topk_e, gate = self.route(ctx, x)
         tile_rows = self._tile_rows(x)
-        offsets, rows, dest, tile_map = self.dispatch(ctx, topk_e, tile_rows)
-        y = self.experts(ctx, x, offsets, rows, tile_map, tile_rows)
-        shared = self.shared(ctx, x) if self.shared_width > 0 else None
+        topk_w, topk_e, gate, offsets, rows, dest, tile_map = self.route_and_dispatch(ctx, x, tile_rows)
+        if self._one_launch(ctx, x, tile_rows):
+            y, shared = self.experts_and_shared(ctx, x, offsets, rows, tile_map, tile_rows)
+        else:
+            y = self.experts(ctx, x, offsets, rows, tile_map, tile_rows)
+            shared = self.shared(ctx, x) if self.shared_width > 0 else None
         return MoeSum(y, dest, topk_w, shared, gate, self.hidden_size)
 
 

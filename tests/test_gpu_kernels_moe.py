@@ -117,6 +117,31 @@ def test_dispatch_is_a_stable_bijection(T, E, k, tile_rows):
         assert covered == list(range(A))  # tiles cover every row once, in order
 
 
+@pytest.mark.parametrize("T,H,E,k,renorm,tile_rows", [(1, 64, 4, 2, False, 16), (8, 2048, 60, 4, False, 16),
+                                                       (37, 96, 8, 3, True, 32), (128, 72, 5, 1, False, 0),
+                                                       (32, 200, 256, 32, True, 16)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_route_and_dispatch_in_two_launches(T, H, E, k, renorm, tile_rows, dtype):
+    """The fused selection + grouping gives exactly what the separate kernels give."""
+    from inferx_amd import ops
+    x, wr, wsg = rnd(T, H, dtype=dtype), rnd(E, H, seed=1, dtype=dtype, scale=0.3), rnd(1, H, seed=2, dtype=dtype, scale=0.1)
+    A = T * k
+    mk = lambda *shape, dt=torch.int32: torch.full(shape, -9, dtype=dt, device=DEV)
+    w1, e1, g1 = mk(T, k, dt=torch.float32), mk(T, k), mk(T, dt=torch.float32)
+    ops.moe_route(x, wr, wsg, w1, e1, g1, renorm, 1.0)
+    o1, r1, d1, tm1 = dispatch(e1, E, tile_rows)
+    w2, e2, g2 = mk(T, k, dt=torch.float32), mk(T, k), mk(T, dt=torch.float32)
+    o2, r2, d2 = mk(E + 1), mk(A), mk(A)
+    tm2 = mk(2 * ops.moe_max_tiles(A, E, tile_rows) + 1) if tile_rows else None
+    ops.moe_route_dispatch(x, wr, wsg, w2, e2, g2, renorm, 1.0, o2, r2, d2, tile_rows, tm2)
+    assert torch.equal(e1, e2) and torch.equal(o1, o2) and torch.equal(r1, r2) and torch.equal(d1, d2)
+    assert rel_err(w2, w1) < 1e-6 and rel_err(g2, g1) < 1e-6
+    if tile_rows:
+        mt = (tm1.numel() - 1) // 2
+        n = int(tm1[2 * mt])
+        assert int(tm2[2 * mt]) == n and torch.equal(tm1[:n], tm2[:n]) and torch.equal(tm1[mt:mt + n], tm2[mt:mt + n])
+
+
 def grouped_reference(a, w, offsets, rows, gate_up):
     a, w = a.double().cpu(), w.double().cpu()
     E = w.shape[0]

@@ -132,7 +132,8 @@ def test_dense_mlp_part(dtype, tol):
 @pytest.mark.parametrize("H,E,k,mi,si,renorm,gated", [(64, 4, 2, 32, 64, False, True), (96, 8, 3, 48, 80, True, True),
                                                       (72, 5, 1, 40, 0, False, True), (64, 6, 6, 32, 48, True, False),
                                                       (64, 1, 1, 32, 0, False, True)])
-def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated):
+@pytest.mark.parametrize("T", [29, 7])  # 7: the few-token path (experts and shared expert in one launch)
+def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated, T):
     from inferx_amd.config import PartSpec
     from inferx_amd.engine.runtime import Runtime
     from inferx_amd.parts import build_part
@@ -142,7 +143,6 @@ def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated):
         "shared_gated": gated, "renormalize": renorm, "init_std": 0.15}))
     w = tensors_for(part, rt, seed=8)
     part.bind({n: v.to(DEV) for n, v in w.items()}, rt)
-    T = 29
     ctx, _ = make_ctx(rt, [T], [T], 16, 4)
     x = torch.randn(T, H, generator=torch.Generator().manual_seed(9)).to(rt.dtype)
     wd = {"m." + n: v.double() for n, v in w.items()}
