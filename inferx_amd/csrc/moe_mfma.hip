@@ -141,9 +141,10 @@ moe_grouped_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__
   grouped_body<MT, GATE_UP, KSPLIT>(a, w, out, rows, e, tile_row0[blockIdx.y], offsets[e + 1], n0, n_out, width, red);
 }
 
-// Routed experts and the shared expert in one launch (decoding: every launch saved counts).  Workgroups
-// [0, n16_e * max_tiles) serve the routed experts' row tiles, the rest the shared expert, which is one more
-// "expert" over all `shared_rows` tokens with weights and sizes of its own.
+// Routed experts and the shared expert in one launch (decoding: every launch saved counts).  The first
+// n16_s * shared_tiles workgroups serve the shared expert, which is one more "expert" over all `shared_rows`
+// tokens with weights and sizes of its own (first, because its reduction may be the longer one and the last
+// workgroups to start set the kernel's end); the rest serve the routed experts' row tiles.
 template <int MT, bool GATE_UP>
 __global__ void __launch_bounds__(256)
 moe_grouped_dual_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w, __bf16* __restrict__ out,
@@ -153,20 +154,21 @@ moe_grouped_dual_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__
                         const __bf16* __restrict__ a_s, const __bf16* __restrict__ w_s, __bf16* __restrict__ out_s,
                         int shared_rows, int n_out_s, int width_s) {
   __shared__ float red[3 * 64 * MT * (GATE_UP ? 2 : 1) * 4];
-  const int n16_e = (n_out + 15) / 16;
+  const int n16_s = (n_out_s + 15) / 16;
+  const int shared_blocks = n16_s * ((shared_rows + 16 * MT - 1) / (16 * MT));
   int idx = blockIdx.x;
-  if (idx < n16_e * max_tiles) {
+  if (idx < shared_blocks) {
+    const int tile = idx / n16_s;
+    grouped_body<MT, GATE_UP, 4>(a_s, w_s, out_s, nullptr, 0, tile * 16 * MT, shared_rows, (idx - tile * n16_s) * 16,
+                                 n_out_s, width_s, red);
+  } else {
+    idx -= shared_blocks;
+    const int n16_e = (n_out + 15) / 16;
     const int tile = idx / n16_e;
     if (tile >= tile_info[0]) return;
     const int e = tile_expert[tile];
     grouped_body<MT, GATE_UP, 4>(a, w, out, rows, e, tile_row0[tile], offsets[e + 1], (idx - tile * n16_e) * 16, n_out,
                                  width, red);
-  } else {
-    idx -= n16_e * max_tiles;
-    const int n16_s = (n_out_s + 15) / 16;
-    const int tile = idx / n16_s;
-    grouped_body<MT, GATE_UP, 4>(a_s, w_s, out_s, nullptr, 0, tile * 16 * MT, shared_rows, (idx - tile * n16_s) * 16,
-                                 n_out_s, width_s, red);
   }
 }
 

@@ -215,3 +215,55 @@ extern "C" int ix_apply_penalties(float* logits, const int32_t* hist_begin, cons
                      presence, frequency, repetition, mask_begin, mask_ids, vocab);
   return ix_check_launch("ix_apply_penalties");
 }
+
+// ---------------------------------------------------------------------------
+// Greedy choice over a large vocabulary in two stages, so that a handful of rows still fills the machine:
+// every workgroup finds the first maximum of one chunk of one row, a second kernel picks among the chunks
+// (chunks ascend, ties go to the lower index: the result equals ix_argmax's).
+#define ARGMAX_CHUNK 4096
+__global__ void __launch_bounds__(256)
+argmax_chunks_kernel(const float* __restrict__ logits, float* __restrict__ part_v, int32_t* __restrict__ part_i,
+                     int64_t vocab, int chunks) {
+  __shared__ ArgPair red[16];
+  const int64_t r = blockIdx.x;
+  const int c = blockIdx.y;
+  const float* row = logits + r * vocab;
+  const int64_t b = static_cast<int64_t>(c) * ARGMAX_CHUNK, e = min<int64_t>(b + ARGMAX_CHUNK, vocab);
+  ArgPair p{-INFINITY, 0x7fffffff};
+  for (int64_t i = b + threadIdx.x; i < e; i += blockDim.x) {
+    const float v = row[i];
+    if (v > p.v) { p.v = v; p.i = (int)i; }
+  }
+  p = block_argmax(p, red);
+  if (threadIdx.x == 0) {
+    part_v[r * chunks + c] = p.v;
+    part_i[r * chunks + c] = p.i;
+  }
+}
+
+__global__ void __launch_bounds__(256)
+argmax_final_kernel(const float* __restrict__ part_v, const int32_t* __restrict__ part_i, int32_t* __restrict__ out,
+                    int64_t vocab, int chunks) {
+  __shared__ ArgPair red[16];
+  const int64_t r = blockIdx.x;
+  ArgPair p{-INFINITY, 0x7fffffff};
+  for (int c = threadIdx.x; c < chunks; c += blockDim.x) {
+    ArgPair o{part_v[r * chunks + c], part_i[r * chunks + c]};
+    p = better(p, o);
+  }
+  p = block_argmax(p, red);
+  if (threadIdx.x == 0) out[r] = (p.i >= 0 && p.i < vocab) ? p.i : 0;
+}
+
+// part_v / part_i: scratch with rows * ceil(vocab / 4096) entries each.
+extern "C" int ix_argmax_two_stage(const float* logits, int32_t* out, float* part_v, int32_t* part_i, int64_t rows,
+                                   int64_t vocab, hipStream_t stream) {
+  IX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "sizes must be positive");
+  if (rows == 0) return 0;
+  const int chunks = static_cast<int>((vocab + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK);
+  IX_REQUIRE(chunks <= 65535, "vocabulary too large");
+  hipLaunchKernelGGL(argmax_chunks_kernel, dim3(rows, chunks), dim3(256), 0, stream, logits, part_v, part_i, vocab,
+                     chunks);
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, stream, part_v, part_i, out, vocab, chunks);
+  return ix_check_launch("ix_argmax_two_stage");
+}

@@ -434,6 +434,12 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
     R, V = logits.shape
     _need(logits.dtype == torch.float32, "logits must be float32")
     _is_i32(out, R)
+    if V > 4 * 4096 and R < 256:  # few long rows: two stages, so that they still fill the machine
+        chunks = -(-V // 4096)
+        part_v = torch.empty((R, chunks), dtype=torch.float32, device=logits.device)
+        part_i = torch.empty((R, chunks), dtype=torch.int32, device=logits.device)
+        _call("ix_argmax_two_stage", _ptr(logits), _ptr(out), _ptr(part_v), _ptr(part_i), _i64(R), _i64(V), _stream())
+        return
     _call("ix_argmax", _ptr(logits), _ptr(out), _i64(R), _i64(V), _stream())
 
 
