@@ -1,0 +1,139 @@
+// Decoding (at most 16 tokens): the fused q/k/v product with its epilogue in one kernel, bfloat16:
+//   qkv = x . Wqkv^T + bias;  rotate q and k (half-split pairs);  q -> q_out,  k, v -> cache pages.
+// What moe_mfma.hip's streaming kernel and elementwise.hip's qkv_rope_append do one after the other
+// (reference: src/model/qwen2.cc:920-969), with one launch less.
+//
+// A workgroup owns, for one head, 16 features of the low half and the 16 of the high half that pair
+// with them; its four wavefronts split the reduction and add up through LDS in a fixed order.  The
+// product is formed transposed (A = weight rows, B = token rows), so lane l ends up with features
+// 4*(l/16)+i of token l%16: four consecutive numbers of one output row.
+#include "common.h"
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(256)
+qkv_rope_skinny_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ w, const void* __restrict__ bias,
+                       int bias_dtype, const float2* __restrict__ cs, const int32_t* __restrict__ slots,
+                       __bf16* __restrict__ q_out, __bf16* __restrict__ k_cache, __bf16* __restrict__ v_cache,
+                       int tokens, int width, int heads, int kv_heads, int head_dim, int page_size,
+                       int64_t total_slots) {
+  __shared__ float red[3 * 64 * 8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int m = lane & 15, g = lane >> 4;
+  const int half = head_dim / 2, per_head = half / 16;
+  const int head = blockIdx.x / per_head, jt = blockIdx.x - head * per_head;
+  const int row_lo = head * head_dim + 16 * jt + m;  // weight row (= output feature) of the low half
+
+  const int kper = (((width + 3) / 4) + 127) & ~127;
+  const int kbegin = wave * kper, kend = min(width, kbegin + kper);
+  const __bf16* wl = w + static_cast<int64_t>(row_lo) * width;
+  const __bf16* wh = wl + static_cast<int64_t>(half) * width;
+  const __bf16* xr = x + static_cast<int64_t>(min(m, tokens - 1)) * width;
+
+  const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
+                       (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+  f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
+  for (int k0 = kbegin; k0 < kend; k0 += 128) {
+    bf16x8 fl[4], fh[4], fx[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int kk = k0 + 32 * g + 8 * j;
+      const bool ok = kk < kend;
+      fl[j] = ok ? *reinterpret_cast<const bf16x8*>(wl + kk) : zero;
+      fh[j] = ok ? *reinterpret_cast<const bf16x8*>(wh + kk) : zero;
+      fx[j] = ok ? *reinterpret_cast<const bf16x8*>(xr + kk) : zero;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fl[j], fx[j], acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fh[j], fx[j], acc[1], 0, 0, 0);
+    }
+  }
+  if (wave > 0) {
+    float* dst = red + ((wave - 1) * 64 + lane) * 8;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) dst[u * 4 + i] = acc[u][i];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int s = 0; s < 3; ++s) {
+    const float* src = red + (s * 64 + lane) * 8;
+#pragma unroll
+    for (int u = 0; u < 2; ++u)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[u][i] += src[u * 4 + i];
+  }
+
+  // lane holds features j = 16 jt + 4 g + i (low) and j + half (high) of token m
+  const int t = m;
+  if (t >= tokens) return;
+  const int j0 = 16 * jt + 4 * g;
+  const int col = head * head_dim + j0;
+  float lo[4], hi[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    // the product is rounded to bfloat16 before the bias joins it, as when the two kernels run one after the other
+    lo[i] = ix_bf16_to_f32(ix_f32_to_bf16(acc[0][i]));
+    hi[i] = ix_bf16_to_f32(ix_f32_to_bf16(acc[1][i]));
+    if (bias) {
+      lo[i] += ix_load_rt(bias, bias_dtype, col + i);
+      hi[i] += ix_load_rt(bias, bias_dtype, col + half + i);
+    }
+  }
+  const bool is_v = head >= heads + kv_heads;
+  if (!is_v && cs) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float2 c = cs[static_cast<int64_t>(t) * half + j0 + i];
+      const float rlo = lo[i] * c.x - hi[i] * c.y;
+      const float rhi = hi[i] * c.x + lo[i] * c.y;
+      lo[i] = rlo;
+      hi[i] = rhi;
+    }
+  }
+  const int64_t slot = slots ? slots[t] : -1;
+  const bool cache_ok = k_cache != nullptr && slot >= 0 && slot < total_slots;
+  const int64_t page = cache_ok ? slot / page_size : 0;
+  const int off = cache_ok ? static_cast<int>(slot % page_size) : 0;
+  if (is_v) {
+    if (!cache_ok) return;
+    __bf16* dst = v_cache + ((page * kv_heads + (head - heads - kv_heads)) * head_dim + j0) * page_size + off;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      dst[static_cast<int64_t>(i) * page_size] = (__bf16)lo[i];
+      dst[static_cast<int64_t>(half + i) * page_size] = (__bf16)hi[i];
+    }
+    return;
+  }
+  __bf16* dst = nullptr;
+  if (head < heads) dst = q_out + (static_cast<int64_t>(t) * heads + head) * head_dim + j0;
+  else if (cache_ok) dst = k_cache + ((page * kv_heads + (head - heads)) * page_size + off) * head_dim + j0;
+  if (dst) {
+    bf16x4 a = {(__bf16)lo[0], (__bf16)lo[1], (__bf16)lo[2], (__bf16)lo[3]};
+    bf16x4 b = {(__bf16)hi[0], (__bf16)hi[1], (__bf16)hi[2], (__bf16)hi[3]};
+    *reinterpret_cast<bf16x4*>(dst) = a;
+    *reinterpret_cast<bf16x4*>(dst + half) = b;
+  }
+}
+
+// x [tokens <= 16, width], w [(heads + 2 kv_heads) * head_dim, width]; head_dim a multiple of 32, width of 8.
+extern "C" int ix_qkv_rope_skinny(const void* x, const void* w, const void* bias, int bias_dtype, const void* cs,
+                                  const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int tokens,
+                                  int64_t width, int heads, int kv_heads, int head_dim, int page_size,
+                                  int64_t total_slots, hipStream_t stream) {
+  IX_REQUIRE(tokens > 0 && tokens <= 16, "between 1 and 16 tokens");
+  IX_REQUIRE(heads > 0 && kv_heads > 0 && page_size > 0 && width > 0, "sizes must be positive");
+  IX_REQUIRE(head_dim % 32 == 0 && head_dim <= 256, "head_dim must be a multiple of 32 up to 256");
+  IX_REQUIRE(width % 8 == 0 && width < (1 << 30), "the reduction width must be a multiple of 8");
+  IX_REQUIRE((k_cache == nullptr) == (v_cache == nullptr), "give both caches or neither");
+  dim3 grid((heads + 2 * kv_heads) * (head_dim / 32)), block(256);
+  hipLaunchKernelGGL(qkv_rope_skinny_kernel, grid, block, 0, stream, (const __bf16*)x, (const __bf16*)w, bias,
+                     bias_dtype, (const float2*)cs, slots, (__bf16*)q_out, (__bf16*)k_cache, (__bf16*)v_cache, tokens,
+                     (int)width, heads, kv_heads, head_dim, page_size, total_slots);
+  return ix_check_launch("ix_qkv_rope_skinny");
+}

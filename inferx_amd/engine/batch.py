@@ -59,16 +59,19 @@ class StepBatch:
         if T and (self.token_ids.min() < 0 or self.token_ids.max() >= vocab_size):
             bad = self.token_ids[(self.token_ids < 0) | (self.token_ids >= vocab_size)][0]
             raise BatchError(f"token id {int(bad)} is outside the vocabulary of {vocab_size}")
-        for s in range(S):
-            b, e = int(self.q_start[s]), int(self.q_start[s + 1])
-            if e < b:
-                raise BatchError("q_start must not descend")
-            n = e - b
-            first = int(self.seq_lens[s]) - n
-            if first < 0:
-                raise BatchError(f"request {s}: more tokens in the step than in the sequence")
-            if n and (np.any(self.seq_of_token[b:e] != s)
-                      or np.any(self.positions[b:e] != np.arange(first, first + n))):
+        n = self.q_start[1:].astype(np.int64) - self.q_start[:-1]
+        if S and n.min() < 0:
+            raise BatchError("q_start must not descend")
+        first = self.seq_lens.astype(np.int64) - n
+        if S and first.min() < 0:
+            s = int(np.argmax(first < 0))
+            raise BatchError(f"request {s}: more tokens in the step than in the sequence")
+        if T:
+            want_seq = np.repeat(np.arange(S, dtype=np.int64), n)
+            want_pos = np.arange(T, dtype=np.int64) - np.repeat(self.q_start[:-1].astype(np.int64), n) + np.repeat(first, n)
+            bad = (self.seq_of_token != want_seq) | (self.positions != want_pos)
+            if bad.any():
+                s = int(want_seq[int(np.argmax(bad))])
                 raise BatchError(f"request {s}: rows must be grouped, positions contiguous and ending at seq_len - 1")
         if len(self.logits_rows) and (self.logits_rows.min() < 0 or self.logits_rows.max() >= T):
             raise BatchError("logits_rows points outside the step's tokens")

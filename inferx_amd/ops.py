@@ -151,6 +151,36 @@ def qkv_rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: Op
           _i32(kv_heads), _i32(head_dim), _i32(page_size), _i64(total), _stream())
 
 
+def qkv_rope_skinny(x: torch.Tensor, w_qkv: torch.Tensor, bias: Optional[torch.Tensor],
+                    cos_sin: Optional[torch.Tensor], slots: Optional[torch.Tensor], q_out: torch.Tensor,
+                    k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], heads: int, kv_heads: int,
+                    head_dim: int) -> None:
+    """For at most 16 tokens (bfloat16): the q/k/v product, bias, rotation and cache append in one launch."""
+    T, K = x.shape
+    width = (heads + 2 * kv_heads) * head_dim
+    _need(x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and q_out.dtype == torch.bfloat16,
+          "the fused q/k/v kernel is bfloat16 only")
+    _need(w_qkv.shape == (width, K), f"q/k/v weight must be [{width}, {K}]")
+    _need(q_out.numel() == T * heads * head_dim, "q_out mismatch")
+    if bias is not None:
+        _need(bias.numel() == width, "bias length differs")
+    if cos_sin is not None:
+        _need(cos_sin.dtype == torch.float32 and cos_sin.shape == (T, head_dim // 2, 2), "rotary table mismatch")
+    page_size, total = 1, 0
+    if k_cache is not None:
+        _need(v_cache is not None and k_cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16,
+              "cache mismatch")
+        _need(k_cache.dim() == 4 and k_cache.shape[1] == kv_heads and k_cache.shape[3] == head_dim, "cache layout")
+        _need(v_cache.shape == (k_cache.shape[0], kv_heads, head_dim, k_cache.shape[2]), "value cache layout")
+        page_size = k_cache.shape[2]
+        total = k_cache.shape[0] * page_size
+        _need(slots is not None, "slots needed to write the cache")
+        _is_i32(slots, T)
+    _call("ix_qkv_rope_skinny", _ptr(x), _ptr(w_qkv), _ptr(bias), _i32(_dt(bias) if bias is not None else F32),
+          _ptr(cos_sin), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _i32(T), _i64(K), _i32(heads),
+          _i32(kv_heads), _i32(head_dim), _i32(page_size), _i64(total), _stream())
+
+
 def _check_caches(q, k_cache, v_cache):
     d = q.shape[2]
     _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype, "cache dtype differs from q")

@@ -71,13 +71,16 @@ class PagedAttention(Mixer):
     def forward(self, ctx, x, cache):
         rt = ctx.rt
         T = x.shape[0]
-        qkv = rt.linear(x, self.w_qkv)
         table = self.position.prepare(ctx) if self.position is not None else None
         q = rt.empty((T, self.num_heads, self.head_dim))
         writes = cache.writes
-        ops.qkv_rope_append(qkv, self.b_qkv, table, ctx.slots[cache.group] if writes else None, q,
-                            cache.k if writes else None, cache.v if writes else None,
-                            self.num_heads, self.num_kv_heads, self.head_dim)
+        epilogue = (self.b_qkv, table, ctx.slots[cache.group] if writes else None, q, cache.k if writes else None,
+                    cache.v if writes else None, self.num_heads, self.num_kv_heads, self.head_dim)
+        if (T <= 16 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16 and self.head_dim % 32 == 0
+                and self.hidden_size % 8 == 0):
+            ops.qkv_rope_skinny(x, self.w_qkv, *epilogue)  # few tokens: product and epilogue in one launch
+        else:
+            ops.qkv_rope_append(rt.linear(x, self.w_qkv), *epilogue)
         out = rt.empty((T, self.num_heads, self.head_dim))
         self.attend(ctx, q, cache, out)
         return rt.linear(out.view(T, self.q_dim), self.w_out)

@@ -121,6 +121,39 @@ def test_qkv_rope_append(dtype, heads, kv, d, page, bias):
     assert rel_err(q2, x[:, :heads * d].view(T, heads, d)) < tol(dtype)
 
 
+@pytest.mark.parametrize("T,H,heads,kv,d,page,bias", [(1, 64, 4, 2, 32, 16, True), (8, 2048, 16, 16, 128, 16, True),
+                                                       (16, 96, 3, 1, 32, 32, False), (5, 72, 6, 3, 64, 16, True)])
+def test_qkv_rope_skinny_equals_product_then_epilogue(T, H, heads, kv, d, page, bias):
+    """The one-launch q/k/v path for few tokens writes what the product followed by qkv_rope_append writes."""
+    from inferx_amd import ops
+    from inferx_amd.parts.rope import Rotary
+    dt = torch.bfloat16
+    width = (heads + 2 * kv) * d
+    x, w = rnd(T, H, dtype=dt), rnd(width, H, seed=1, dtype=dt, scale=H ** -0.5)
+    b = rnd(width, seed=2, dtype=dt) if bias else None
+    pos = torch.arange(40, 40 + T, dtype=torch.int32, device=DEV)
+    slots = (torch.arange(T, dtype=torch.int32, device=DEV) * 3 + 5)
+    table = torch.empty(T, d // 2, 2, device=DEV)
+    ops.rope_table(table, pos, Rotary(1e6, d).frequencies().to(DEV))
+    pages = 6
+    outs = []
+    for fused in (False, True):
+        q = torch.full((T, heads, d), float("nan"), dtype=dt, device=DEV)
+        kc = torch.zeros(pages, kv, page, d, dtype=dt, device=DEV)
+        vc = torch.zeros(pages, kv, d, page, dtype=dt, device=DEV)
+        if fused:
+            ops.qkv_rope_skinny(x, w, b, table, slots, q, kc, vc, heads, kv, d)
+        else:
+            ops.qkv_rope_append(torch.matmul(x, w.t()), b, table, slots, q, kc, vc, heads, kv, d)
+        outs.append((q, kc, vc))
+    for a, c in zip(outs[0], outs[1]):
+        assert rel_err(c, a) < 1e-2  # the two products round differently in the last bit of bfloat16
+    # and against float64 from the start
+    xd = x.double().cpu() @ w.double().cpu().T + (b.double().cpu() if bias else 0)
+    wq = pm.apply_rope(xd[:, :heads * d].view(T, heads, d), pos.cpu(), 1e6)
+    assert rel_err(outs[1][0], wq) < 1.5e-2
+
+
 def test_argmax_first_maximum():
     # reference vector: tests/unit/host_sampling_test.cc:12-17 ({1, 4, 2} -> 1); ties go to the lowest index
     from inferx_amd import ops
