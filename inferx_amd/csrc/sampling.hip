@@ -267,3 +267,53 @@ extern "C" int ix_argmax_two_stage(const float* logits, int32_t* out, float* par
   hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(256), 0, stream, part_v, part_i, out, vocab, chunks);
   return ix_check_launch("ix_argmax_two_stage");
 }
+
+// ---------------------------------------------------------------------------
+// Log-probabilities of the chosen token and of the `n_top` most probable ones, from the logits as they
+// were sampled from (after penalties and masks): logprob_i = l_i - (max + log sum exp(l - max))
+// (reference: ComputeLogprobsKernel layers.cu:1351-1458; host_sampling.cc:113-141; ties by lower index).
+#define LOGPROB_MAX_TOP 20
+__global__ void __launch_bounds__(SAMPLE_THREADS)
+logprobs_kernel(const float* __restrict__ logits, const int32_t* __restrict__ chosen, float* __restrict__ chosen_lp,
+                int32_t* __restrict__ top_ids, float* __restrict__ top_lp, int64_t vocab, int n_top) {
+  __shared__ ArgPair ared[16];
+  __shared__ float red[16];
+  __shared__ int32_t taken[LOGPROB_MAX_TOP];
+  const int r = blockIdx.x, tid = threadIdx.x;
+  const float* row = logits + static_cast<int64_t>(r) * vocab;
+  float mx = -INFINITY;
+  for (int64_t i = tid; i < vocab; i += SAMPLE_THREADS) mx = fmaxf(mx, row[i]);
+  mx = ix_block_max(mx, red);
+  float s = 0.f;
+  for (int64_t i = tid; i < vocab; i += SAMPLE_THREADS) s += expf(row[i] - mx);
+  s = ix_block_sum(s, red);
+  const float log_z = mx + logf(s);
+  if (tid == 0) chosen_lp[r] = row[chosen[r]] - log_z;
+  for (int n = 0; n < n_top; ++n) {
+    ArgPair p{-INFINITY, 0x7fffffff};
+    for (int64_t i = tid; i < vocab; i += SAMPLE_THREADS) {
+      bool used = false;
+      for (int j = 0; j < n; ++j) used |= (taken[j] == (int)i);
+      const float v = row[i];
+      if (!used && v > p.v) { p.v = v; p.i = (int)i; }
+    }
+    p = block_argmax(p, ared);
+    if (tid == 0) {
+      const int id = (p.i >= 0 && p.i < vocab) ? p.i : 0;
+      taken[n] = id;
+      top_ids[r * n_top + n] = id;
+      top_lp[r * n_top + n] = row[id] - log_z;
+    }
+    __syncthreads();
+  }
+}
+
+extern "C" int ix_logprobs(const float* logits, const int32_t* chosen, float* chosen_lp, int32_t* top_ids,
+                           float* top_lp, int64_t rows, int64_t vocab, int n_top, hipStream_t stream) {
+  IX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "sizes must be positive");
+  IX_REQUIRE(n_top >= 0 && n_top <= LOGPROB_MAX_TOP && n_top <= vocab, "at most 20 top log-probabilities");
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(logprobs_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, chosen, chosen_lp, top_ids,
+                     top_lp, vocab, n_top);
+  return ix_check_launch("ix_logprobs");
+}

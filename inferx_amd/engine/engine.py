@@ -131,7 +131,7 @@ class LLMEngine:
                 s = self.scheduler.sequence(c.rid)
                 rows.append((s.params, s.draws, s.tokens[s.prompt_len:]))
         sampled = self.sampler.sample(logits, rows)
-        self.scheduler.commit_step(sampled)
+        self.scheduler.commit_step(sampled, self.sampler.last_logprobs)
         self.stats.steps += 1
         self.stats.tokens_in += plan.num_tokens
         self.stats.tokens_out += len(sampled)
@@ -158,6 +158,7 @@ class LLMEngine:
         missing = [i for i in ids if i not in done]
         if missing:
             raise RuntimeError(f"requests {missing} never finished")
+        self.last_completions = [done[i] for i in ids]  # with finish reasons and log-probabilities
         if with_reasons:
             return [(done[i].output_tokens, done[i].reason) for i in ids]
         return [done[i].output_tokens for i in ids]

@@ -38,6 +38,7 @@ class Sequence:
     params: SamplingParams
     cancelled: bool = False
     draws: int = 0  # sampled tokens so far: the counter of this request's random stream
+    logprobs: List = field(default_factory=list)  # per generated token, when asked for
 
     def generated(self) -> int:
         return len(self.tokens) - self.prompt_len
@@ -48,6 +49,7 @@ class Completion:
     rid: Hashable
     output_tokens: List[int]
     reason: str
+    logprobs: Optional[List] = None  # per output token (chosen log-probability, [(token, log-probability), ...])
 
 
 @dataclass
@@ -119,7 +121,8 @@ class Scheduler:
         return len(s.tokens) - self.cache.cached(s.rid)
 
     def _retire(self, s: Sequence, reason: str) -> None:
-        self.completed.append(Completion(s.rid, s.tokens[s.prompt_len:], reason))
+        self.completed.append(Completion(s.rid, s.tokens[s.prompt_len:], reason,
+                                         list(s.logprobs) if s.logprobs else None))
         if s.rid in self.cache:
             self.cache.free(s.rid)
 
@@ -215,8 +218,9 @@ class Scheduler:
         self._plan = plan
         return plan
 
-    def commit_step(self, sampled: List[int]) -> None:
-        """`sampled`: one token per contribution that samples, in order."""
+    def commit_step(self, sampled: List[int], logprobs: Optional[List] = None) -> None:
+        """`sampled`: one token per contribution that samples, in order; `logprobs`: what the sampler reported
+        for those rows (or None)."""
         plan, self._plan = self._plan, None
         if plan is None:
             raise RuntimeError("commit_step without prepare_step")
@@ -224,6 +228,7 @@ class Scheduler:
         if len(sampled) != want:
             raise ValueError(f"{len(sampled)} sampled tokens for {want} sampling rows")
         it = iter(sampled)
+        lp_it = iter(logprobs) if logprobs is not None else None
         finished: List[Tuple[Sequence, str]] = []
         by_id = {s.rid: s for s in self.running}
         for c in plan.contributions:
@@ -232,6 +237,9 @@ class Scheduler:
             if not c.samples:
                 continue
             token = int(next(it))
+            lp = next(lp_it) if lp_it is not None else None
+            if lp is not None:
+                s.logprobs.append(lp)
             s.tokens.append(token)
             s.draws += 1
             if token in s.params.stop_tokens and s.generated() > s.params.min_tokens:

@@ -487,6 +487,20 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: torch.Tensor, t
           _ptr(rng_key), _ptr(rng_counter), _i64(R), _i64(V), _stream())
 
 
+def logprobs(logits: torch.Tensor, chosen: torch.Tensor, chosen_lp: torch.Tensor, top_ids: torch.Tensor,
+             top_lp: torch.Tensor) -> None:
+    """Log-probability of each row's chosen token and of its n_top most probable tokens (n_top = top_ids.shape[1])."""
+    R, V = logits.shape
+    n_top = top_ids.shape[1]
+    _need(logits.dtype == torch.float32, "logits must be float32")
+    _is_i32(chosen, R)
+    _need(chosen_lp.dtype == torch.float32 and chosen_lp.numel() >= R, "chosen_lp must be float32 [rows]")
+    _need(top_ids.shape == (R, n_top) and top_ids.dtype == torch.int32, "top_ids must be int32 [rows, n_top]")
+    _need(top_lp.shape == (R, n_top) and top_lp.dtype == torch.float32, "top_lp must be float32 [rows, n_top]")
+    _call("ix_logprobs", _ptr(logits), _ptr(chosen), _ptr(chosen_lp), _ptr(top_ids), _ptr(top_lp), _i64(R), _i64(V),
+          _i32(n_top), _stream())
+
+
 def apply_penalties(logits: torch.Tensor, hist_begin: torch.Tensor, hist_ids: torch.Tensor,
                     hist_counts: torch.Tensor, presence: torch.Tensor, frequency: torch.Tensor,
                     repetition: torch.Tensor, mask_begin: torch.Tensor, mask_ids: torch.Tensor) -> None:

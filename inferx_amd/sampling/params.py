@@ -20,12 +20,16 @@ class SamplingParams:
     min_tokens: int = 0             # stop tokens are masked for the first min_tokens generated tokens
     ignore_eos: bool = False
     seed: int = 0                   # fixes the draws of this request
+    want_logprobs: bool = False     # report the chosen token's log-probability ...
+    top_logprobs: int = 0           # ... and up to this many (at most 20) of the most probable alternatives
 
     def validate(self) -> None:
         if self.max_tokens <= 0:
             raise ValueError("max_tokens must be positive")
         if self.top_k < 0 or not 0.0 < self.top_p or self.min_p < 0 or self.min_p > 1:
             raise ValueError("top_k must be >= 0, top_p > 0 and min_p within [0, 1]")
+        if not 0 <= self.top_logprobs <= 20:
+            raise ValueError("top_logprobs must be between 0 and 20")
         if self.repetition_penalty <= 0:
             raise ValueError("repetition_penalty must be positive")
 

@@ -23,6 +23,8 @@ Row = Tuple[SamplingParams, int, Sequence[int]]
 class Sampler:
     def __init__(self, rt):
         self.rt = rt
+        # after `sample`: per row None, or (log-probability of the chosen token, [(token, log-probability), ...])
+        self.last_logprobs = None
 
     def _dev(self, values, dtype) -> torch.Tensor:
         return torch.tensor(list(values), dtype=dtype).to(self.rt.device)
@@ -65,4 +67,15 @@ class Sampler:
                 self._dev([p.min_p for p, _, _ in rows], torch.float32),
                 self._dev([to_i64(p.seed % (1 << 64)) for p, _, _ in rows], torch.int64),
                 self._dev([n for _, n, _ in rows], torch.int64))
+        self.last_logprobs = None
+        if any(p.want_logprobs or p.top_logprobs for p, _, _ in rows):
+            n_top = max(p.top_logprobs for p, _, _ in rows)
+            chosen_lp = self.rt.empty((R,), torch.float32)
+            top_ids = self.rt.empty((R, n_top), torch.int32)
+            top_lp = self.rt.empty((R, n_top), torch.float32)
+            ops.logprobs(logits, out, chosen_lp, top_ids, top_lp)
+            lp, ids, tlp = chosen_lp.tolist(), top_ids.tolist(), top_lp.tolist()
+            self.last_logprobs = [
+                (lp[r], list(zip(ids[r][:p.top_logprobs], tlp[r][:p.top_logprobs])))
+                if (p.want_logprobs or p.top_logprobs) else None for r, (p, _, _) in enumerate(rows)]
         return out.tolist()

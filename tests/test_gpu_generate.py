@@ -78,6 +78,25 @@ def test_temperature_sampling_is_seeded_and_in_the_support(tmp_path):
     assert other.generate(prompts, SamplingParams(max_tokens=12, temperature=0.7, top_k=6, seed=100)) != runs[0]
 
 
+def test_logprobs_through_the_engine(tmp_path):
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_A, 39, str(tmp_path), "float32")
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    prompt = tiny.random_tokens(11, cfg["vocab_size"], 71)
+    engine = LLMEngine(str(tmp_path), "float32", max_num_seqs=2, max_model_len=64, num_gpu_blocks_override=8)
+    out = engine.generate([prompt], SamplingParams(max_tokens=4, want_logprobs=True, top_logprobs=3))[0]
+    lps = engine.last_completions[0].logprobs
+    assert len(lps) == 4
+    seq = list(prompt)
+    for tok, (lp, top) in zip(out, lps):
+        want = torch.log_softmax(pm.forward(cfg, weights, seq)[-1], -1)
+        assert abs(lp - float(want[tok])) < 1e-4
+        assert [t for t, _ in top] == torch.topk(want, 3).indices.tolist() and top[0][0] == tok  # greedy: chosen = top
+        assert max(abs(v - float(want[t])) for t, v in top) < 1e-4
+        seq.append(tok)
+
+
 def test_preempted_generation_equals_unpreempted(tmp_path):
     """So few pages that running requests are preempted and recomputed: same tokens (reference:
     tests/unit/scheduler_test.cc:742-812)."""

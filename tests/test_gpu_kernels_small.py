@@ -217,6 +217,28 @@ def test_sampling_follows_the_distribution():
     assert float((counts / n - p).abs().max()) < 0.03
 
 
+def test_logprobs():
+    # reference vector: tests/unit/host_sampling_test.cc:55-69 (logits {0, 1, 2}, top 2 -> ids {2, 1})
+    from inferx_amd import ops
+    logits = torch.tensor([[0.0, 1.0, 2.0], [3.0, 3.0, -1.0]], device=DEV)
+    chosen = torch.tensor([2, 1], dtype=torch.int32, device=DEV)
+    lp, ids, tlp = torch.empty(2, device=DEV), torch.empty(2, 2, dtype=torch.int32, device=DEV), torch.empty(2, 2, device=DEV)
+    ops.logprobs(logits, chosen, lp, ids, tlp)
+    log_z = math.log(math.exp(0) + math.exp(1) + math.exp(2))
+    assert abs(float(lp[0]) - (2 - log_z)) < 1e-6
+    assert ids.tolist() == [[2, 1], [0, 1]]  # equal logits: the lower index first
+    assert abs(float(tlp[0, 0]) - (2 - log_z)) < 1e-6 and abs(float(tlp[0, 1]) - (1 - log_z)) < 1e-6
+    big = rnd(3, 151936, seed=9, scale=3.0)
+    chosen = torch.tensor([5, 77777, 151935], dtype=torch.int32, device=DEV)
+    lp, ids, tlp = torch.empty(3, device=DEV), torch.empty(3, 5, dtype=torch.int32, device=DEV), torch.empty(3, 5, device=DEV)
+    ops.logprobs(big, chosen, lp, ids, tlp)
+    want = torch.log_softmax(big.double().cpu(), -1)
+    top = torch.topk(want, 5, dim=-1)
+    assert ids.cpu().long().tolist() == top.indices.tolist()
+    assert float((tlp.cpu().double() - top.values).abs().max()) < 1e-4
+    assert float((lp.cpu().double() - want[torch.arange(3), chosen.cpu().long()]).abs().max()) < 1e-4
+
+
 def test_penalties_and_masks():
     # reference vector: tests/unit/host_sampling_test.cc:19-32 ({5, 4, 3}, presence 3 on id 0, mask on id 1 -> 2)
     from inferx_amd import ops
