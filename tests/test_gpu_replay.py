@@ -58,6 +58,22 @@ def test_whole(folders, name, dtype):
     print(f"whole {name} {dtype}: worst {worst:.2e}")
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_bfloat16_run_keeps_tensors_stored_in_32_bits(folders, name):
+    """A folder stored in float32, run with dtype bfloat16: every tensor stays float32 (activations are
+    bfloat16), so the result is closer to the plain implementation on the float32 weights than bfloat16 weights
+    would allow; and it goes through the kernels' mixed-type paths."""
+    from inferx_amd.engine.runner import ModelRunner
+    runner = ModelRunner.from_directory(folders[(name, "float32")], dtype="bfloat16", page_size=16, num_pages=64,
+                                        max_requests=4, max_seq_len=1024)
+    assert runner.model.embedding.dtype == torch.float32
+    assert runner.model.blocks[-1].mixer.w_qkv.dtype == torch.float32
+    prompts = prompts_for(name)
+    for steps in (ru.whole(prompts), ru.tail_decoded(prompts, 8), ru.mixed(prompts, seed=3)):
+        got = ru.replay(runner, steps)
+        ru.compare(got, expected_for(folders, name, "float32"), ru.BF16_TOL, f"mixed types {name}")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 def test_last_tokens_one_by_one(folders, name, dtype):
