@@ -108,6 +108,16 @@ def route(x: torch.Tensor, w_router: torch.Tensor, top_k: int, renormalize: bool
     return weights, experts
 
 
+def router_margin(x: torch.Tensor, w_router: torch.Tensor, top_k: int) -> torch.Tensor:
+    """Per token, how far the last chosen expert is ahead of the first one left out: (p_k - p_{k+1}) / p_k
+    (1 when every expert is chosen).  A run in reduced precision may legitimately choose the other one where
+    this is tiny; the tests leave such places out of bfloat16 comparisons."""
+    p = torch.softmax(x @ w_router.T, -1).sort(-1, descending=True).values
+    if top_k >= p.shape[-1]:
+        return torch.ones(p.shape[0], dtype=p.dtype)
+    return (p[:, top_k - 1] - p[:, top_k]) / p[:, top_k - 1]
+
+
 def moe_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, num_experts: int, top_k: int,
               renormalize: bool, shared_width: int) -> torch.Tensor:
     """Every chosen expert applied per token and summed in slot order, plus the sigmoid-gated shared expert:
@@ -150,11 +160,13 @@ def window_of_layer(cfg: dict, layer: int) -> int:
 
 def forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequence[int],
             positions: Optional[Sequence[int]] = None,
-            schedule: Optional[List[Tuple[int, Optional[int]]]] = None) -> torch.Tensor:
+            schedule: Optional[List[Tuple[int, Optional[int]]]] = None,
+            margins: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence.  Layer order and the place of every norm and residual:
     src/model/qwen2.cc:902-1066 (embed :902; input norm :912; qkv + bias :920-923; rope :925-926; attention
     :1021-1023; o_proj + residual :1026-1030; post norm :1036; feed-forward :1042-1048; residual :1051; final norm
-    and head :1059-1066).  `schedule`: (layer, cache_from) per execution, default each layer once."""
+    and head :1059-1066).  `schedule`: (layer, cache_from) per execution, default each layer once.
+    `margins`: if a list, the router margin per token of every sparse layer run is appended to it."""
     w = {k: v.to(F64) for k, v in weights.items()}
     H = cfg["hidden_size"]
     heads = cfg["num_attention_heads"]
@@ -189,6 +201,8 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequence[int
         x = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
         m = p + "mlp."
         if is_moe_layer(cfg, layer):
+            if margins is not None:
+                margins.append(router_margin(x, w[m + "gate.weight"], cfg["num_experts_per_tok"]))
             f = moe_block(x, w, m, cfg["num_experts"], cfg["num_experts_per_tok"],
                           bool(cfg.get("norm_topk_prob", False)), cfg.get("shared_expert_intermediate_size", 0))
         else:

@@ -106,8 +106,27 @@ def expected_logits(cfg: dict, weights, prompts: Dict[str, List[int]]) -> Dict[s
     return {rid: plain_model.forward(cfg, weights, toks) for rid, toks in prompts.items()}
 
 
-def compare(got, expected: Dict[str, torch.Tensor], tol: float, what: str = "") -> float:
-    """Largest |difference| relative to the largest |expected logit|; names the first bad place."""
+NEAR_TIE = 5e-3  # relative gap between the last chosen expert's probability and the first one's left out
+
+
+def near_ties(cfg: dict, weights, prompts: Dict[str, List[int]]):
+    """Places where the plain implementation's routing hangs on a gap below NEAR_TIE in some sparse layer.
+    bfloat16 activations put an error of about 6e-4 on a router score here, so there a bfloat16 run may choose the other
+    expert, which changes that token's feed-forward output by far more than rounding; such places are left out
+    of bfloat16 comparisons (never of float32 ones).  The tolerance of all other places stays what it is."""
+    out = set()
+    for rid, toks in prompts.items():
+        margins: List[torch.Tensor] = []
+        plain_model.forward(cfg, weights, toks, margins=margins)
+        if margins:
+            worst = torch.stack(margins).min(0).values
+            out |= {(rid, int(p)) for p in torch.nonzero(worst < NEAR_TIE).flatten()}
+    return out
+
+
+def compare(got, expected: Dict[str, torch.Tensor], tol: float, what: str = "", skip=()) -> float:
+    """Largest |difference| relative to the largest |expected logit|; names the first bad place.
+    Places in `skip` (near ties of the routing, bfloat16 only) must be present and finite, no more."""
     worst = 0.0
     scale = max(float(e.abs().max()) for e in expected.values())
     n = 0
@@ -118,6 +137,8 @@ def compare(got, expected: Dict[str, torch.Tensor], tol: float, what: str = "") 
             row = got[(rid, pos)].double()
             assert torch.isfinite(row).all(), f"{what}: non-finite logits at request {rid} position {pos}"
             err = float((row - exp[pos]).abs().max()) / scale
+            if (rid, pos) in skip:
+                continue
             if err > tol:
                 raise AssertionError(
                     f"{what}: request {rid} position {pos} is the first wrong place: error {err:.3e} of the largest "

@@ -8,7 +8,7 @@ import tiny
 
 pytestmark = pytest.mark.gpu
 
-PROMPT_LENGTHS = {"A": (5, 9, 17, 70), "B": (7, 23, 40, 75), "C": (11, 50)}
+PROMPT_LENGTHS = {"A": (5, 9, 17, 70), "B": (7, 23, 40, 75), "C": (11, 50), "D": (3, 37, 66)}
 
 
 @pytest.fixture(scope="module")
@@ -39,6 +39,21 @@ def expected_for(folders, name, dtype):
     return _expected_cache[key]
 
 
+_ties_cache = {}
+
+
+def ties_for(folders, name, dtype):
+    """Near ties of the routing: left out of bfloat16 comparisons only."""
+    if dtype == "float32":
+        return set()
+    if name not in _ties_cache:
+        cfg, weights = tiny.read_folder(folders[(name, dtype)])
+        _ties_cache[name] = ru.near_ties(cfg, weights, prompts_for(name))
+        total = sum(len(p) for p in prompts_for(name).values())
+        assert len(_ties_cache[name]) < 0.15 * total, "too many near ties for the comparison to mean much"
+    return _ties_cache[name]
+
+
 def make_runner(folders, name, dtype, num_pages=64, page_size=16):
     from inferx_amd.engine.runner import ModelRunner
     return ModelRunner.from_directory(folders[(name, dtype)], dtype=dtype, page_size=page_size, num_pages=num_pages,
@@ -50,11 +65,12 @@ def tol_of(dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_whole(folders, name, dtype):
     runner = make_runner(folders, name, dtype)
     got = ru.replay(runner, ru.whole(prompts_for(name)))
-    worst = ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"whole {name} {dtype}")
+    worst = ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"whole {name} {dtype}",
+                       ties_for(folders, name, dtype))
     print(f"whole {name} {dtype}: worst {worst:.2e}")
 
 
@@ -75,23 +91,25 @@ def test_bfloat16_run_keeps_tensors_stored_in_32_bits(folders, name):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_last_tokens_one_by_one(folders, name, dtype):
     runner = make_runner(folders, name, dtype)
     got = ru.replay(runner, ru.tail_decoded(prompts_for(name), 32))
-    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"tail {name} {dtype}")
+    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"tail {name} {dtype}",
+               ties_for(folders, name, dtype))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_portions_of_changing_size(folders, name, dtype):
     runner = make_runner(folders, name, dtype)
     got = ru.replay(runner, ru.chunked(prompts_for(name)))
-    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"chunked {name} {dtype}")
+    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"chunked {name} {dtype}",
+               ties_for(folders, name, dtype))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_mixed_with_few_pages(folders, name, dtype):
     prompts = prompts_for(name)
     # room for about two of the longer requests: pages are given back and used again
@@ -100,5 +118,6 @@ def test_mixed_with_few_pages(folders, name, dtype):
     used = set()
     steps = ru.mixed(prompts, seed=5, max_tokens=max_tokens)
     got = ru.replay(runner, steps)
-    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"mixed {name} {dtype}")
+    ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"mixed {name} {dtype}",
+               ties_for(folders, name, dtype))
     assert all(p.used_pages == 0 for p in runner.cache.pools)

@@ -34,7 +34,17 @@ CONFIG_C = {
     "qkv_bias": False,
 }
 
-CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C}
+# awkward sizes: nothing is a multiple of 8 where the architecture allows it; the kernels' general paths run
+CONFIG_D = {
+    "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe",
+    "num_hidden_layers": 2, "hidden_size": 100, "num_attention_heads": 5, "num_key_value_heads": 5, "head_dim": 24,
+    "num_experts": 3, "num_experts_per_tok": 2, "moe_intermediate_size": 36, "shared_expert_intermediate_size": 28,
+    "intermediate_size": 52, "decoder_sparse_step": 1, "mlp_only_layers": [0], "norm_topk_prob": True,
+    "vocab_size": 131, "rope_theta": 10000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 256,
+    "use_sliding_window": False, "tie_word_embeddings": False,
+}
+
+CONFIGS = {"A": CONFIG_A, "B": CONFIG_B, "C": CONFIG_C, "D": CONFIG_D}
 
 
 def make_folder(raw_config: dict, seed: int, out_dir: str, dtype: str = "bfloat16", std_scale: float = 1.0) -> str:
