@@ -7,6 +7,9 @@
                 (reference: BlockTable, include/inferx/core/kv_cache.h:158-186;
                 Reserve / ReleaseBlocks, src/scheduler/scheduler.cc:99-111, 170-190)
 
+The bookkeeping itself is C++ (`inferx_amd/csrc/host/cache.cc`, built into
+libinferx_host.so with the host compiler); these classes are its Python face.
+
 A page group is a set of cache-owning layer executions with the same need (kv
 heads, head size, window).  Every group has pages of its own: its own pool, its
 own block list per request.  A group with window W gives a page back as soon as
@@ -20,44 +23,92 @@ their own; the manager hands out slot numbers, the runner owns the memory.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+import ctypes
+from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence
+
+from ..csrc import build as _build
 
 
 class CacheError(RuntimeError):
     """Misuse of the cache manager (unknown request, double free, ...)."""
 
 
+_configured = False
+
+
+def host_lib():
+    """libinferx_host.so with its argument types declared."""
+    global _configured
+    lib = _build.load_host()
+    if not _configured:
+        i32p, i64p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64)
+        vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+        sig = {
+            "ixh_cache_create": (vp, [ci, i32p, i32p, ci, ci, i64]),
+            "ixh_cache_destroy": (None, [vp]),
+            "ixh_cache_error": (ctypes.c_char_p, [vp]),
+            "ixh_cache_max_blocks": (ci, [vp]),
+            "ixh_cache_add": (ci, [vp, i64]),
+            "ixh_cache_free": (ci, [vp, i64]),
+            "ixh_cache_reset": (ci, [vp, i64]),
+            "ixh_cache_reserve": (ci, [vp, i64, i64]),
+            "ixh_cache_commit": (ci, [vp, i64, i64]),
+            "ixh_cache_cached": (i64, [vp, i64]),
+            "ixh_cache_slot": (ci, [vp, i64]),
+            "ixh_cache_contains": (ci, [vp, i64]),
+            "ixh_cache_can_add": (ci, [vp]),
+            "ixh_cache_block_row": (ci, [vp, i64, ci, i32p, ci]),
+            "ixh_cache_slot_index": (i64, [vp, i64, ci, i64]),
+            "ixh_cache_pool_stats": (None, [vp, ci, i32p, i32p]),
+            "ixh_cache_check": (ci, [vp]),
+            "ixh_build_batch": (ci, [vp, ci, i64p, i32p, i32p, i32p, i32p] + [i32p] * 9 + [ctypes.POINTER(ci)]),
+            "ixh_pool_create": (vp, [ci]),
+            "ixh_pool_destroy": (None, [vp]),
+            "ixh_pool_allocate": (ci, [vp]),
+            "ixh_pool_release": (ci, [vp, ci]),
+            "ixh_pool_free_pages": (ci, [vp]),
+        }
+        for name, (res, args) in sig.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _configured = True
+    return lib
+
+
 class PagePool:
+    """A pool on its own."""
+
     def __init__(self, num_pages: int):
         if num_pages <= 0:
             raise CacheError("a page pool needs at least one page")
         self.num_pages = num_pages
-        self._free: List[int] = list(range(num_pages - 1, -1, -1))  # page 0 is handed out first
-        self._is_free = [True] * num_pages
+        self._lib = host_lib()
+        self._h = self._lib.ixh_pool_create(num_pages)
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.ixh_pool_destroy(self._h)
+            self._h = None
 
     @property
     def free_pages(self) -> int:
-        return len(self._free)
+        return self._lib.ixh_pool_free_pages(self._h)
 
     @property
     def used_pages(self) -> int:
-        return self.num_pages - len(self._free)
+        return self.num_pages - self.free_pages
 
     def allocate(self) -> Optional[int]:
-        if not self._free:
-            return None
-        page = self._free.pop()
-        self._is_free[page] = False
-        return page
+        page = self._lib.ixh_pool_allocate(self._h)
+        return None if page < 0 else page
 
     def release(self, page: int) -> None:
-        if not 0 <= page < self.num_pages:
+        rc = self._lib.ixh_pool_release(self._h, int(page))
+        if rc == -1:
             raise CacheError(f"page {page} is outside the pool of {self.num_pages}")
-        if self._is_free[page]:
+        if rc == -2:
             raise CacheError(f"page {page} freed twice")
-        self._is_free[page] = True
-        self._free.append(page)
 
 
 @dataclass(frozen=True)
@@ -67,15 +118,33 @@ class GroupLayout:
     window: int = 0
 
 
-@dataclass
-class _Request:
-    cached: int = 0
-    reserved: int = 0  # tokens that pages have been reserved for (>= cached)
-    slot: int = -1
-    blocks: List[List[int]] = field(default_factory=list)  # per group, by logical page; -1 = given back
+class _PoolView:
+    """What the manager shows of one group's pool."""
+
+    def __init__(self, manager: "CacheManager", group: int):
+        self._m, self._g = manager, group
+
+    def _stats(self):
+        num, free = ctypes.c_int32(), ctypes.c_int32()
+        self._m._lib.ixh_cache_pool_stats(self._m._h, self._g, ctypes.byref(num), ctypes.byref(free))
+        return num.value, free.value
+
+    @property
+    def num_pages(self) -> int:
+        return self._stats()[0]
+
+    @property
+    def free_pages(self) -> int:
+        return self._stats()[1]
+
+    @property
+    def used_pages(self) -> int:
+        num, free = self._stats()
+        return num - free
 
 
 RESERVE_OK, RESERVE_POOL_EMPTY, RESERVE_CONTEXT_FULL = "ok", "pool_empty", "context_full"
+_RESERVE = {0: RESERVE_OK, 1: RESERVE_POOL_EMPTY, 2: RESERVE_CONTEXT_FULL}
 
 
 class CacheManager:
@@ -85,147 +154,109 @@ class CacheManager:
             raise CacheError("page_size, max_requests and max_seq_len must be positive")
         if len(groups) != len(pages_per_group):
             raise CacheError("one page count per group is needed")
+        if any(n <= 0 for n in pages_per_group):
+            raise CacheError("a page pool needs at least one page")
         self.groups = list(groups)
         self.page_size = page_size
         self.max_requests = max_requests
         self.max_seq_len = max_seq_len
         self.max_blocks = -(-max_seq_len // page_size)
-        self.pools = [PagePool(n) for n in pages_per_group]
-        self._free_slots = list(range(max_requests - 1, -1, -1))
-        self._requests: Dict[Hashable, _Request] = {}
+        self._lib = host_lib()
+        G = len(self.groups)
+        windows = (ctypes.c_int32 * max(G, 1))(*[g.window for g in self.groups])
+        pages = (ctypes.c_int32 * max(G, 1))(*pages_per_group)
+        self._h = self._lib.ixh_cache_create(G, windows, pages, page_size, max_requests, max_seq_len)
+        if not self._h:
+            raise CacheError("the cache manager could not be created")
+        self.pools = [_PoolView(self, g) for g in range(G)]
+        self._ids: Dict[Hashable, int] = {}  # request id (any hashable) -> the integer the library knows it by
+        self._next = 0
 
-    # ---- requests -------------------------------------------------------
-    def __contains__(self, rid) -> bool:
-        return rid in self._requests
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.ixh_cache_destroy(self._h)
+            self._h = None
 
-    def live_requests(self):
-        return list(self._requests)
+    def _err(self, rid=None) -> CacheError:
+        msg = self._lib.ixh_cache_error(self._h).decode("utf-8", "replace")
+        return CacheError(f"request {rid!r}: {msg}" if rid is not None else msg)
 
-    def _get(self, rid) -> _Request:
+    def _id(self, rid) -> int:
         try:
-            return self._requests[rid]
+            return self._ids[rid]
         except KeyError:
             raise CacheError(f"unknown request {rid!r}") from None
 
+    # ---- requests -------------------------------------------------------
+    def __contains__(self, rid) -> bool:
+        return rid in self._ids
+
+    def live_requests(self):
+        return list(self._ids)
+
     def can_add(self) -> bool:
-        return bool(self._free_slots)
+        return bool(self._lib.ixh_cache_can_add(self._h))
 
     def add(self, rid) -> int:
         """Start a request: takes a state slot, no pages yet.  Returns the slot."""
-        if rid in self._requests:
+        if rid in self._ids:
             raise CacheError(f"request {rid!r} is already live")
-        if not self._free_slots:
-            raise CacheError(f"all {self.max_requests} request slots are taken")
-        slot = self._free_slots.pop()
-        self._requests[rid] = _Request(slot=slot, blocks=[[] for _ in self.groups])
+        slot = self._lib.ixh_cache_add(self._h, self._next)
+        if slot < 0:
+            raise self._err(rid)
+        self._ids[rid] = self._next
+        self._next += 1
         return slot
 
     def free(self, rid) -> None:
         """End a request: every page and the state slot go back."""
-        req = self._get(rid)
-        self._drop_pages(req)
-        self._free_slots.append(req.slot)
-        del self._requests[rid]
+        if self._lib.ixh_cache_free(self._h, self._id(rid)) != 0:
+            raise self._err(rid)
+        del self._ids[rid]
 
     def reset(self, rid) -> None:
         """Preemption by recomputation: pages go back, the request starts over at
         position 0 and keeps its slot (reference: Preempt, scheduler.cc:206-229)."""
-        req = self._get(rid)
-        self._drop_pages(req)
-        req.cached = req.reserved = 0
-
-    def _drop_pages(self, req: _Request) -> None:
-        for g, blocks in enumerate(req.blocks):
-            for page in blocks:
-                if page >= 0:
-                    self.pools[g].release(page)
-            blocks.clear()
+        if self._lib.ixh_cache_reset(self._h, self._id(rid)) != 0:
+            raise self._err(rid)
 
     # ---- pages ----------------------------------------------------------
     def cached(self, rid) -> int:
-        return self._get(rid).cached
+        return self._lib.ixh_cache_cached(self._h, self._id(rid))
 
     def slot_of(self, rid) -> int:
-        return self._get(rid).slot
-
-    def _first_live_page(self, group: int, cached: int) -> int:
-        w = self.groups[group].window
-        if w <= 0:
-            return 0
-        return max(0, cached + 1 - w) // self.page_size
-
-    def _release_passed(self, req: _Request) -> None:
-        for g, blocks in enumerate(req.blocks):
-            first = min(self._first_live_page(g, req.cached), len(blocks))
-            for j in range(first):
-                if blocks[j] >= 0:
-                    self.pools[g].release(blocks[j])
-                    blocks[j] = -1
-
-    def pages_short(self, rid, new_len: int) -> List[int]:
-        """Per group, how many pages a growth to `new_len` tokens would need beyond what is free."""
-        req = self._get(rid)
-        short = []
-        for g, blocks in enumerate(req.blocks):
-            need = max(0, -(-new_len // self.page_size) - len(blocks))
-            # pages of this request that the window has passed come back first
-            first = min(self._first_live_page(g, req.cached), len(blocks))
-            coming = sum(1 for j in range(first) if blocks[j] >= 0)
-            short.append(max(0, need - self.pools[g].free_pages - coming))
-        return short
+        return self._lib.ixh_cache_slot(self._h, self._id(rid))
 
     def reserve(self, rid, new_len: int) -> str:
         """Make sure pages exist for tokens [0, new_len) (as far as each group's
         window still needs them).  All groups or nothing."""
-        req = self._get(rid)
-        if new_len > self.max_seq_len:
-            return RESERVE_CONTEXT_FULL
-        if new_len <= req.reserved:
-            return RESERVE_OK
-        self._release_passed(req)
-        want_pages = -(-new_len // self.page_size)
-        needs = [max(0, want_pages - len(b)) for b in req.blocks]
-        if any(n > self.pools[g].free_pages for g, n in enumerate(needs)):
-            return RESERVE_POOL_EMPTY
-        for g, n in enumerate(needs):
-            for _ in range(n):
-                req.blocks[g].append(self.pools[g].allocate())
-        req.reserved = new_len
-        return RESERVE_OK
+        rc = self._lib.ixh_cache_reserve(self._h, self._id(rid), int(new_len))
+        if rc < 0:
+            raise self._err(rid)
+        return _RESERVE[rc]
 
     def commit(self, rid, tokens: int) -> None:
         """`tokens` more tokens are now in the cache."""
-        req = self._get(rid)
-        if tokens < 0 or req.cached + tokens > req.reserved:
-            raise CacheError(f"request {rid!r}: commit of {tokens} tokens beyond the {req.reserved} reserved")
-        req.cached += tokens
-        self._release_passed(req)
+        if self._lib.ixh_cache_commit(self._h, self._id(rid), int(tokens)) != 0:
+            raise self._err(rid)
 
     def block_row(self, rid, group: int) -> List[int]:
         """The request's pages in this group by logical page number, -1 where none is held."""
-        return self._get(rid).blocks[group]
+        buf = (ctypes.c_int32 * self.max_blocks)()
+        n = self._lib.ixh_cache_block_row(self._h, self._id(rid), group, buf, self.max_blocks)
+        if n < 0:
+            raise self._err(rid)
+        return list(buf[:n])
 
     def slot_index(self, rid, group: int, position: int) -> int:
         """Flat index page * page_size + offset of the token at `position`."""
-        blocks = self._get(rid).blocks[group]
-        j = position // self.page_size
-        if j >= len(blocks) or blocks[j] < 0:
-            raise CacheError(f"request {rid!r}: no page holds position {position} in group {group}")
-        return blocks[j] * self.page_size + position % self.page_size
+        idx = self._lib.ixh_cache_slot_index(self._h, self._id(rid), group, int(position))
+        if idx < 0:
+            raise self._err(rid)
+        return idx
 
     # ---- invariants (used by tests and by debug runs) ---------------------
     def check(self) -> None:
         """Every page is free or held exactly once; every slot likewise."""
-        for g, pool in enumerate(self.pools):
-            held = [p for r in self._requests.values() for p in r.blocks[g] if p >= 0]
-            if len(held) != len(set(held)):
-                raise CacheError(f"group {g}: a page is held twice")
-            if any(pool._is_free[p] for p in held):
-                raise CacheError(f"group {g}: a held page is on the free list")
-            if len(held) + pool.free_pages != pool.num_pages:
-                raise CacheError(f"group {g}: {pool.num_pages - len(held) - pool.free_pages} pages lost")
-            if len(set(pool._free)) != len(pool._free):
-                raise CacheError(f"group {g}: a page is on the free list twice")
-        slots = [r.slot for r in self._requests.values()]
-        if len(set(slots + self._free_slots)) != self.max_requests or len(slots) + len(self._free_slots) != self.max_requests:
-            raise CacheError("a state slot is lost or held twice")
+        if self._lib.ixh_cache_check(self._h) != 0:
+            raise self._err()

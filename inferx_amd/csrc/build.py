@@ -131,6 +131,73 @@ def build(verbose: bool = True) -> str:
     return lib
 
 
+# ---- the host library (no GPU code): cache manager, batch layout, scheduler ----------------------------
+HOST_DIR = os.path.join(HERE, "host")
+HOST_LIB_NAME = "libinferx_host.so"
+HOST_FLAGS = ["-std=c++17", "-O2", "-fPIC", "-shared", "-Wall"]
+_host_lib: Optional[ctypes.CDLL] = None
+
+
+def host_sources() -> List[str]:
+    return sorted(f for f in os.listdir(HOST_DIR) if f.endswith(".cc"))
+
+
+def _host_digest() -> str:
+    h = hashlib.sha256()
+    for name in sorted(os.listdir(HOST_DIR)):
+        if name.endswith((".cc", ".h")):
+            h.update(name.encode())
+            with open(os.path.join(HOST_DIR, name), "rb") as f:
+                h.update(f.read())
+    h.update(" ".join(HOST_FLAGS).encode())
+    return h.hexdigest()[:16]
+
+
+def find_built_host() -> Optional[str]:
+    want = _host_digest()
+    for d in _build_dirs():
+        lib, stamp = os.path.join(d, HOST_LIB_NAME), os.path.join(d, "host_digest.txt")
+        if os.path.isfile(lib) and os.path.isfile(stamp):
+            with open(stamp) as f:
+                if f.read().strip() == want:
+                    return lib
+    return None
+
+
+def build_host(verbose: bool = True) -> str:
+    """Compile the host sources with the C++ compiler (g++, else hipcc).  Returns the library's path."""
+    cxx = next((c for c in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"))
+                if c and os.path.isfile(c)), None) or _hipcc()
+    out_dir = next((d for d in _build_dirs() if _usable(d)), None)
+    if out_dir is None:
+        raise BuildError("no writable folder for the build: tried " + ", ".join(_build_dirs()))
+    lib = os.path.join(out_dir, HOST_LIB_NAME)
+    tmp = lib + f".tmp{os.getpid()}"
+    t0 = time.time()
+    p = subprocess.run([cxx] + HOST_FLAGS + ["-o", tmp] + [os.path.join(HOST_DIR, s) for s in host_sources()],
+                       capture_output=True, text=True)
+    if p.returncode != 0:
+        raise BuildError(f"{cxx} failed on the host sources:\n{p.stdout}\n{p.stderr}")
+    os.replace(tmp, lib)
+    with open(os.path.join(out_dir, "host_digest.txt"), "w") as f:
+        f.write(_host_digest())
+    if verbose:
+        _say(f"built {lib} in {time.time() - t0:.0f}s")
+    return lib
+
+
+def load_host() -> ctypes.CDLL:
+    """The host library, built first if no current build exists."""
+    global _host_lib
+    if _host_lib is None:
+        path = find_built_host() or build_host()
+        try:
+            _host_lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise BuildError(f"cannot load {path}: {e}") from None
+    return _host_lib
+
+
 def load() -> ctypes.CDLL:
     """The library, built first if no current build exists.  Raises if it cannot be had."""
     global _lib

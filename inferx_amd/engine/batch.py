@@ -13,7 +13,9 @@ from typing import Hashable, List, Sequence, Tuple
 
 import numpy as np
 
-from ..cache.manager import CacheManager, RESERVE_OK
+import ctypes
+
+from ..cache.manager import RESERVE_CONTEXT_FULL, RESERVE_POOL_EMPTY, CacheManager
 
 
 class BatchError(ValueError):
@@ -96,55 +98,38 @@ Entry = Tuple[Hashable, Sequence[int], Sequence[int]]  # request id, its next to
 
 
 def build_step_batch(cache: CacheManager, entries: Sequence[Entry]) -> StepBatch:
-    """Reserve pages for every entry and lay the step out flat.  On a shortage
-    nothing of this step stays reserved beyond what earlier steps held... the
-    caller decides what to do (`OutOfPages`); commit happens after the step ran."""
-    seen = set()
-    for rid, tokens, want in entries:
-        if rid in seen:
-            raise BatchError(f"request {rid!r} appears twice in one step")
-        seen.add(rid)
+    """Reserve pages for every entry and lay the step out flat (done by the host library in one call).  On a
+    shortage `OutOfPages` is raised: entries before the failing one keep what they reserved, nothing was run,
+    and the caller decides what to do.  Commit happens after the step ran."""
+    S = len(entries)
+    G = len(cache.groups)
+    for rid, _, _ in entries:
         if rid not in cache:
             raise BatchError(f"request {rid!r} is not live")
-        for w in want:
-            if not 0 <= w < len(tokens):
-                raise BatchError(f"request {rid!r}: wanted place {w} is outside its {len(tokens)} tokens")
-    for rid, tokens, _ in entries:
-        status = cache.reserve(rid, cache.cached(rid) + len(tokens))
-        if status != RESERVE_OK:
-            raise OutOfPages(rid, status)
-
-    G = len(cache.groups)
-    P = cache.page_size
-    S = len(entries)
-    T = sum(len(tokens) for _, tokens, _ in entries)
-    token_ids = np.zeros(T, np.int32)
-    positions = np.zeros(T, np.int32)
-    seq_of_token = np.zeros(T, np.int32)
-    q_start = np.zeros(S + 1, np.int32)
-    seq_lens = np.zeros(S, np.int32)
-    state_slots = np.zeros(S, np.int32)
-    slots = [np.zeros(T, np.int32) for _ in range(G)]
-    tables = [np.full((S, cache.max_blocks), -1, np.int32) for _ in range(G)]
-    logits_rows: List[int] = []
-    row = 0
-    for s, (rid, tokens, want) in enumerate(entries):
-        n = len(tokens)
-        first = cache.cached(rid)
-        q_start[s] = row
-        seq_lens[s] = first + n
-        state_slots[s] = cache.slot_of(rid)
-        token_ids[row:row + n] = np.asarray(tokens, dtype=np.int64)
-        pos = np.arange(first, first + n, dtype=np.int32)
-        positions[row:row + n] = pos
-        seq_of_token[row:row + n] = s
-        for g in range(G):
-            blocks = np.asarray(cache.block_row(rid, g), dtype=np.int32)
-            tables[g][s, :len(blocks)] = blocks
-            if n:
-                slots[g][row:row + n] = blocks[pos // P] * P + pos % P
-        logits_rows.extend(row + w for w in want)
-        row += n
-    q_start[S] = row
-    return StepBatch(token_ids, positions, seq_of_token, q_start, seq_lens, state_slots,
-                     np.asarray(logits_rows, dtype=np.int32), slots, tables, [e[0] for e in entries])
+    rids = np.fromiter((cache._ids[e[0]] for e in entries), dtype=np.int64, count=S)
+    n_tokens = np.fromiter((len(e[1]) for e in entries), dtype=np.int32, count=S)
+    n_want = np.fromiter((len(e[2]) for e in entries), dtype=np.int32, count=S)
+    T, R = int(n_tokens.sum()), int(n_want.sum())
+    tokens_flat = np.fromiter((t for e in entries for t in e[1]), dtype=np.int64, count=T)
+    if T and (tokens_flat.min() < -(1 << 31) or tokens_flat.max() >= (1 << 31)):
+        raise BatchError("a token id does not fit 32 bits")
+    tokens_flat = tokens_flat.astype(np.int32)
+    want_flat = np.fromiter((w for e in entries for w in e[2]), dtype=np.int32, count=R)
+    token_ids, positions, seq_of_token = (np.empty(T, np.int32) for _ in range(3))
+    q_start, seq_lens, state_slots = np.empty(S + 1, np.int32), np.empty(S, np.int32), np.empty(S, np.int32)
+    logits_rows = np.empty(R, np.int32)
+    slots = np.empty((G, T), np.int32)
+    tables = np.empty((G, S, cache.max_blocks), np.int32)
+    failed = ctypes.c_int(0)
+    p32 = lambda a: a.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+    rc = cache._lib.ixh_build_batch(
+        cache._h, S, rids.ctypes.data_as(ctypes.POINTER(ctypes.c_int64)), p32(n_tokens), p32(tokens_flat),
+        p32(n_want), p32(want_flat), p32(token_ids), p32(positions), p32(seq_of_token), p32(q_start), p32(seq_lens),
+        p32(state_slots), p32(logits_rows), p32(slots), p32(tables), ctypes.byref(failed))
+    if rc != 0:
+        rid = entries[failed.value][0] if 0 <= failed.value < S else None
+        if rc in (1, 2):
+            raise OutOfPages(rid, RESERVE_POOL_EMPTY if rc == 1 else RESERVE_CONTEXT_FULL)
+        raise BatchError(f"request {rid!r} " + cache._lib.ixh_cache_error(cache._h).decode("utf-8", "replace"))
+    return StepBatch(token_ids, positions, seq_of_token, q_start, seq_lens, state_slots, logits_rows,
+                     [slots[g] for g in range(G)], [tables[g] for g in range(G)], [e[0] for e in entries])
