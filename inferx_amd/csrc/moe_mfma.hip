@@ -27,9 +27,9 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // The work of one wavefront (KSPLIT == 1) or workgroup (KSPLIT == 4): rows [row0, row_end) x out-features
 // [n0, n0 + 16) of expert e.  `red`: LDS for the partial sums of a split reduction.
-template <int MT, bool GATE_UP, int KSPLIT>
+template <int MT, bool GATE_UP, int KSPLIT, typename TO = __bf16>
 __device__ __forceinline__ void grouped_body(const __bf16* __restrict__ a, const __bf16* __restrict__ w,
-                                             __bf16* __restrict__ out, const int32_t* __restrict__ rows, int e,
+                                             TO* __restrict__ out, const int32_t* __restrict__ rows, int e,
                                              int row0, int row_end, int n0, int n_out, int width, float* red) {
   constexpr int NACC = GATE_UP ? 2 : 1;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -115,16 +115,30 @@ __device__ __forceinline__ void grouped_body(const __bf16* __restrict__ a, const
       v[i] = acc[0][t][i];
       if (GATE_UP) v[i] = v[i] / (1.0f + __expf(-v[i])) * acc[1][t][i];
     }
-    __bf16* dst = out + static_cast<int64_t>(r) * n_out + nb;
+    TO* dst = out + static_cast<int64_t>(r) * n_out + nb;
     if (nb + 4 <= n_out && (n_out & 3) == 0) {
-      bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-      *reinterpret_cast<bf16x4*>(dst) = o;
+      if constexpr (sizeof(TO) == 4) {
+        *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+      } else {
+        bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+        *reinterpret_cast<bf16x4*>(dst) = o;
+      }
     } else {
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        if (nb + i < n_out) dst[i] = (__bf16)v[i];
+        if (nb + i < n_out) dst[i] = (TO)v[i];
     }
   }
+}
+
+// x [rows <= 16 * MT, width] . w[n_out, width]^T -> float32 [rows, n_out]: the head of a decoding step, whose
+// logits stay float32 (one workgroup per 16 out-features, the reduction split over its four wavefronts).
+template <int MT>
+__global__ void __launch_bounds__(256)
+linear_skinny_f32_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ w, float* __restrict__ out,
+                         int rows, int n_out, int width) {
+  __shared__ float red[3 * 64 * MT * 4];
+  grouped_body<MT, false, 4, float>(x, w, out, nullptr, 0, 0, rows, blockIdx.x * 16, n_out, width, red);
 }
 
 template <int MT, bool GATE_UP, int KSPLIT>
@@ -234,4 +248,23 @@ extern "C" int ix_moe_grouped_dual(const void* a, const void* w, void* out, cons
 #undef PICK
 #undef LAUNCH
   return ix_check_launch("ix_moe_grouped_dual");
+}
+
+// out float32 [rows, n_out] = x [rows, width] . w[n_out, width]^T, rows <= 64, bfloat16 operands.
+extern "C" int ix_linear_skinny_f32(const void* x, const void* w, float* out, int rows, int64_t n_out, int64_t width,
+                                    hipStream_t stream) {
+  IX_REQUIRE(rows > 0 && rows <= 64 && n_out > 0 && width > 0, "between 1 and 64 rows, positive sizes");
+  IX_REQUIRE(width % 8 == 0, "the reduction width must be a multiple of 8");
+  IX_REQUIRE(n_out < (1ll << 31) - 16 && width < (1 << 30), "sizes too large");
+  dim3 grid(static_cast<unsigned>((n_out + 15) / 16)), block(256);
+  if (rows <= 16)
+    hipLaunchKernelGGL(linear_skinny_f32_kernel<1>, grid, block, 0, stream, (const __bf16*)x, (const __bf16*)w, out,
+                       rows, (int)n_out, (int)width);
+  else if (rows <= 32)
+    hipLaunchKernelGGL(linear_skinny_f32_kernel<2>, grid, block, 0, stream, (const __bf16*)x, (const __bf16*)w, out,
+                       rows, (int)n_out, (int)width);
+  else
+    hipLaunchKernelGGL(linear_skinny_f32_kernel<4>, grid, block, 0, stream, (const __bf16*)x, (const __bf16*)w, out,
+                       rows, (int)n_out, (int)width);
+  return ix_check_launch("ix_linear_skinny_f32");
 }

@@ -108,6 +108,11 @@ class Runtime:
         if x.dtype == torch.float32 and w.dtype == torch.float32:
             return torch.matmul(x, w.t())
         if x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+            if self._skinny_ok(x, w):  # few rows: the vocabulary's weights are the traffic
+                from .. import ops
+                out = self.empty((x.shape[0], w.shape[0]), torch.float32)
+                ops.linear_skinny_f32(x, w, out)
+                return out
             if self._mm_out_dtype_ok is not False:
                 try:
                     out = torch.mm(x, w.t(), out_dtype=torch.float32)

@@ -382,6 +382,16 @@ def moe_grouped_dual(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
           _ptr(a_s), _ptr(w_s), _ptr(out_s), _i32(T), _i64(n_out_s), _i64(K_s), _i32(1 if gate_up else 0), _stream())
 
 
+def linear_skinny_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:
+    """out float32 [T, N] = x [T, K] . w[N, K]^T for at most 64 rows, bfloat16 operands (the head of a decode step)."""
+    T, K = x.shape
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype == torch.float32,
+          "bfloat16 operands and a float32 result")
+    _need(w.dim() == 2 and w.shape[1] == K and out.shape == (T, w.shape[0]), "shapes do not fit")
+    _need(0 < T <= 64 and K % 8 == 0, "between 1 and 64 rows and a reduction width that is a multiple of 8")
+    _call("ix_linear_skinny_f32", _ptr(x), _ptr(w), _ptr(out), _i32(T), _i64(w.shape[0]), _i64(K), _stream())
+
+
 def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
                       rows: Optional[torch.Tensor], tile_map: torch.Tensor, gate_up: bool) -> None:
     """Grouped product staged through LDS (bfloat16, many rows per expert); `tile_map` made for tiles of 64 rows."""

@@ -226,6 +226,15 @@ def test_grouped_tiled(T, H, E, k, mi):
         assert rel_err(act, act2) < 1e-2 and rel_err(y, y2) < 1e-2
 
 
+@pytest.mark.parametrize("T,N,K", [(1, 301, 72), (8, 151936, 2048), (16, 384, 96), (33, 1000, 64), (64, 256, 40)])
+def test_linear_skinny_f32(T, N, K):
+    from inferx_amd import ops
+    x, w = rnd(T, K, dtype=torch.bfloat16), rnd(N, K, seed=1, dtype=torch.bfloat16, scale=K ** -0.5)
+    out = torch.full((T, N), float("nan"), device=DEV)
+    ops.linear_skinny_f32(x, w, out)
+    assert rel_err(out, x.double().cpu() @ w.double().cpu().T) < 1e-5  # float32 accumulation of exact products
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_gather_then_combine_is_the_identity(dtype):
     # reference: moe_test.cc:352-411 (weights 0.25 / 0.75)
