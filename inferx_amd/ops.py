@@ -237,6 +237,38 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
           _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(1 if prefetch else 0), _stream())
 
 
+def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                      tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float, window: int,
+                      tile_queries: int = 64, pairs: Optional[torch.Tensor] = None) -> None:
+    """Paged attention for prompt portions (bfloat16, head_dim <= 128): tiles of up to 64 or 128 queries of one
+    request, keys and values shared through LDS.  `tiles` as for attention_mfma.  `pairs` int32 [2, n]: the two
+    tiles that workgroup i takes one after the other (second -1: none); every tile is to be named exactly once
+    (one left out stays unwritten).  Without `pairs` every tile gets a workgroup of its own."""
+    T, heads, d = q.shape
+    _need(q.dtype == torch.bfloat16, "the matrix-core attention kernel is bfloat16 only")
+    _need(out.shape == q.shape and out.dtype == q.dtype, "out mismatch")
+    _check_caches(q, k_cache, v_cache)
+    kv_heads, page_size = k_cache.shape[1], k_cache.shape[2]
+    _need(block_table.dim() == 2, "block table must be [requests, pages]")
+    _is_i32(block_table)
+    _is_i32(positions, T)
+    _is_i32(tiles)
+    _need(tiles.dim() == 2 and tiles.shape[0] == 3 and tiles.is_contiguous(), "tiles must be int32 [3, n_tiles]")
+    n_tiles = tiles.shape[1]
+    if pairs is None:
+        pairs = torch.stack([torch.arange(n_tiles, dtype=torch.int32), torch.full((n_tiles,), -1, dtype=torch.int32)])
+        pairs = pairs.to(q.device)
+    _is_i32(pairs)
+    _need(pairs.dim() == 2 and pairs.shape[0] == 2 and pairs.is_contiguous(), "pairs must be int32 [2, n_pairs]")
+    _need(pairs.shape[1] <= n_tiles <= 2 * pairs.shape[1], "pairs must name every tile once")
+    _need(page_size & (page_size - 1) == 0, "this kernel takes pages of a power of two of keys")
+    _call("ix_attention_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
+          _ptr(tiles[1]), _ptr(tiles[2]), _ptr(pairs[0]), _ptr(pairs[1]), _i32(pairs.shape[1]), _ptr(positions),
+          _ptr(out), _i32(n_tiles), _i32(tile_queries),
+          _i32(heads), _i32(kv_heads), _i32(d), _i32(page_size), _i32(block_table.shape[1]), _f32(scale),
+          _i32(window), _stream())
+
+
 ROUTE_SMALL_TOKENS = 128
 
 

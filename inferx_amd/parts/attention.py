@@ -86,9 +86,18 @@ class PagedAttention(Mixer):
         return rt.linear(out.view(T, self.q_dim), self.w_out)
 
     def attend(self, ctx, q, cache, out) -> None:
-        """bfloat16 with pages and heads in multiples of 16: the matrix-core kernel; else the plain one."""
+        """bfloat16 with pages and heads in multiples of 16: a matrix-core kernel (the one that shares keys through
+        LDS when the step is mostly prompt portions, the wavefront-level one otherwise); else the plain one."""
         page_size = cache.k.shape[2]
         if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0:
+            T, S = ctx.num_tokens, ctx.num_requests
+            if (self.head_dim <= 128 and page_size & (page_size - 1) == 0 and T >= PREFILL_MIN_TOKENS
+                    and T >= PREFILL_MIN_ROWS * S):
+                tile = 128 if T * self.num_heads >= PREFILL_LARGE_TILE_UNITS else 64
+                tiles, pairs = paired_tiles(ctx, tile, self.window)
+                ops.attention_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, out,
+                                      self.scale, self.window, tile, pairs)
+                return
             tiles, tile, n_splits = query_tiles(ctx, self.window, self.num_heads, self.head_dim)
             work = None
             if n_splits > 1:
@@ -106,17 +115,15 @@ LARGE_QUERY_TILE = 32    # ... or 32 when the step brings many tokens (keys and 
 LARGE_TILE_TOKENS = 1 << 30  # measured: no faster than tiles of 16 on MI355X, so off
 WAVES_WANTED = 4096      # enough wavefronts to fill 256 compute units
 MIN_KEYS_PER_SPLIT = 128
+PREFILL_MIN_TOKENS = 128  # the LDS-sharing kernel: steps of at least this many tokens ...
+PREFILL_MIN_ROWS = 16     # ... and this many per request on average (a workgroup per 64 or 128 queries of a request)
+PREFILL_LARGE_TILE_UNITS = 1 << 30  # tokens x heads from which a workgroup takes 128 queries
 
 
-def query_tiles(ctx, window: int, heads: int, head_dim: int = 128):
-    """Tiles of consecutive queries per request (int32 [3, n]: request, first row, rows) on the device, the tile
-    size (16 or 32) and into how many slices each tile's keys are cut.  Planned on the host from the step's
-    batch, once per step; a captured step finds its (static) plan already in `ctx.memo`."""
-    tile = LARGE_QUERY_TILE if (ctx.num_tokens >= LARGE_TILE_TOKENS and head_dim <= 128) else QUERY_TILE
-    key = ("attention_tiles", window, heads, tile)
-    hit = ctx.memo.get(key)
-    if hit is not None:
-        return hit
+def plan_tiles(ctx, tile: int):
+    """Tiles of up to `tile` consecutive queries per request (int32 [3, n]: request, first row, rows) on the
+    device, their number, and the longest context.  Planned on the host from the step's batch, once per step; a
+    captured step finds its (static) plan already in `ctx.memo`."""
     base = ctx.memo.get(("attention_tiles_host", tile))
     if base is None:
         b = ctx.host
@@ -130,9 +137,48 @@ def query_tiles(ctx, window: int, heads: int, head_dim: int = 128):
         tiles_dev = torch.from_numpy(np.ascontiguousarray(tiles_host)).to(ctx.rt.device)
         longest = int(b.seq_lens.max()) if len(b.seq_lens) else 0
         base = ctx.memo[("attention_tiles_host", tile)] = (tiles_dev, tiles_host.shape[1], longest)
-    tiles_dev, n_tiles, longest = base
+        ctx.memo[("attention_tiles_np", tile)] = tiles_host
+    return base
+
+
+def paired_tiles(ctx, tile: int, window: int):
+    """The LDS-sharing kernel's plan: tiles (see plan_tiles) and, int32 [2, n_pairs] on the device, which two
+    tiles each workgroup takes.  A tile's work grows with the keys it reads (all up to its last query, or a
+    window of them), so the tile that reads most is paired with the one that reads least, and so on inwards:
+    workgroups then take about equally long.  Pairs are ordered by falling work."""
+    key = ("attention_pairs", tile, window)
+    hit = ctx.memo.get(key)
+    if hit is not None:
+        return hit
+    tiles_dev, n_tiles, _ = plan_tiles(ctx, tile)
+    t = ctx.memo[("attention_tiles_np", tile)].astype(np.int64)
+    b = ctx.host
+    new = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
+    first_row = t[1] - b.q_start[:-1].astype(np.int64)[t[0]]           # the tile's first query within its portion
+    end = b.seq_lens.astype(np.int64)[t[0]] - new[t[0]] + first_row + t[2]  # one past the last key it reads
+    start = np.maximum(0, end - t[2] + 1 - window) if window > 0 else np.zeros_like(end)
+    work = -(-(end - (start // 64) * 64) // 64)  # rounds of 64 keys
+    order = np.argsort(-work, kind="stable")
+    half = (n_tiles + 1) // 2
+    pairs = np.full((2, half), -1, dtype=np.int32)
+    pairs[0] = order[:half]
+    pairs[1, :n_tiles - half] = order[::-1][:n_tiles - half]
+    ctx.memo[key] = (tiles_dev, torch.from_numpy(pairs).to(ctx.rt.device))
+    return ctx.memo[key]
+
+
+def query_tiles(ctx, window: int, heads: int, head_dim: int = 128):
+    """The wavefront-level kernel's plan: tiles (see plan_tiles), the tile size (16 or 32) and into how many
+    slices each tile's keys are cut."""
+    tile = LARGE_QUERY_TILE if (ctx.num_tokens >= LARGE_TILE_TOKENS and head_dim <= 128) else QUERY_TILE
+    key = ("attention_tiles", window, heads, tile)
+    hit = ctx.memo.get(key)
+    if hit is not None:
+        return hit
+    tiles_dev, n_tiles, longest = plan_tiles(ctx, tile)
     span = min(longest, window + tile + 32) if window > 0 else longest
-    n_splits = max(1, min(WAVES_WANTED // max(1, n_tiles * heads), -(-span // MIN_KEYS_PER_SPLIT), 64))
+    units = n_tiles * heads
+    n_splits = 1 if units >= 2048 else max(1, min(WAVES_WANTED // max(1, units), -(-span // MIN_KEYS_PER_SPLIT), 64))
     n_splits = 1 << (n_splits.bit_length() - 1)  # a power of two: few distinct values, few captured graphs
     ctx.memo[key] = (tiles_dev, tile, n_splits)
     return ctx.memo[key]

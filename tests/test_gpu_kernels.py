@@ -130,6 +130,60 @@ def test_attention_mfma(case, n_splits, tile):
           f"attention_mfma splits={n_splits} tile={tile}")
 
 
+PREFILL_CASES = ATTN_CASES + [
+    ([1500], [1500], 5, 1, 128, 16, 0),                   # many tiles of one request
+    ([777, 300], [130, 300], 4, 2, 112, 16, 0),           # a portion that starts off a tile's edge; odd head blocks
+    ([900, 450], [500, 450], 2, 2, 96, 32, 70),           # window shorter than a workgroup's queries
+]
+
+
+def outside_in_pairs(n_tiles):
+    """Tile i with tile n - 1 - i (the middle one alone): two tiles per workgroup, of different requests and lengths."""
+    half = (n_tiles + 1) // 2
+    second = [n_tiles - 1 - i if n_tiles - 1 - i >= half else -1 for i in range(half)]
+    return torch.tensor([list(range(half)), second], dtype=torch.int32).to(DEV)
+
+
+@pytest.mark.parametrize("paired", [False, True])
+@pytest.mark.parametrize("tile", [64, 128])
+@pytest.mark.parametrize("case", PREFILL_CASES)
+def test_attention_prefill(case, tile, paired):
+    """The kernel whose wavefronts share keys through LDS, against float64 attention per request."""
+    from inferx_amd import ops
+    seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, torch.bfloat16, seed=6)
+    out = torch.full_like(p["q"], float("nan"))
+    scale = d ** -0.5
+    tiles = tiles_for(q_lens, tile)
+    ops.attention_prefill(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles, p["positions"],
+                          out, scale, window, tile, outside_in_pairs(tiles.shape[1]) if paired else None)
+    close(out, attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window), TOL[torch.bfloat16],
+          f"attention_prefill tile={tile}")
+
+
+@pytest.mark.parametrize("tile", [64, 128])
+def test_attention_prefill_finds_far_keys(tile):
+    """Each of a few queries of a long portion matches one key far before it: its output must be that key's value
+    (a tile staged from the wrong page, a wrong causal bound of a wavefront or a stale LDS buffer would miss)."""
+    from inferx_amd import ops
+    L, n, d, heads = 1200, 500, 64, 2
+    p = build_paged([L], [n], heads, heads, d, 16, torch.bfloat16, seed=9)
+    k, v = p["dense"][0]
+    q = p["qs"][0]
+    pairs = [(0, 0), (63, 640), (64, 63), (130, 829), (257, 700), (499, 1199), (300, 1000)]  # (query row, key)
+    for row, far in pairs:
+        assert far <= L - n + row
+        page, off = int(p["table"][0, far // 16]), far % 16
+        p["k_cache"][page, :, off, :] = (q[row] * 6.0).to(DEV)
+        k[far] = q[row] * 6.0
+    out = torch.empty_like(p["q"])
+    ops.attention_prefill(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for([n], tile), p["positions"], out,
+                          d ** -0.5, 0, tile)
+    close(out, attention_reference(p, [L], [n], heads, heads, d ** -0.5, 0), TOL[torch.bfloat16], "far keys")
+    for row, far in pairs:
+        assert float((out[row].float().cpu() - v[far].float()).abs().max()) < 0.05 * float(v[far].abs().max())
+
+
 def test_attention_finds_one_far_key():
     """One key among 2,000 matches the query: the output must be that key's value (a skipped page, a wrong
     split boundary or a wrong table entry would miss it)."""
