@@ -1,16 +1,21 @@
 // Paged attention for prompt portions (bfloat16): the four wavefronts of a
 // workgroup share each tile of keys and values through LDS.
 //
-// A workgroup owns up to 64 * QT consecutive queries of one request and one
-// query head (wavefront w: queries 16*QT*w ..), and walks that tile's keys
-// [lo, hi) 64 at a time.  Keys are staged as [64][D] rows, values as [D][64]
-// (they are stored transposed within a page), each padded so that the sixteen
-// 16-byte operand reads of a quarter wavefront fall on distinct banks.  The
-// next tile's global loads are issued into registers before the current tile
-// is multiplied.  Arithmetic, masking and the operand mapping are those of the
-// wavefront-level kernel in attention_mfma.hip (S^T = K Q^T, O^T += V^T P^T
-// with v_mfma_f32_16x16x32_bf16, a lane ending up with eight consecutive keys
-// of one query), which remains the kernel for decoding and for small steps.
+// A workgroup owns up to 64 consecutive queries of one request and one query
+// head (wavefront w: queries 16 w ..), and walks that tile's keys [lo, hi) 64
+// at a time.  Keys are staged as [64][128] rows whose 16-byte pieces are
+// permuted, values as [D][64 + 8] (they are stored transposed within a page),
+// so that the sixteen 16-byte operand reads of a quarter wavefront fall on
+// distinct banks.  Tiles are double-buffered: a tile's global loads are issued
+// two rounds ahead into registers and written to LDS one round ahead.
+// Arithmetic, masking and the operand mapping are those of the wavefront-level
+// kernel in attention_mfma.hip (S^T = K Q^T, O^T += V^T P^T with
+// v_mfma_f32_16x16x32_bf16, a lane ending up with eight consecutive keys of one
+// query), which remains the kernel for decoding and for small steps.
+//
+// QT is the number of sixteens of queries per wavefront.  Only 1 is launched:
+// 2 halves the LDS reads per product but leaves one wavefront per SIMD, and
+// measured slower on MI355X.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -110,12 +115,22 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
   const __bf16* k_head = k_cache + static_cast<int64_t>(kvh) * page_size * D;
   const __bf16* v_head = v_cache + static_cast<int64_t>(kvh) * page_size * D;
   const int last_page = (hi - 1) >> page_shift;
-  int64_t k_at[GROUPS], v_at[GROUPS];  // where each group of the tile to fetch next starts (uniform)
+  // The table entries of a tile's groups are asked for one round before they are used, with vector loads (every
+  // lane the same address): a scalar load would share its counter with the LDS reads of the round and be waited
+  // for at the first of them.
+  int pages[GROUPS];
+  int vzero = 0;
+  asm volatile("" : "+v"(vzero));  // zero in a vector register that the compiler takes for any number
+  auto ask_pages = [&](int kb) {
+#pragma unroll
+    for (int j = 0; j < GROUPS; ++j) pages[j] = table[min((kb + 16 * j) >> page_shift, last_page) + vzero];
+  };
+  int64_t k_at[GROUPS], v_at[GROUPS];  // where each group of the tile to fetch starts (uniform)
   auto locate = [&](int kb) {
 #pragma unroll
     for (int j = 0; j < GROUPS; ++j) {
-      const int key = kb + 16 * j, off = key & (page_size - 1);
-      const int64_t page = max(table[min(key >> page_shift, last_page)], 0);
+      const int off = (kb + 16 * j) & (page_size - 1);
+      const int64_t page = max(__builtin_amdgcn_readfirstlane(pages[j]), 0);
       k_at[j] = page * page_elems + off * D;
       v_at[j] = page * page_elems + off;
     }
@@ -147,13 +162,15 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
 
   // a tile has at least one query, so kb0 < hi: the first key tile is staged without a condition (the wait for
   // it also covers the loads of the queries above, which the loop then need not wait for again)
+  ask_pages(kb0);
   locate(kb0);
   fetch();
-  locate(kb0 + PF_KEYS);
+  ask_pages(kb0 + PF_KEYS);
   stage(0);
   if (kb0 + PF_KEYS < hi) {
+    locate(kb0 + PF_KEYS);
     fetch();
-    locate(kb0 + 2 * PF_KEYS);
+    ask_pages(kb0 + 2 * PF_KEYS);
   }
   __syncthreads();
   const int bp16 = (lane ^ 16) << 2, bp32 = (lane ^ 32) << 2;  // ds_bpermute addresses of the lanes 16 and 32 away
@@ -164,8 +181,9 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
     if (kb + PF_KEYS < hi) {
       stage(buf ^ 1);
       if (kb + 2 * PF_KEYS < hi) {
+        locate(kb + 2 * PF_KEYS);
         fetch();
-        locate(kb + 3 * PF_KEYS);
+        ask_pages(kb + 3 * PF_KEYS);
       }
     }
     const __bf16* ks = k_tiles[buf];
@@ -285,17 +303,14 @@ static void launch_prefill(int tile_queries, dim3 grid, hipStream_t stream, cons
                            int page_size, int max_blocks, float scale_log2, int window) {
   int page_shift = 4;  // log2 of the page size, a power of two (the entry point has checked)
   while ((1 << page_shift) < page_size) ++page_shift;
-  if (tile_queries == 64)
-    hipLaunchKernelGGL((attn_prefill_kernel<NB, 1>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
-                       (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, pair_a, pair_b, positions, (__bf16*)out, heads, kv_heads,
-                       page_size, max_blocks, scale_log2, window, page_shift);
-  else
-    hipLaunchKernelGGL((attn_prefill_kernel<NB, 2>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
-                       (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, pair_a, pair_b, positions, (__bf16*)out, heads, kv_heads,
-                       page_size, max_blocks, scale_log2, window, page_shift);
+  (void)tile_queries;  // 64: the entry point has checked
+  hipLaunchKernelGGL((attn_prefill_kernel<NB, 1>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
+                     (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, pair_a, pair_b, positions, (__bf16*)out, heads, kv_heads,
+                     page_size, max_blocks, scale_log2, window, page_shift);
 }
 
-// Tiles of up to `tile_queries` (64 or 128) consecutive queries of one request; head_dim a multiple of 16 up to 128.
+// Tiles of up to `tile_queries` (64) consecutive queries of one request; head_dim a multiple of 16 up to 128; pages
+// of a power of two (from 16) of keys.
 // Workgroup p (per head) takes tiles pair_a[p] and then pair_b[p] (or none if that is -1); the caller names every
 // tile exactly once (a tile left out stays unwritten).
 extern "C" int ix_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
@@ -308,7 +323,7 @@ extern "C" int ix_attention_prefill(const void* q, const void* k_cache, const vo
   IX_REQUIRE(heads % kv_heads == 0, "heads must be a multiple of kv_heads");
   IX_REQUIRE(head_dim % 16 == 0 && head_dim >= 16 && head_dim <= 128, "head_dim must be a multiple of 16 up to 128");
   IX_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0, "page_size must be a power of two from 16 on");
-  IX_REQUIRE(tile_queries == 64 || tile_queries == 128, "a query tile holds up to 64 or 128 queries");
+  IX_REQUIRE(tile_queries == 64, "a query tile holds up to 64 queries");
   IX_REQUIRE(window >= 0, "window must not be negative");
   IX_REQUIRE(heads <= 65535, "too many heads");
   IX_REQUIRE(n_pairs >= 0 && n_pairs <= n_tiles, "there are at most as many pairs as tiles");

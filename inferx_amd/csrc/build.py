@@ -26,6 +26,10 @@ LIB_NAME = "libinferx_hip.so"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-target-feature", "-Xclang",
          "-packed-fp32-ops", "-Wno-unused-command-line-argument", "-Wno-unknown-attributes"]
 
+# per source: matrix-core accumulators in ordinary vector registers, where a kernel also rescales them with vector
+# instructions between products (the compiler otherwise copies them to and from accumulation registers every time)
+FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -44,6 +48,7 @@ def _digest() -> str:
         with open(os.path.join(HERE, name), "rb") as f:
             h.update(f.read())
     h.update(" ".join(FLAGS).encode())
+    h.update(repr(sorted(FILE_FLAGS.items())).encode())
     return h.hexdigest()[:16]
 
 
@@ -102,7 +107,7 @@ def build(verbose: bool = True) -> str:
 
     def compile_one(name: str):
         obj = os.path.join(out_dir, name[:-4] + ".o")
-        cmd = [hipcc] + FLAGS + ["-c", os.path.join(HERE, name), "-o", obj]
+        cmd = [hipcc] + FLAGS + FILE_FLAGS.get(name, []) + ["-c", os.path.join(HERE, name), "-o", obj]
         p = subprocess.run(cmd, capture_output=True, text=True, env=env)
         return name, obj, p
 

@@ -240,7 +240,7 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float, window: int,
                       tile_queries: int = 64, pairs: Optional[torch.Tensor] = None) -> None:
-    """Paged attention for prompt portions (bfloat16, head_dim <= 128): tiles of up to 64 or 128 queries of one
+    """Paged attention for prompt portions (bfloat16, head_dim <= 128): tiles of up to 64 queries of one
     request, keys and values shared through LDS.  `tiles` as for attention_mfma.  `pairs` int32 [2, n]: the two
     tiles that workgroup i takes one after the other (second -1: none); every tile is to be named exactly once
     (one left out stays unwritten).  Without `pairs` every tile gets a workgroup of its own."""

@@ -93,7 +93,7 @@ class PagedAttention(Mixer):
             T, S = ctx.num_tokens, ctx.num_requests
             if (self.head_dim <= 128 and page_size & (page_size - 1) == 0 and T >= PREFILL_MIN_TOKENS
                     and T >= PREFILL_MIN_ROWS * S):
-                tile = 128 if T * self.num_heads >= PREFILL_LARGE_TILE_UNITS else 64
+                tile = PREFILL_TILE
                 tiles, pairs = paired_tiles(ctx, tile, self.window)
                 ops.attention_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, out,
                                       self.scale, self.window, tile, pairs)
@@ -116,8 +116,8 @@ LARGE_TILE_TOKENS = 1 << 30  # measured: no faster than tiles of 16 on MI355X, s
 WAVES_WANTED = 4096      # enough wavefronts to fill 256 compute units
 MIN_KEYS_PER_SPLIT = 128
 PREFILL_MIN_TOKENS = 128  # the LDS-sharing kernel: steps of at least this many tokens ...
-PREFILL_MIN_ROWS = 16     # ... and this many per request on average (a workgroup per 64 or 128 queries of a request)
-PREFILL_LARGE_TILE_UNITS = 1 << 30  # tokens x heads from which a workgroup takes 128 queries
+PREFILL_MIN_ROWS = 16     # ... and this many per request on average
+PREFILL_TILE = 64         # queries of one request per workgroup of that kernel
 
 
 def plan_tiles(ctx, tile: int):

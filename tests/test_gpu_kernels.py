@@ -145,9 +145,8 @@ def outside_in_pairs(n_tiles):
 
 
 @pytest.mark.parametrize("paired", [False, True])
-@pytest.mark.parametrize("tile", [64, 128])
 @pytest.mark.parametrize("case", PREFILL_CASES)
-def test_attention_prefill(case, tile, paired):
+def test_attention_prefill(case, paired, tile=64):
     """The kernel whose wavefronts share keys through LDS, against float64 attention per request."""
     from inferx_amd import ops
     seq_lens, q_lens, heads, kv_heads, d, page, window = case
@@ -161,8 +160,7 @@ def test_attention_prefill(case, tile, paired):
           f"attention_prefill tile={tile}")
 
 
-@pytest.mark.parametrize("tile", [64, 128])
-def test_attention_prefill_finds_far_keys(tile):
+def test_attention_prefill_finds_far_keys(tile=64):
     """Each of a few queries of a long portion matches one key far before it: its output must be that key's value
     (a tile staged from the wrong page, a wrong causal bound of a wavefront or a stale LDS buffer would miss)."""
     from inferx_amd import ops
