@@ -3,28 +3,34 @@
 // each operand per wavefront, which is right when the weights are the traffic
 // (decoding) and wasteful when dozens of rows share them.
 //
-// A workgroup owns 64 rows of one expert (a row tile of the grouping kernel's
-// map) x 128 weight rows: for the gate|up product 64 gate rows and the 64 up
-// rows that belong to them (64 output columns after SwiGLU), for the down
-// product 128 output columns.  The reduction runs in stages of 64: the next
-// stage's global loads are issued into registers before the current stage is
-// multiplied out of LDS.  LDS rows are padded to 144 bytes so that the sixteen
+// A workgroup owns up to 160 rows of one expert (a row tile of the grouping
+// kernel's map; with a few hundred tokens that is all rows of the expert, so
+// its weights are read once) x 128 weight rows: for the gate|up product 64 gate
+// rows and the 64 up rows that belong to them (64 output columns after SwiGLU),
+// for the down product 128 output columns.  Only the sixteens of rows that the
+// tile really holds are multiplied.  The reduction runs in stages of 64: the
+// next stage's global loads are issued into registers before the current stage
+// is multiplied out of LDS.  LDS rows are padded to 144 bytes so that the
 // 16-byte operand reads of a wavefront quarter fall on distinct banks.
 //
 // As in moe_mfma.hip the product is formed transposed (A = weight rows,
 // B = activation rows), so lane l ends up with four consecutive output
-// columns of one row.  Wavefront w owns weight blocks (w, 4 + w) [gate|up] or
-// (2w, 2w + 1) [down] and all four row blocks.
+// columns of one row.  The four wavefronts are laid out 2 x 2: wavefront
+// (wi, xi) owns 64 of the weight rows (for gate|up: 32 gate rows and their up
+// rows) and every second sixteen of activation rows, so it reads 4 + 5 operand
+// pieces for 20 products.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-#define TL_ROWS 64
+#define TL_ROWS 160   // the row-tile map is made for tiles of this many rows
 #define TL_WROWS 128
 #define TL_K 64
 #define TL_STRIDE 72  // elements per LDS row: 64 + 8 of padding
+#define TL_XPER (TL_ROWS * 8 / 256)  // 16-byte pieces of activations per thread and stage
+#define TL_XBLK (TL_ROWS / 32)       // sixteens of activation rows per wavefront
 
 template <bool GATE_UP>
 __global__ void __launch_bounds__(256)
@@ -37,116 +43,141 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
   if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
+  const int wi = wave & 1, xi = wave >> 1;
   const int e = tile_expert[blockIdx.y];
   const int row0 = tile_row0[blockIdx.y];
   const int row_end = offsets[e + 1];
+  const int nblk = (min(TL_ROWS, row_end - row0) + 15) >> 4;  // sixteens of rows this tile holds
   constexpr int COLS = GATE_UP ? 64 : 128;  // output columns of this workgroup
   const int n0 = blockIdx.x * COLS;
 
-  // what this thread copies per stage: 4 chunks of 8 weights, 2 chunks of 8 activations
+  // what this thread copies per stage: 4 pieces of 8 weights, up to TL_XPER pieces of 8 activations
   const int64_t w_rows = GATE_UP ? 2 * static_cast<int64_t>(n_out) : n_out;
-  const __bf16* wsrc[4];
-  int wdst[4];
+  // (32-bit offsets: the entry point has checked that one expert's weights and the activations stay below 2^31)
+  const __bf16* w_expert = w + static_cast<int64_t>(e) * w_rows * width;
+  int wsrc[4], wdst[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int c = tid + 256 * i, r = c >> 3, kc = (c & 7) * 8;
-    int64_t src_row;
+    int src_row;
     if (GATE_UP)
       src_row = (r < 64 ? 0 : n_out) + min(n0 + (r & 63), n_out - 1);
     else
       src_row = min(n0 + r, n_out - 1);
-    wsrc[i] = w + (static_cast<int64_t>(e) * w_rows + src_row) * width + kc;
+    wsrc[i] = src_row * width + kc;
     wdst[i] = r * TL_STRIDE + kc;
   }
-  const __bf16* xsrc[2];
-  int xdst[2];
+  int xsrc[TL_XPER];
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    const int c = tid + 256 * i, r = c >> 3, kc = (c & 7) * 8;
-    const int gr = min(row0 + r, row_end - 1);
-    xsrc[i] = a + static_cast<int64_t>(rows ? rows[gr] : gr) * width + kc;
-    xdst[i] = r * TL_STRIDE + kc;
+  for (int i = 0; i < TL_XPER; ++i) {
+    const int r = (tid >> 3) + 32 * i;
+    const int gr = min(row0 + r, row_end - 1);  // rows past the end repeat the last one; their results are dropped
+    xsrc[i] = (rows ? rows[gr] : gr) * width + (tid & 7) * 8;
   }
-  const int kc_mine = (tid & 7) * 8;  // the same for all of this thread's chunks
+  const int kc_mine = (tid & 7) * 8;  // the same for all of this thread's pieces
+  const int xdst = (tid >> 3) * TL_STRIDE + kc_mine;
 
   const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
                        (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
-  bf16x8 wreg[4], xreg[2];
-  auto fetch = [&](int k0) {
+  // Two register sets: while stage s is multiplied out of LDS, stage s + 1 is on its way in one set (asked for a
+  // round earlier) and stage s + 2 is asked for into the other, so a load has two rounds to arrive.
+  bf16x8 wreg[2][4], xreg[2][TL_XPER];
+  auto fetch = [&](int k0, bf16x8 (&wr)[4], bf16x8 (&xr)[TL_XPER]) {
     const bool ok = k0 + kc_mine < width;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) wreg[i] = ok ? *reinterpret_cast<const bf16x8*>(wsrc[i] + k0) : zero;
+    for (int i = 0; i < 4; ++i) wr[i] = ok ? *reinterpret_cast<const bf16x8*>(w_expert + wsrc[i] + k0) : zero;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) xreg[i] = ok ? *reinterpret_cast<const bf16x8*>(xsrc[i] + k0) : zero;
+    for (int i = 0; i < TL_XPER; ++i)  // piece i lies in sixteens 2 i and 2 i + 1 (uniform over the workgroup)
+      if (2 * i < nblk) xr[i] = ok ? *reinterpret_cast<const bf16x8*>(a + xsrc[i] + k0) : zero;
   };
-  auto stage = [&]() {
+  auto stage = [&](const bf16x8 (&wr)[4], const bf16x8 (&xr)[TL_XPER]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + wdst[i]) = wreg[i];
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + wdst[i]) = wr[i];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) *reinterpret_cast<bf16x8*>(xs + xdst[i]) = xreg[i];
+    for (int i = 0; i < TL_XPER; ++i)
+      if (2 * i < nblk) *reinterpret_cast<bf16x8*>(xs + xdst + 32 * i * TL_STRIDE) = xr[i];
   };
 
-  const int wblock0 = GATE_UP ? 16 * wave : 32 * wave;
-  const int wblock1 = GATE_UP ? 64 + 16 * wave : 32 * wave + 16;
-  f32x4 acc[2][4];
+  // weight blocks of this wavefront: gate|up 32 wi + {0, 16} and the same + 64; down 64 wi + 16 j
+  int wblock[4];
 #pragma unroll
-  for (int j = 0; j < 2; ++j)
+  for (int j = 0; j < 4; ++j) wblock[j] = GATE_UP ? 32 * wi + 16 * (j & 1) + 64 * (j >> 1) : 64 * wi + 16 * j;
+  f32x4 acc[4][TL_XBLK];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int t = 0; t < TL_XBLK; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  fetch(0);
-  stage();
-  __syncthreads();
-  for (int k0 = 0; k0 < width; k0 += TL_K) {
-    const bool more = k0 + TL_K < width;
-    if (more) fetch(k0 + TL_K);
+  auto multiply = [&]() {
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       const int col = 32 * kk + 8 * g;
-      const bf16x8 wa0 = *reinterpret_cast<const bf16x8*>(ws + (wblock0 + m) * TL_STRIDE + col);
-      const bf16x8 wa1 = *reinterpret_cast<const bf16x8*>(ws + (wblock1 + m) * TL_STRIDE + col);
+      bf16x8 wa[4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xs + (16 * t + m) * TL_STRIDE + col);
-        acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa0, xb, acc[0][t], 0, 0, 0);
-        acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa1, xb, acc[1][t], 0, 0, 0);
+      for (int j = 0; j < 4; ++j) wa[j] = *reinterpret_cast<const bf16x8*>(ws + (wblock[j] + m) * TL_STRIDE + col);
+#pragma unroll
+      for (int t = 0; t < TL_XBLK; ++t) {
+        if (2 * t + xi >= nblk) continue;  // uniform over the wavefront
+        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xs + (16 * (2 * t + xi) + m) * TL_STRIDE + col);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[j], xb, acc[j][t], 0, 0, 0);
       }
     }
+  };
+
+  fetch(0, wreg[0], xreg[0]);
+  stage(wreg[0], xreg[0]);
+  if (TL_K < width) fetch(TL_K, wreg[1], xreg[1]);
+  __syncthreads();
+  // two stages per turn, so that the register sets are named statically
+  for (int k0 = 0; k0 < width; k0 += 2 * TL_K) {
+    if (k0 + 2 * TL_K < width) fetch(k0 + 2 * TL_K, wreg[0], xreg[0]);
+    multiply();  // stage k0
     __syncthreads();
-    if (more) {
-      stage();
+    if (k0 + TL_K >= width) break;
+    stage(wreg[1], xreg[1]);
+    __syncthreads();
+    if (k0 + 3 * TL_K < width) fetch(k0 + 3 * TL_K, wreg[1], xreg[1]);
+    multiply();  // stage k0 + 64
+    __syncthreads();
+    if (k0 + 2 * TL_K < width) {
+      stage(wreg[0], xreg[0]);
       __syncthreads();
     }
   }
 
-  // lane holds weight rows (block) + 4 g + i of activation row row0 + 16 t + m
+  // lane holds weight rows (block) + 4 g + i of activation row row0 + 16 (2 t + xi) + m
+  const bool vec = (n_out & 3) == 0;
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    const int r = row0 + 16 * t + m;
-    if (r >= row_end) continue;
+  for (int t = 0; t < TL_XBLK; ++t) {
+    const int r = row0 + 16 * (2 * t + xi) + m;
+    if (2 * t + xi >= nblk || r >= row_end) continue;
     if (GATE_UP) {
-      const int nb = n0 + 16 * wave + 4 * g;
-      float v[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float gate = acc[0][t][i];
-        v[i] = gate / (1.0f + __expf(-gate)) * acc[1][t][i];
-      }
-      __bf16* dst = out + static_cast<int64_t>(r) * n_out + nb;
-      if (nb + 4 <= n_out && (n_out & 3) == 0) {
-        bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-        *reinterpret_cast<bf16x4*>(dst) = o;
-      } else {
+      for (int j = 0; j < 2; ++j) {
+        const int nb = n0 + 32 * wi + 16 * j + 4 * g;
+        float v[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i)
-          if (nb + i < n_out) dst[i] = (__bf16)v[i];
+        for (int i = 0; i < 4; ++i) {
+          const float gate = acc[j][t][i];
+          v[i] = gate / (1.0f + __expf(-gate)) * acc[2 + j][t][i];
+        }
+        __bf16* dst = out + static_cast<int64_t>(r) * n_out + nb;
+        if (nb + 4 <= n_out && vec) {
+          bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+          *reinterpret_cast<bf16x4*>(dst) = o;
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (nb + i < n_out) dst[i] = (__bf16)v[i];
+        }
       }
     } else {
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        const int nb = n0 + 32 * wave + 16 * j + 4 * g;
+      for (int j = 0; j < 4; ++j) {
+        const int nb = n0 + 64 * wi + 16 * j + 4 * g;
         __bf16* dst = out + static_cast<int64_t>(r) * n_out + nb;
-        if (nb + 4 <= n_out && (n_out & 3) == 0) {
+        if (nb + 4 <= n_out && vec) {
           bf16x4 o = {(__bf16)acc[j][t][0], (__bf16)acc[j][t][1], (__bf16)acc[j][t][2], (__bf16)acc[j][t][3]};
           *reinterpret_cast<bf16x4*>(dst) = o;
         } else {
@@ -159,14 +190,16 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
   }
 }
 
-// The row-tile map must have been made for tiles of 64 rows.
+// The row-tile map must have been made for tiles of TL_ROWS (160) rows.
 extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, const int32_t* offsets,
                                     const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
-                                    const int32_t* tile_info, int max_tiles, int64_t n_out, int64_t width, int gate_up,
-                                    hipStream_t stream) {
+                                    const int32_t* tile_info, int max_tiles, int64_t a_rows, int64_t n_out,
+                                    int64_t width, int gate_up, hipStream_t stream) {
   IX_REQUIRE(n_out > 0 && width > 0 && max_tiles >= 0, "sizes must be positive");
   IX_REQUIRE(width % 8 == 0, "the reduction width must be a multiple of 8 for the matrix-core kernel");
   IX_REQUIRE(n_out < (1 << 30) && width < (1 << 30), "sizes too large");
+  IX_REQUIRE(a_rows >= 0 && a_rows * width < (int64_t(1) << 31) && (gate_up ? 2 : 1) * n_out * width < (int64_t(1) << 31),
+             "the activations, and one expert's weights, must hold fewer than 2^31 numbers");
   IX_REQUIRE(max_tiles <= 65535, "too many row tiles for one launch");
   if (max_tiles == 0) return 0;
   const int cols = gate_up ? 64 : 128;

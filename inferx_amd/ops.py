@@ -424,9 +424,13 @@ def linear_skinny_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> No
     _call("ix_linear_skinny_f32", _ptr(x), _ptr(w), _ptr(out), _i32(T), _i64(w.shape[0]), _i64(K), _stream())
 
 
+MOE_TILED_ROWS = 160  # rows per tile of the LDS-staged grouped product
+
+
 def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
                       rows: Optional[torch.Tensor], tile_map: torch.Tensor, gate_up: bool) -> None:
-    """Grouped product staged through LDS (bfloat16, many rows per expert); `tile_map` made for tiles of 64 rows."""
+    """Grouped product staged through LDS (bfloat16, many rows per expert); `tile_map` made for tiles of
+    MOE_TILED_ROWS rows."""
     E = w.shape[0]
     A, n_out = out.shape
     K = a.shape[1]
@@ -440,10 +444,10 @@ def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offse
         _is_i32(rows, A)
     else:
         _need(a.shape[0] >= A, "a has fewer rows than out")
-    mt = moe_max_tiles(A, E, 64)
+    mt = moe_max_tiles(A, E, MOE_TILED_ROWS)
     _is_i32(tile_map, 2 * mt + 1)
     _call("ix_moe_grouped_tiled", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
-          _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i64(n_out), _i64(K),
+          _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i64(a.shape[0]), _i64(n_out), _i64(K),
           _i32(1 if gate_up else 0), _stream())
 
 

@@ -83,7 +83,7 @@ class MoeFeedForward(FeedForward):
         if not ok:
             return 0
         per_expert = x.shape[0] * self.top_k / self.num_experts
-        return 16 if per_expert <= 16 else (32 if per_expert <= 32 else 64)
+        return 16 if per_expert <= 16 else (32 if per_expert <= 32 else ops.MOE_TILED_ROWS)
 
     def dispatch(self, ctx, topk_e, tile_rows: int = 0):
         rt, A = ctx.rt, topk_e.numel()
@@ -100,7 +100,7 @@ class MoeFeedForward(FeedForward):
         rt, A = ctx.rt, rows.numel()
         act = rt.empty((A, self.expert_width))
         y = rt.empty((A, self.hidden_size))
-        if tile_rows == 64:  # many rows per expert: operands staged through LDS
+        if tile_rows == ops.MOE_TILED_ROWS:  # many rows per expert: operands staged through LDS
             ops.moe_grouped_tiled(x, self.w13, act, offsets, rows, tile_map, True)
             ops.moe_grouped_tiled(act, self.w2, y, offsets, None, tile_map, False)
         elif tile_rows:
