@@ -103,6 +103,28 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   }
 }
 
+// bfloat16 with a width that is a multiple of 8: eight numbers per thread, 16-byte loads and stores
+__global__ void __launch_bounds__(256)
+silu_mul_vec8_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ out, int64_t tokens, int64_t width) {
+  const int64_t per_row = width / 8, n = tokens * per_row;
+  for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < n;
+       p += static_cast<int64_t>(gridDim.x) * blockDim.x) {
+    const int64_t t = p / per_row, c = (p - t * per_row) * 8;
+    const uint4 g4 = *reinterpret_cast<const uint4*>(gu + t * 2 * width + c);
+    const uint4 u4 = *reinterpret_cast<const uint4*>(gu + t * 2 * width + width + c);
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float g0 = __uint_as_float(gw[i] << 16), g1 = __uint_as_float(gw[i] & 0xffff0000u);
+      const float u0 = __uint_as_float(uw[i] << 16), u1 = __uint_as_float(uw[i] & 0xffff0000u);
+      o[i] = ix_f32_to_bf16(g0 / (1.0f + expf(-g0)) * u0) |
+             static_cast<uint32_t>(ix_f32_to_bf16(g1 / (1.0f + expf(-g1)) * u1)) << 16;
+    }
+    *reinterpret_cast<uint4*>(out + t * width + c) = make_uint4(o[0], o[1], o[2], o[3]);
+  }
+}
+
 extern "C" int ix_silu_mul(const void* gu, void* out, int dtype, int64_t tokens, int64_t width, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
   if (tokens == 0) return 0;
@@ -110,7 +132,12 @@ extern "C" int ix_silu_mul(const void* gu, void* out, int dtype, int64_t tokens,
   dim3 grid(static_cast<unsigned>(std::min<int64_t>((n + 255) / 256, 65536))), block(256);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(silu_mul_kernel<float>, grid, block, 0, stream, (const float*)gu, (float*)out, tokens, width);
-  else if (dtype == IX_BF16)
+  else if (dtype == IX_BF16 && width % 8 == 0 &&
+           ((reinterpret_cast<uintptr_t>(gu) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+    dim3 grid8(static_cast<unsigned>(std::min<int64_t>((n / 8 + 255) / 256, 65536)));
+    hipLaunchKernelGGL(silu_mul_vec8_kernel, grid8, block, 0, stream, (const uint16_t*)gu, (uint16_t*)out, tokens,
+                       width);
+  } else if (dtype == IX_BF16)
     hipLaunchKernelGGL(silu_mul_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)gu, (bf16_t*)out, tokens,
                        width);
   else
@@ -211,10 +238,10 @@ qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __rest
                             const float2* __restrict__ cs, const int32_t* __restrict__ slots,
                             uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache,
                             uint16_t* __restrict__ v_cache, int heads, int kv_heads, int head_dim, int page_size,
-                            int64_t total_slots) {
+                            int64_t total_slots, int skip_v) {
   const int64_t t = blockIdx.x;
   const int half = head_dim / 2, per_head = half / 8;
-  const int items = (heads + 2 * kv_heads) * per_head;
+  const int items = (heads + (skip_v ? 1 : 2) * kv_heads) * per_head;  // values may be left to the kernel below
   const int64_t in_width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
   const uint16_t* in = qkv + t * in_width;
   const int64_t slot = slots ? slots[t] : -1;
@@ -286,6 +313,49 @@ qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __rest
   }
 }
 
+// Values of many tokens (bfloat16): the cache keeps them transposed, so a token's values are head_dim separate
+// 2-byte stores.  A workgroup takes 32 tokens of one kv head, turns the tile in LDS and stores with neighbouring
+// lanes on neighbouring tokens: tokens of one request have consecutive slots, so 32 lanes fill 64 contiguous bytes.
+#define V_TILE_TOKENS 32
+__global__ void __launch_bounds__(256)
+v_append_tile_kernel(const uint16_t* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
+                     const int32_t* __restrict__ slots, uint16_t* __restrict__ v_cache, int64_t tokens, int heads,
+                     int kv_heads, int head_dim, int page_size, int64_t total_slots) {
+  extern __shared__ __align__(16) uint16_t v_tile[];  // [32][head_dim + 2]
+  const int stride = head_dim + 2;
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * V_TILE_TOKENS;
+  const int g = blockIdx.y, tid = threadIdx.x;
+  const int64_t in_width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
+  const int col0 = (heads + kv_heads + g) * head_dim;
+  const int pieces = head_dim / 8;
+  for (int item = tid; item < V_TILE_TOKENS * pieces; item += 256) {
+    const int i = item / pieces, d0 = (item - i * pieces) * 8;
+    if (t0 + i >= tokens) continue;
+    const uint4 v4 = *reinterpret_cast<const uint4*>(qkv + (t0 + i) * in_width + col0 + d0);
+    const uint32_t vw[4] = {v4.x, v4.y, v4.z, v4.w};
+    uint32_t* dst = reinterpret_cast<uint32_t*>(v_tile + i * stride + d0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float a = __uint_as_float(vw[j] << 16), b = __uint_as_float(vw[j] & 0xffff0000u);
+      if (bias) {
+        a += ix_load_rt(bias, bias_dtype, col0 + d0 + 2 * j);
+        b += ix_load_rt(bias, bias_dtype, col0 + d0 + 2 * j + 1);
+      }
+      dst[j] = ix_f32_to_bf16(a) | static_cast<uint32_t>(ix_f32_to_bf16(b)) << 16;
+    }
+  }
+  __syncthreads();
+  const int i = tid & (V_TILE_TOKENS - 1);
+  if (t0 + i >= tokens) return;
+  const int64_t slot = slots[t0 + i];
+  if (slot < 0 || slot >= total_slots) return;
+  const int64_t page = slot / page_size;
+  const int off = static_cast<int>(slot % page_size);
+  uint16_t* dst = v_cache + (page * kv_heads + g) * head_dim * page_size + off;
+  for (int d = tid / V_TILE_TOKENS; d < head_dim; d += 256 / V_TILE_TOKENS)
+    dst[static_cast<int64_t>(d) * page_size] = v_tile[i * stride + d];
+}
+
 extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const void* cs,
                                   const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int64_t tokens,
                                   int heads, int kv_heads, int head_dim, int page_size, int64_t total_slots,
@@ -301,11 +371,19 @@ extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, 
                        (const float2*)cs, slots, (float*)q_out, (float*)k_cache, (float*)v_cache, heads, kv_heads,
                        head_dim, page_size, total_slots);
   else if (dtype == IX_BF16 && head_dim % 16 == 0) {
-    const int items8 = (heads + 2 * kv_heads) * (head_dim / 16);
+    // from a few dozen tokens on, the values go through the kernel that turns tiles of them
+    const int skip_v = (tokens >= 2 * V_TILE_TOKENS && v_cache != nullptr && slots != nullptr && kv_heads <= 65535) ? 1 : 0;
+    const int items8 = (heads + (skip_v ? 1 : 2) * kv_heads) * (head_dim / 16);
     dim3 grid8(tokens, std::min((items8 + 255) / 256, 8));
     hipLaunchKernelGGL(qkv_rope_append_vec8_kernel, grid8, block, 0, stream, (const uint16_t*)qkv, bias, bias_dtype,
                        (const float2*)cs, slots, (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, heads,
-                       kv_heads, head_dim, page_size, total_slots);
+                       kv_heads, head_dim, page_size, total_slots, skip_v);
+    if (skip_v) {
+      dim3 grid_v(static_cast<unsigned>((tokens + V_TILE_TOKENS - 1) / V_TILE_TOKENS), kv_heads);
+      const size_t lds = static_cast<size_t>(V_TILE_TOKENS) * (head_dim + 2) * sizeof(uint16_t);
+      hipLaunchKernelGGL(v_append_tile_kernel, grid_v, block, lds, stream, (const uint16_t*)qkv, bias, bias_dtype,
+                         slots, (uint16_t*)v_cache, tokens, heads, kv_heads, head_dim, page_size, total_slots);
+    }
   } else if (dtype == IX_BF16)
     hipLaunchKernelGGL(qkv_rope_append_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)qkv, bias, bias_dtype,
                        (const float2*)cs, slots, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads,

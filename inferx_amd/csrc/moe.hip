@@ -154,7 +154,55 @@ moe_route_select_kernel(const float* __restrict__ logits, float* __restrict__ to
   route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale);
 }
 
-// `logits_scratch`: float32 [tokens, experts + 1], used when tokens <= ROUTE_SMALL_TOKENS (may be null otherwise).
+// Many tokens, bfloat16 activations and weights: the scores on the matrix cores (exact products of bfloat16
+// numbers, float32 sums), to `logits` as above.  A workgroup takes 16 tokens and 16 rows (of the router, then the
+// shared gate's row); its four wavefronts split the reduction (32-wide pieces in turn, four of them in flight)
+// and add up through LDS.  As in the grouped products the weight rows are the A operand, so a lane ends up with
+// four consecutive scores of one token.
+typedef __bf16 route_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float route_f32x4 __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256)
+moe_route_logits_mfma_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ wr,
+                             const __bf16* __restrict__ shared_gate_w, float* __restrict__ logits, int64_t tokens,
+                             int width, int experts) {
+  __shared__ route_f32x4 part[4][64];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int m = lane & 15, g = lane >> 4;
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * 16;
+  const int rows = experts + (shared_gate_w ? 1 : 0);
+  const int r = 16 * blockIdx.y + m;  // this lane's weight row
+  const __bf16* xrow = x + min(t0 + m, tokens - 1) * width;  // tokens past the end repeat the last; not written
+  const __bf16* wrow = r < experts ? wr + static_cast<int64_t>(r) * width : (r < rows ? shared_gate_w : nullptr);
+  route_bf16x8 zero;
+  for (int j = 0; j < 8; ++j) zero[j] = (__bf16)0.f;
+  route_f32x4 acc = route_f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int kc = 32 * wave; kc < width; kc += 512) {  // uniform over the wavefront
+    route_bf16x8 xb[4], wa[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k0 = kc + 128 * u + 8 * g;
+      const bool ok = k0 < width;  // width is a multiple of 8: a lane's piece is whole or absent
+      xb[u] = ok ? *reinterpret_cast<const route_bf16x8*>(xrow + k0) : zero;
+      wa[u] = (ok && wrow) ? *reinterpret_cast<const route_bf16x8*>(wrow + k0) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[u], xb[u], acc, 0, 0, 0);
+  }
+  part[wave][lane] = acc;
+  __syncthreads();
+  if (wave == 0) {
+    const route_f32x4 sum = part[0][lane] + part[1][lane] + part[2][lane] + part[3][lane];
+    const int64_t t = t0 + m;  // lane holds rows 16 y + 4 g + i of token t0 + m
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int row = 16 * blockIdx.y + 4 * g + i;
+      if (t < tokens && row < rows) logits[t * (experts + 1) + row] = sum[i];
+    }
+  }
+}
+
+// `logits_scratch`: float32 [tokens, experts + 1], used when tokens <= ROUTE_SMALL_TOKENS, and for more tokens when
+// activations and weights are bfloat16 (may be null: then one kernel per token computes and selects).
 #define ROUTE_SMALL_TOKENS 128
 extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dtype, const void* shared_gate_w,
                             int sg_dtype, float* topk_w, int32_t* topk_e, float* shared_gate, float* logits_scratch,
@@ -177,6 +225,18 @@ extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dty
     else
       hipLaunchKernelGGL(moe_route_logits_kernel<bf16_t>, grid, block, xs_bytes, stream, (const bf16_t*)x, wr,
                          wr_dtype, shared_gate_w, sg_dtype, logits_scratch, width, experts);
+    hipLaunchKernelGGL(moe_route_select_kernel, dim3(tokens), dim3(64), experts * sizeof(float), stream,
+                       logits_scratch, topk_w, topk_e, shared_gate_w ? shared_gate : nullptr, experts, k, renormalize,
+                       scale);
+    return ix_check_launch("ix_moe_route");
+  }
+  if (logits_scratch != nullptr && dtype == IX_BF16 && wr_dtype == IX_BF16 &&
+      (shared_gate_w == nullptr || sg_dtype == IX_BF16) && width % 8 == 0 && width < (1 << 30) &&
+      ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(wr) | reinterpret_cast<uintptr_t>(shared_gate_w)) & 15) == 0) {
+    const int row_blocks = (experts + (shared_gate_w ? 1 : 0) + 15) / 16;
+    hipLaunchKernelGGL(moe_route_logits_mfma_kernel, dim3(static_cast<unsigned>((tokens + 15) / 16), row_blocks),
+                       dim3(256), 0, stream, (const __bf16*)x, (const __bf16*)wr, (const __bf16*)shared_gate_w, logits_scratch,
+                       tokens, (int)width, experts);
     hipLaunchKernelGGL(moe_route_select_kernel, dim3(tokens), dim3(64), experts * sizeof(float), stream,
                        logits_scratch, topk_w, topk_e, shared_gate_w ? shared_gate : nullptr, experts, k, renormalize,
                        scale);

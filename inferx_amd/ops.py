@@ -286,7 +286,11 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
         _need(shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= T,
               "shared_gate must be float32 [T]")
     scratch = None
-    if T <= ROUTE_SMALL_TOKENS:  # few tokens: scores go through a scratch so that many workgroups share the rows
+    all_bf16 = (x.dtype == torch.bfloat16 and router_w.dtype == torch.bfloat16
+                and (shared_gate_w is None or shared_gate_w.dtype == torch.bfloat16))
+    if T <= ROUTE_SMALL_TOKENS or all_bf16:
+        # few tokens: scores go through a scratch so that many workgroups share the rows; many tokens in
+        # bfloat16: the scores are a product on the matrix cores
         scratch = torch.empty((T, E + 1), dtype=torch.float32, device=x.device)
     _call("ix_moe_route", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
           _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(topk_w), _ptr(topk_e),

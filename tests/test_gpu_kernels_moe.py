@@ -27,7 +27,8 @@ def route_reference(x, wr, k, renorm, scale=1.0):
 
 
 @pytest.mark.parametrize("T,H,E,k,renorm", [(24, 64, 8, 2, False), (7, 200, 60, 4, True), (130, 72, 5, 1, False),
-                                            (3, 2048, 64, 8, True), (50, 96, 32, 32, True)])
+                                            (3, 2048, 64, 8, True), (50, 96, 32, 32, True),
+                                            (300, 136, 60, 4, True), (203, 40, 70, 6, False)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_route(T, H, E, k, renorm, dtype):
     # reference: moe_test.cc:170-246 (router equals host to 1e-5, renormalised sums to 1, un-normalised below)

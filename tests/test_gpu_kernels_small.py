@@ -69,6 +69,18 @@ def test_silu_mul(dtype):
     assert rel_err(out, pm.silu(g) * u) < tol(dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("T,width", [(33, 1408), (5, 24), (64, 100)])
+def test_silu_mul_sizes(dtype, T, width):
+    """Widths that take the 16-byte path (multiples of 8) and one that does not."""
+    from inferx_amd import ops
+    gu = rnd(T, 2 * width, dtype=dtype, scale=3.0)
+    out = torch.empty(T, width, dtype=dtype, device=DEV)
+    ops.silu_mul(gu, out)
+    g, u = gu.double().cpu()[:, :width], gu.double().cpu()[:, width:]
+    assert rel_err(out, pm.silu(g) * u) < tol(dtype)
+
+
 @pytest.mark.parametrize("theta,d", [(10000.0, 16), (1e6, 128), (50000.0, 48)])
 def test_rope_table(theta, d):
     from inferx_amd import ops
@@ -119,6 +131,46 @@ def test_qkv_rope_append(dtype, heads, kv, d, page, bias):
     q2 = torch.empty_like(q)
     ops.qkv_rope_append(qkv, b, None, None, q2, None, None, heads, kv, d)
     assert rel_err(q2, x[:, :heads * d].view(T, heads, d)) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("heads,kv,d,page,bias", [(4, 2, 16, 16, True), (5, 5, 128, 16, True), (6, 3, 48, 32, False)])
+def test_qkv_rope_append_many_tokens(dtype, heads, kv, d, page, bias):
+    """Portions of two requests, each starting in the middle of a page and running over several pages that
+    do not follow each other in the pool (the values of many tokens are written by a kernel of their own)."""
+    from inferx_amd import ops
+    from inferx_amd.parts.rope import Rotary
+    theta, pages = 10000.0, 24
+    starts, counts = [5, page + 3], [4 * page + 7, 3 * page - 2]
+    order = torch.randperm(pages, generator=torch.Generator().manual_seed(5)).tolist()
+    tables = [order[:8], order[8:16]]
+    pos = torch.tensor([p0 + i for p0, n in zip(starts, counts) for i in range(n)], dtype=torch.int32)
+    slot_list = [tables[r][(p0 + i) // page] * page + (p0 + i) % page
+                 for r, (p0, n) in enumerate(zip(starts, counts)) for i in range(n)]
+    slot_list[3] = -1  # one token that writes nothing
+    T, width = len(slot_list), (heads + 2 * kv) * d
+    slots = torch.tensor(slot_list, dtype=torch.int32, device=DEV)
+    qkv = rnd(T, width, dtype=dtype)
+    b = rnd(width, seed=1, dtype=dtype) if bias else None
+    table = torch.empty(T, d // 2, 2, device=DEV)
+    ops.rope_table(table, pos.to(DEV), Rotary(theta, d).frequencies().to(DEV))
+    q = torch.empty(T, heads, d, dtype=dtype, device=DEV)
+    kc = torch.zeros(pages, kv, page, d, dtype=dtype, device=DEV)
+    vc = torch.zeros(pages, kv, d, page, dtype=dtype, device=DEV)
+    ops.qkv_rope_append(qkv, b, table, slots, q, kc, vc, heads, kv, d)
+    x = qkv.double().cpu() + (b.double().cpu() if bias else 0)
+    wq = pm.apply_rope(x[:, :heads * d].view(T, heads, d), pos, theta)
+    wk = pm.apply_rope(x[:, heads * d:(heads + kv) * d].view(T, kv, d), pos, theta)
+    wv = x[:, (heads + kv) * d:].view(T, kv, d)
+    assert rel_err(q, wq) < tol(dtype)
+    want_k, want_v = torch.zeros(pages, kv, page, d, dtype=torch.float64), torch.zeros(pages, kv, d, page, dtype=torch.float64)
+    for t, slot in enumerate(slot_list):
+        if slot >= 0:
+            want_k[slot // page, :, slot % page, :] = wk[t]
+            want_v[slot // page, :, :, slot % page] = wv[t]
+    assert rel_err(kc, want_k) < tol(dtype) and rel_err(vc, want_v) < tol(dtype)
+    untouched = want_v == 0
+    assert float(vc.double().cpu()[untouched].abs().sum()) == 0  # nothing else was written
 
 
 @pytest.mark.parametrize("T,H,heads,kv,d,page,bias", [(1, 64, 4, 2, 32, 16, True), (8, 2048, 16, 16, 128, 16, True),
