@@ -69,6 +69,50 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ h, const TD* __restrict__
   }
 }
 
+// bfloat16 delta and output with a width that is a multiple of 4: four columns per thread
+__global__ void add_rmsnorm_vec4_kernel(float* __restrict__ h, const uint16_t* __restrict__ delta,
+                                        const void* __restrict__ w, int w_dtype, uint16_t* __restrict__ out,
+                                        const int32_t* __restrict__ rows, int64_t width, float eps) {
+  __shared__ float red[16];
+  const int64_t r = blockIdx.x;
+  const int64_t row = rows ? rows[r] : r;
+  float* hr = h + row * width;
+  const uint16_t* dr = delta ? delta + row * width : nullptr;
+  const bool write_back = (rows == nullptr) && (dr != nullptr);
+  auto value = [&](int64_t c) {
+    float4 v = *reinterpret_cast<const float4*>(hr + c);
+    if (dr) {
+      const uint2 d = *reinterpret_cast<const uint2*>(dr + c);
+      v.x += __uint_as_float(d.x << 16);
+      v.y += __uint_as_float(d.x & 0xffff0000u);
+      v.z += __uint_as_float(d.y << 16);
+      v.w += __uint_as_float(d.y & 0xffff0000u);
+    }
+    return v;
+  };
+  float sumsq = 0.f;
+  for (int64_t c = 4 * threadIdx.x; c < width; c += 4 * blockDim.x) {
+    const float4 v = value(c);
+    sumsq += v.x * v.x;
+    sumsq += v.y * v.y;
+    sumsq += v.z * v.z;
+    sumsq += v.w * v.w;
+  }
+  sumsq = ix_block_sum(sumsq, red);
+  const float inv = 1.0f / sqrtf(sumsq / static_cast<float>(width) + eps);
+  uint16_t* outr = out + r * width;
+  for (int64_t c = 4 * threadIdx.x; c < width; c += 4 * blockDim.x) {
+    const float4 v = value(c);  // h is still as it was: it is written here, after its last reading
+    if (write_back) *reinterpret_cast<float4*>(hr + c) = v;
+    uint2 o;
+    o.x = ix_f32_to_bf16(v.x * inv * ix_load_rt(w, w_dtype, c)) |
+          static_cast<uint32_t>(ix_f32_to_bf16(v.y * inv * ix_load_rt(w, w_dtype, c + 1))) << 16;
+    o.y = ix_f32_to_bf16(v.z * inv * ix_load_rt(w, w_dtype, c + 2)) |
+          static_cast<uint32_t>(ix_f32_to_bf16(v.w * inv * ix_load_rt(w, w_dtype, c + 3))) << 16;
+    *reinterpret_cast<uint2*>(outr + c) = o;
+  }
+}
+
 extern "C" int ix_add_rmsnorm(void* h, const void* delta, int delta_dtype, const void* w, int w_dtype, void* out,
                               int out_dtype, const int32_t* rows, int64_t n_out_rows, int64_t width, float eps,
                               hipStream_t stream) {
@@ -79,6 +123,12 @@ extern "C" int ix_add_rmsnorm(void* h, const void* delta, int delta_dtype, const
 #define LAUNCH(TD, TO)                                                                                          \
   hipLaunchKernelGGL((add_rmsnorm_kernel<TD, TO>), grid, block, 0, stream, (float*)h, (const TD*)delta, w, w_dtype, \
                      (TO*)out, rows, width, eps)
+  if (out_dtype == IX_BF16 && (delta == nullptr || delta_dtype == IX_BF16) && width % 4 == 0 &&
+      ((reinterpret_cast<uintptr_t>(h) | reinterpret_cast<uintptr_t>(delta) | reinterpret_cast<uintptr_t>(out)) & 15) == 0) {
+    hipLaunchKernelGGL(add_rmsnorm_vec4_kernel, grid, dim3(width >= 4096 ? 1024 : (width >= 2048 ? 512 : 256)), 0, stream,
+                       (float*)h, (const uint16_t*)delta, w, w_dtype, (uint16_t*)out, rows, width, eps);
+    return ix_check_launch("ix_add_rmsnorm");
+  }
   if (delta_dtype == IX_F32 && out_dtype == IX_F32) LAUNCH(float, float);
   else if (delta_dtype == IX_F32 && out_dtype == IX_BF16) LAUNCH(float, bf16_t);
   else if (delta_dtype == IX_BF16 && out_dtype == IX_F32) LAUNCH(bf16_t, float);
