@@ -58,24 +58,36 @@ __device__ __forceinline__ void grouped_body(const __bf16* __restrict__ a, const
 
   const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
                        (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
-  for (int k0 = kbegin; k0 < kend; k0 += 128) {
-    bf16x8 fw[NACC][4], fx[MT][4];
+  // the loads of the next 128 of K are issued before the products of the present ones, so that a wavefront
+  // always has loads on their way
+  bf16x8 fw[2][NACC][4], fx[2][MT][4];
+  auto fetch = [&](int k0, bf16x8 (&w_)[NACC][4], bf16x8 (&x_)[MT][4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int kk = k0 + 32 * g + 8 * j;
       const bool ok = kk < kend;
-      fw[0][j] = ok ? *reinterpret_cast<const bf16x8*>(wg + kk) : zero;
-      if (GATE_UP) fw[1][j] = ok ? *reinterpret_cast<const bf16x8*>(wu + kk) : zero;
+      w_[0][j] = ok ? *reinterpret_cast<const bf16x8*>(wg + kk) : zero;
+      if (GATE_UP) w_[1][j] = ok ? *reinterpret_cast<const bf16x8*>(wu + kk) : zero;
 #pragma unroll
-      for (int t = 0; t < MT; ++t) fx[t][j] = ok ? *reinterpret_cast<const bf16x8*>(xr[t] + kk) : zero;
+      for (int t = 0; t < MT; ++t) x_[t][j] = ok ? *reinterpret_cast<const bf16x8*>(xr[t] + kk) : zero;
     }
+  };
+  auto multiply = [&](const bf16x8 (&w_)[NACC][4], const bf16x8 (&x_)[MT][4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
       for (int t = 0; t < MT; ++t)
 #pragma unroll
         for (int u = 0; u < NACC; ++u)
-          acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fw[u][j], fx[t][j], acc[u][t], 0, 0, 0);
+          acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_[u][j], x_[t][j], acc[u][t], 0, 0, 0);
+  };
+  if (kbegin < kend) fetch(kbegin, fw[0], fx[0]);
+  for (int k0 = kbegin; k0 < kend; k0 += 256) {  // two rounds per turn, so that the register sets are named statically
+    if (k0 + 128 < kend) fetch(k0 + 128, fw[1], fx[1]);
+    multiply(fw[0], fx[0]);
+    if (k0 + 128 >= kend) break;
+    if (k0 + 256 < kend) fetch(k0 + 256, fw[0], fx[0]);
+    multiply(fw[1], fx[1]);
   }
 
   if (KSPLIT > 1) {
