@@ -63,6 +63,26 @@ def host_lib():
             "ixh_cache_pool_stats": (None, [vp, ci, i32p, i32p]),
             "ixh_cache_check": (ci, [vp]),
             "ixh_build_batch": (ci, [vp, ci, i64p, i32p, i32p, i32p, i32p] + [i32p] * 9 + [ctypes.POINTER(ci)]),
+            "ixh_cache_num_live": (ci, [vp]),
+            "ixh_cache_live": (ci, [vp, i64p, ci]),
+            "ixh_sched_create": (vp, [vp, ci, i64, i64]),
+            "ixh_sched_destroy": (None, [vp]),
+            "ixh_sched_error": (ctypes.c_char_p, [vp]),
+            "ixh_sched_add": (ci, [vp, i64, i32p, ci, i64, i64, i32p, ci]),
+            "ixh_sched_cancel": (None, [vp, i64]),
+            "ixh_sched_has_work": (ci, [vp]),
+            "ixh_sched_preemptions": (i64, [vp]),
+            "ixh_sched_prepare": (ci, [vp]),
+            "ixh_sched_plan_tokens": (i64, [vp]),
+            "ixh_sched_plan": (None, [vp, i64p, i64p, i32p, i32p, i32p]),
+            "ixh_sched_commit": (ci, [vp, i32p, ci]),
+            "ixh_sched_num_completed": (ci, [vp]),
+            "ixh_sched_completed": (None, [vp, ci, i64p, i32p, i32p]),
+            "ixh_sched_completed_tokens": (None, [vp, ci, i32p]),
+            "ixh_sched_clear_completed": (None, [vp]),
+            "ixh_sched_list": (ci, [vp, ci, i64p, ci]),
+            "ixh_sched_seq_info": (ci, [vp, i64, i32p, i64p, i64p]),
+            "ixh_sched_seq_tokens": (ci, [vp, i64, i64, i32p, i64]),
             "ixh_pool_create": (vp, [ci]),
             "ixh_pool_destroy": (None, [vp]),
             "ixh_pool_allocate": (ci, [vp]),
@@ -170,6 +190,8 @@ class CacheManager:
             raise CacheError("the cache manager could not be created")
         self.pools = [_PoolView(self, g) for g in range(G)]
         self._ids: Dict[Hashable, int] = {}  # request id (any hashable) -> the integer the library knows it by
+        self._names: Dict[int, Hashable] = {}  # and back
+        self._pinned = set()  # names that stay known while the request holds nothing (see intern)
         self._next = 0
 
     def __del__(self):
@@ -187,32 +209,61 @@ class CacheManager:
         except KeyError:
             raise CacheError(f"unknown request {rid!r}") from None
 
+    def intern(self, rid) -> int:
+        """The integer the library knows `rid` by, given out now if it has none.  A name interned here stays
+        known until `forget`, also while the request holds nothing (the scheduler's library adds and frees
+        requests by these integers on its own)."""
+        if rid not in self._ids:
+            self._ids[rid] = self._next
+            self._names[self._next] = rid
+            self._next += 1
+        self._pinned.add(rid)
+        return self._ids[rid]
+
+    def forget(self, rid) -> None:
+        self._pinned.discard(rid)
+        if rid in self._ids and not self._lib.ixh_cache_contains(self._h, self._ids[rid]):
+            del self._names[self._ids.pop(rid)]
+
+    def name_of(self, ident: int):
+        return self._names[ident]
+
     # ---- requests -------------------------------------------------------
     def __contains__(self, rid) -> bool:
-        return rid in self._ids
+        return rid in self._ids and bool(self._lib.ixh_cache_contains(self._h, self._ids[rid]))
 
     def live_requests(self):
-        return list(self._ids)
+        n = self._lib.ixh_cache_num_live(self._h)
+        buf = (ctypes.c_int64 * max(n, 1))()
+        self._lib.ixh_cache_live(self._h, buf, n)
+        return [self._names[i] for i in buf[:n]]
 
     def can_add(self) -> bool:
         return bool(self._lib.ixh_cache_can_add(self._h))
 
     def add(self, rid) -> int:
         """Start a request: takes a state slot, no pages yet.  Returns the slot."""
-        if rid in self._ids:
+        if rid in self:
             raise CacheError(f"request {rid!r} is already live")
-        slot = self._lib.ixh_cache_add(self._h, self._next)
+        fresh = rid not in self._ids
+        if fresh:
+            self._ids[rid] = self._next
+            self._names[self._next] = rid
+            self._next += 1
+        slot = self._lib.ixh_cache_add(self._h, self._ids[rid])
         if slot < 0:
-            raise self._err(rid)
-        self._ids[rid] = self._next
-        self._next += 1
+            err = self._err(rid)
+            if fresh:
+                del self._names[self._ids.pop(rid)]
+            raise err
         return slot
 
     def free(self, rid) -> None:
         """End a request: every page and the state slot go back."""
         if self._lib.ixh_cache_free(self._h, self._id(rid)) != 0:
             raise self._err(rid)
-        del self._ids[rid]
+        if rid not in self._pinned:
+            del self._names[self._ids.pop(rid)]
 
     def reset(self, rid) -> None:
         """Preemption by recomputation: pages go back, the request starts over at

@@ -128,8 +128,7 @@ class LLMEngine:
         rows = []
         for c in plan.contributions:
             if c.samples:
-                s = self.scheduler.sequence(c.rid)
-                rows.append((s.params, s.draws, s.tokens[s.prompt_len:]))
+                rows.append(self.scheduler.sequence(c.rid).sampling_row())
         sampled = self.sampler.sample(logits, rows)
         self.scheduler.commit_step(sampled, self.sampler.last_logprobs)
         self.stats.steps += 1

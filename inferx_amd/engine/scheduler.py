@@ -1,5 +1,8 @@
 """The scheduler: all policy, no GPU.  It decides who runs, in which portions,
-and what gives when pages run out; the model runner decides nothing.
+and what gives when pages run out; the model runner decides nothing.  The
+decisions are made in the host library (inferx_amd/csrc/host/scheduler.cc); this
+module is its face and keeps what only Python has use for (sampling
+parameters, log-probabilities).
 
 Policies are the reference's (src/scheduler/scheduler.cc):
   admission   first come first served while fewer than `max_running` run; pages
@@ -19,29 +22,70 @@ Pages go back the moment a sequence finishes or is preempted (:231-245).
 """
 from __future__ import annotations
 
-from collections import deque
+import ctypes
 from dataclasses import dataclass, field
-from typing import Deque, Dict, Hashable, List, Optional, Tuple
+from typing import Dict, Hashable, List, Optional
 
-from ..cache.manager import (RESERVE_CONTEXT_FULL, RESERVE_OK, RESERVE_POOL_EMPTY, CacheManager)
+import numpy as np
+
+from ..cache.manager import CacheManager, host_lib
 from ..sampling.params import SamplingParams
 
 FINISH_STOP, FINISH_LENGTH, FINISH_CANCELLED = "stop_token", "max_tokens", "cancelled"
 FINISH_CONTEXT, FINISH_OOM = "context_limit", "out_of_memory"
+_REASONS = [FINISH_STOP, FINISH_LENGTH, FINISH_CANCELLED, FINISH_CONTEXT, FINISH_OOM]  # the library's numbering
 
 
-@dataclass
+class GeneratedTokens:
+    """The tokens a sequence has generated so far: its length is known at once, the tokens are fetched from the
+    library only when somebody iterates (penalties)."""
+
+    def __init__(self, sched: "Scheduler", ident: int, prompt_len: int, count: int):
+        self._sched, self._ident, self._prompt_len, self._count = sched, ident, prompt_len, count
+
+    def __len__(self) -> int:
+        return self._count
+
+    def __iter__(self):
+        return iter(self._sched._tokens(self._ident, self._prompt_len, self._count))
+
+
 class Sequence:
-    rid: Hashable
-    tokens: List[int]
-    prompt_len: int
-    params: SamplingParams
-    cancelled: bool = False
-    draws: int = 0  # sampled tokens so far: the counter of this request's random stream
-    logprobs: List = field(default_factory=list)  # per generated token, when asked for
+    """A look at one request the scheduler knows."""
+
+    def __init__(self, sched: "Scheduler", rid: Hashable):
+        self._sched, self.rid = sched, rid
+        self._ident = sched.cache.intern(rid)
+        self.params: SamplingParams = sched._params[rid]
+
+    def _info(self):
+        p, n, d = ctypes.c_int32(), ctypes.c_int64(), ctypes.c_int64()
+        if self._sched._lib.ixh_sched_seq_info(self._sched._h, self._ident, ctypes.byref(p), ctypes.byref(n),
+                                               ctypes.byref(d)) != 0:
+            raise KeyError(self.rid)
+        return p.value, n.value, d.value
+
+    @property
+    def prompt_len(self) -> int:
+        return self._info()[0]
+
+    @property
+    def draws(self) -> int:
+        """Sampled tokens so far: the counter of this request's random stream."""
+        return self._info()[2]
+
+    @property
+    def tokens(self) -> List[int]:
+        return self._sched._tokens(self._ident, 0, self._info()[1])
 
     def generated(self) -> int:
-        return len(self.tokens) - self.prompt_len
+        p, n, _ = self._info()
+        return n - p
+
+    def sampling_row(self):
+        """(parameters, draws so far, generated tokens) as the sampler wants them."""
+        p, n, d = self._info()
+        return self.params, d, GeneratedTokens(self._sched, self._ident, p, n - p)
 
 
 @dataclass
@@ -73,6 +117,14 @@ class StepPlan:
         return sum(len(c.tokens) for c in self.contributions)
 
 
+def _p32(a):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_int32))
+
+
+def _p64(a):
+    return a.ctypes.data_as(ctypes.POINTER(ctypes.c_int64))
+
+
 class Scheduler:
     def __init__(self, cache: CacheManager, max_running: int = 8, max_batch_tokens: int = 2048,
                  max_seq_len: Optional[int] = None):
@@ -82,11 +134,26 @@ class Scheduler:
         self.max_running = min(max_running, cache.max_requests)
         self.max_batch_tokens = max_batch_tokens
         self.max_seq_len = min(max_seq_len or cache.max_seq_len, cache.max_seq_len)
-        self.waiting: Deque[Sequence] = deque()
-        self.running: List[Sequence] = []
-        self.completed: List[Completion] = []
-        self.preemptions = 0
+        self._lib = host_lib()
+        self._h = self._lib.ixh_sched_create(cache._h, self.max_running, self.max_batch_tokens, self.max_seq_len)
+        if not self._h:
+            raise RuntimeError("the scheduler could not be created")
+        self._params: Dict[Hashable, SamplingParams] = {}
+        self._logprobs: Dict[Hashable, List] = {}
         self._plan: Optional[StepPlan] = None
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            self._lib.ixh_sched_destroy(self._h)
+            self._h = None
+
+    def _error(self) -> str:
+        return self._lib.ixh_sched_error(self._h).decode("utf-8", "replace")
+
+    def _tokens(self, ident: int, start: int, count: int) -> List[int]:
+        buf = np.empty(max(count, 1), np.int32)
+        n = self._lib.ixh_sched_seq_tokens(self._h, ident, start, _p32(buf), count)
+        return buf[:max(n, 0)].tolist()
 
     # ---- requests --------------------------------------------------------
     def add_request(self, rid: Hashable, prompt: List[int], params: Optional[SamplingParams] = None) -> None:
@@ -94,127 +161,85 @@ class Scheduler:
         params.validate()
         if not prompt:
             raise ValueError("a request needs at least one prompt token")
-        if any(s.rid == rid for s in list(self.waiting) + self.running):
+        if rid in self._params:
             raise ValueError(f"request {rid!r} is already known")
-        self.waiting.append(Sequence(rid, list(prompt), len(prompt), params))
+        ids = np.asarray(prompt, dtype=np.int32)
+        stop = np.asarray(sorted(params.stop_tokens), dtype=np.int32)
+        rc = self._lib.ixh_sched_add(self._h, self.cache.intern(rid), _p32(ids), len(ids), int(params.max_tokens),
+                                     int(params.min_tokens), _p32(stop) if len(stop) else None, len(stop))
+        if rc != 0:
+            self.cache.forget(rid)
+            raise ValueError(f"request {rid!r} was refused by the scheduler ({rc})")
+        self._params[rid] = params
+        self._logprobs[rid] = []
 
     def cancel(self, rid: Hashable) -> None:
-        for s in list(self.waiting) + self.running:
-            if s.rid == rid:
-                s.cancelled = True
+        if rid in self._params:
+            self._lib.ixh_sched_cancel(self._h, self.cache.intern(rid))
 
     def has_work(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self._lib.ixh_sched_has_work(self._h))
 
-    def take_completed(self) -> List[Completion]:
-        out, self.completed = self.completed, []
-        return out
+    @property
+    def preemptions(self) -> int:
+        return self._lib.ixh_sched_preemptions(self._h)
+
+    def _list(self, which: int) -> List[Sequence]:
+        n = self._lib.ixh_sched_list(self._h, which, None, 0)
+        buf = np.empty(max(n, 1), np.int64)
+        self._lib.ixh_sched_list(self._h, which, _p64(buf), n)
+        return [Sequence(self, self.cache.name_of(int(i))) for i in buf[:n]]
+
+    @property
+    def running(self) -> List[Sequence]:
+        """The running sequences in order of admission."""
+        return self._list(0)
+
+    @property
+    def waiting(self) -> List[Sequence]:
+        """The waiting sequences from the head of the queue."""
+        return self._list(1)
 
     def sequence(self, rid) -> Sequence:
-        for s in self.running:
-            if s.rid == rid:
-                return s
-        raise KeyError(rid)
+        if rid not in self._params:
+            raise KeyError(rid)
+        return Sequence(self, rid)
 
-    # ---- internals ---------------------------------------------------------
-    def _pending(self, s: Sequence) -> int:
-        return len(s.tokens) - self.cache.cached(s.rid)
-
-    def _retire(self, s: Sequence, reason: str) -> None:
-        self.completed.append(Completion(s.rid, s.tokens[s.prompt_len:], reason,
-                                         list(s.logprobs) if s.logprobs else None))
-        if s.rid in self.cache:
-            self.cache.free(s.rid)
-
-    def _preempt(self, index: int) -> None:
-        victim = self.running.pop(index)
-        self.cache.free(victim.rid)
-        self.waiting.appendleft(victim)
-        self.preemptions += 1
-
-    def _admit(self) -> None:
-        while self.waiting and len(self.running) < self.max_running:
-            s = self.waiting[0]
-            if s.cancelled:
-                self.waiting.popleft()
-                self._retire(s, FINISH_CANCELLED)
-                continue
-            if len(s.tokens) > self.max_seq_len:
-                self.waiting.popleft()
-                self._retire(s, FINISH_OOM)
-                continue
-            if not self.cache.can_add():
-                return
-            self.cache.add(s.rid)
-            if self.cache.reserve(s.rid, len(s.tokens)) != RESERVE_OK:
-                self.cache.free(s.rid)  # not a preemption site: it waits at the head of the queue
-                return
-            self.waiting.popleft()
-            self.running.append(s)
-
-    def _take(self) -> List[int]:
-        take = [0] * len(self.running)
-        budget = self.max_batch_tokens
-        for i, s in enumerate(self.running):
-            if budget > 0 and self._pending(s) == 1:
-                take[i] = 1
-                budget -= 1
-        for i, s in enumerate(self.running):
-            pending = self._pending(s)
-            if budget > 0 and pending > 1:
-                take[i] = min(pending, budget)
-                budget -= take[i]
-        return take
+    def take_completed(self) -> List[Completion]:
+        n = self._lib.ixh_sched_num_completed(self._h)
+        out = []
+        for i in range(n):
+            ident, reason, count = ctypes.c_int64(), ctypes.c_int32(), ctypes.c_int32()
+            self._lib.ixh_sched_completed(self._h, i, ctypes.byref(ident), ctypes.byref(reason), ctypes.byref(count))
+            buf = np.empty(max(count.value, 1), np.int32)
+            self._lib.ixh_sched_completed_tokens(self._h, i, _p32(buf))
+            rid = self.cache.name_of(ident.value)
+            lps = self._logprobs.pop(rid, None)
+            self._params.pop(rid, None)
+            out.append(Completion(rid, buf[:count.value].tolist(), _REASONS[reason.value], list(lps) if lps else None))
+            self.cache.forget(rid)
+        if n:
+            self._lib.ixh_sched_clear_completed(self._h)
+        return out
 
     # ---- one step ------------------------------------------------------------
     def prepare_step(self) -> Optional[StepPlan]:
         """Decide the next step.  None when nothing can run."""
-        if self._plan is not None:
-            raise RuntimeError("prepare_step called twice without commit_step")
-        for s in [s for s in self.running if s.cancelled]:
-            self.running.remove(s)
-            self._retire(s, FINISH_CANCELLED)
-        self._admit()
-        take: List[int] = []
-        for _ in range(len(self.running) + 1):
-            if not self.running:
-                return None
-            take = self._take()
-            replan = False
-            for i, s in enumerate(self.running):
-                if take[i] == 0:
-                    continue
-                status = self.cache.reserve(s.rid, self.cache.cached(s.rid) + take[i])
-                if status == RESERVE_OK:
-                    continue
-                if status == RESERVE_CONTEXT_FULL:
-                    self.running.pop(i)
-                    self._retire(s, FINISH_CONTEXT)
-                else:
-                    victim = len(self.running) - 1
-                    if victim == i:
-                        if len(self.running) == 1:
-                            self.running.pop(i)
-                            self._retire(s, FINISH_OOM)
-                            replan = True
-                            break
-                        victim = len(self.running) - 2
-                    self._preempt(victim)
-                replan = True
-                break
-            if not replan:
-                break
-        if not self.running:
+        n = self._lib.ixh_sched_prepare(self._h)
+        if n < 0:
+            raise RuntimeError(self._error())
+        if n == 0:
             return None
-        plan = StepPlan()
-        for i, s in enumerate(self.running):
-            if take[i] == 0:
-                continue
-            at = self.cache.cached(s.rid)
-            plan.contributions.append(Contribution(s.rid, s.tokens[at:at + take[i]], at,
-                                                   samples=at + take[i] == len(s.tokens)))
-        if not plan.contributions:
-            return None
+        total = self._lib.ixh_sched_plan_tokens(self._h)
+        rids, first = np.empty(n, np.int64), np.empty(n, np.int64)
+        counts, samples, tokens = np.empty(n, np.int32), np.empty(n, np.int32), np.empty(total, np.int32)
+        self._lib.ixh_sched_plan(self._h, _p64(rids), _p64(first), _p32(counts), _p32(samples), _p32(tokens))
+        plan, at, flat = StepPlan(), 0, tokens.tolist()
+        for i in range(n):
+            c = int(counts[i])
+            plan.contributions.append(Contribution(self.cache.name_of(int(rids[i])), flat[at:at + c], int(first[i]),
+                                                   bool(samples[i])))
+            at += c
         self._plan = plan
         return plan
 
@@ -224,28 +249,15 @@ class Scheduler:
         plan, self._plan = self._plan, None
         if plan is None:
             raise RuntimeError("commit_step without prepare_step")
-        want = sum(1 for c in plan.contributions if c.samples)
-        if len(sampled) != want:
-            raise ValueError(f"{len(sampled)} sampled tokens for {want} sampling rows")
-        it = iter(sampled)
-        lp_it = iter(logprobs) if logprobs is not None else None
-        finished: List[Tuple[Sequence, str]] = []
-        by_id = {s.rid: s for s in self.running}
-        for c in plan.contributions:
-            s = by_id[c.rid]
-            self.cache.commit(c.rid, len(c.tokens))
-            if not c.samples:
-                continue
-            token = int(next(it))
-            lp = next(lp_it) if lp_it is not None else None
-            if lp is not None:
-                s.logprobs.append(lp)
-            s.tokens.append(token)
-            s.draws += 1
-            if token in s.params.stop_tokens and s.generated() > s.params.min_tokens:
-                finished.append((s, FINISH_STOP))
-            elif s.generated() >= s.params.max_tokens:
-                finished.append((s, FINISH_LENGTH))
-        for s, reason in finished:
-            self.running.remove(s)
-            self._retire(s, reason)
+        arr = np.asarray([int(t) for t in sampled], dtype=np.int32)
+        rc = self._lib.ixh_sched_commit(self._h, _p32(arr) if len(arr) else None, len(arr))
+        if rc == -2:
+            self._plan = plan
+            raise ValueError(self._error())
+        if rc != 0:
+            raise RuntimeError(self._error())
+        if logprobs is not None:
+            rows = [c.rid for c in plan.contributions if c.samples]
+            for rid, lp in zip(rows, logprobs):
+                if lp is not None and rid in self._logprobs:
+                    self._logprobs[rid].append(lp)

@@ -221,3 +221,51 @@ def test_max_running_and_windowed_group():
     done = drain(sched, cache, check=lambda plan, b: live.append(len(plan.contributions)))
     assert max(live) <= 2 and len(done) == 4 and all(c.reason == FINISH_LENGTH for c in done)
     assert all(p.used_pages == 0 for p in cache.pools)
+
+
+@pytest.mark.parametrize("seed", [0, 1, 2, 3])
+def test_random_arrivals_scarce_pages(seed):
+    """Requests arrive at random steps, some are cancelled, pages are scarce so that sequences are preempted:
+    every request finishes exactly once, no page or slot is lost at any step, every step keeps its budget, and
+    (tokens being a function of the position) each output equals the one of an unconstrained run."""
+    import random
+    rng = random.Random(seed)
+    n_req = 14
+    prompts = {r: [rng.randrange(1000) for _ in range(rng.randrange(1, 40))] for r in range(n_req)}
+    limits = {r: rng.randrange(1, 30) for r in range(n_req)}
+    arrive = {r: rng.randrange(0, 25) for r in range(n_req)}
+    cancel_at = {r: arrive[r] + rng.randrange(0, 12) for r in rng.sample(range(n_req), 3)}
+
+    def run(pages, budget, cancels):
+        sched, cache = make(pages=pages, page_size=4, max_running=4, budget=budget, max_seq_len=80)
+        done, step = [], 0
+        while step < 60 or sched.has_work():
+            for r in range(n_req):
+                if arrive[r] == step:
+                    sched.add_request(r, prompts[r], P(limits[r]))
+                if cancels and cancel_at.get(r) == step:
+                    sched.cancel(r)
+            plan = sched.prepare_step()
+            if plan is not None:
+                assert 0 < plan.num_tokens <= budget and len(plan.contributions) <= 4
+                batch = build_step_batch(cache, plan.entries())
+                batch.validate(10 ** 6, [p.num_pages for p in cache.pools], cache.page_size)
+                sched.commit_step([fake_token(int(batch.positions[r])) for r in batch.logits_rows])
+            done += sched.take_completed()
+            cache.check()
+            step += 1
+            assert step < 5000
+        assert all(p.used_pages == 0 for p in cache.pools) and not cache.live_requests()
+        return {c.rid: c for c in done}, sched.preemptions, len(done)
+
+    free, _, n_free = run(pages=400, budget=4096, cancels=False)
+    tight, preemptions, n_tight = run(pages=22, budget=24, cancels=True)
+    assert n_free == n_req and n_tight == n_req and set(tight) == set(range(n_req))
+    assert preemptions > 0
+    for r in range(n_req):
+        assert free[r].reason == FINISH_LENGTH and len(free[r].output_tokens) == limits[r]
+        if tight[r].reason == FINISH_CANCELLED:
+            assert r in cancel_at
+            assert tight[r].output_tokens == free[r].output_tokens[:len(tight[r].output_tokens)]
+        else:
+            assert tight[r].reason == FINISH_LENGTH and tight[r].output_tokens == free[r].output_tokens
