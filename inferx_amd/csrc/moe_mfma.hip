@@ -13,10 +13,10 @@
 // of row l%16, i.e. four consecutive numbers of one output row.
 //
 // A wavefront owns 16 out-features x (16 * MT) rows.  Per iteration it covers
-// 128 of K: lane (m, g) reads 64 contiguous bytes of weight row m (k0 + 32 g ..
-// + 32), as four 16-byte pieces j; piece j of all four lane groups forms the 32
-// reduction slots of MFMA j, and the activations are read with the same
-// mapping.  KSPLIT = 4 (decoding: few rows, the weights are the traffic) lets
+// 128 of K with four loads: in load j lane (m, g) reads the 16 bytes at
+// k0 + 32 j + 8 g of weight row m, so the four lane groups cover 64 contiguous
+// bytes of each row and the 32 reduction slots of MFMA j; the activations are
+// read with the same mapping.  KSPLIT = 4 (decoding: few rows, the weights are the traffic) lets
 // the four wavefronts of a workgroup take a quarter of K each and add up through
 // LDS; KSPLIT = 1 gives each wavefront its own 16 out-features.
 #include "common.h"
@@ -64,7 +64,7 @@ __device__ __forceinline__ void grouped_body(const __bf16* __restrict__ a, const
   auto fetch = [&](int k0, bf16x8 (&w_)[NACC][4], bf16x8 (&x_)[MT][4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int kk = k0 + 32 * g + 8 * j;
+      const int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row per load
       const bool ok = kk < kend;
       w_[0][j] = ok ? *reinterpret_cast<const bf16x8*>(wg + kk) : zero;
       if (GATE_UP) w_[1][j] = ok ? *reinterpret_cast<const bf16x8*>(wu + kk) : zero;

@@ -39,7 +39,7 @@ qkv_rope_skinny_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ 
     bf16x8 fl[4], fh[4], fx[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int kk = k0 + 32 * g + 8 * j;
+      const int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row per load
       const bool ok = kk < kend;
       fl[j] = ok ? *reinterpret_cast<const bf16x8*>(wl + kk) : zero;
       fh[j] = ok ? *reinterpret_cast<const bf16x8*>(wh + kk) : zero;
