@@ -113,7 +113,7 @@ class PagedAttention(Mixer):
 QUERY_TILE = 16          # queries of one request per wavefront ...
 LARGE_QUERY_TILE = 32    # ... or 32 when the step brings many tokens (keys and values are then read once per 32)
 LARGE_TILE_TOKENS = 1 << 30  # measured: no faster than tiles of 16 on MI355X, so off
-WAVES_WANTED = 4096      # enough wavefronts to fill 256 compute units
+WAVES_WANTED = 2048      # two wavefronts per SIMD of 256 compute units: measured best at batch 8 (longer slices per wavefront)
 MIN_KEYS_PER_SPLIT = 128
 PREFILL_MIN_TOKENS = 128  # the LDS-sharing kernel: steps of at least this many tokens ...
 PREFILL_MIN_ROWS = 16     # ... and this many per request on average
