@@ -79,13 +79,29 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
 
   const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
                        (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
-  // Two register sets: while stage s is multiplied out of LDS, stage s + 1 is on its way in one set (asked for a
-  // round earlier) and stage s + 2 is asked for into the other, so a load has two rounds to arrive.
-  bf16x8 wreg[2][4], xreg[2][TL_XPER];
-  auto fetch = [&](int k0, bf16x8 (&wr)[4], bf16x8 (&xr)[TL_XPER]) {
+  // The weights come from memory and are what the kernel waits for: three register sets keep the loads of three
+  // stages on their way while a fourth stage is multiplied out of LDS.  The activations are asked for two stages
+  // ahead, in two sets.
+  bf16x8 wreg[3][4], xreg[2][TL_XPER];
+  // Row tiles walk the reduction in the same order but start at different stages (and wrap round): were all
+  // workgroups at the same offset of their weight rows at the same time, a row length that is a power of two
+  // would send their loads to the same few memory channels (measured with few rows per expert: 4.0 instead of
+  // 5.0 TB/s at rows of 4,096 bytes).  The order of a workgroup's additions depends only on its place in the
+  // grid, so results repeat bit for bit.
+  const int kspan = ((width + TL_K - 1) / TL_K) * TL_K;
+  const int rot = (width % 512 == 0)  // rows of a multiple of 1,024 bytes; workgroups of one row tile stay together
+                      ? static_cast<int>((blockIdx.y * 3u) % static_cast<unsigned>(kspan / TL_K)) * TL_K
+                      : 0;         // (they read the same activations, which then stay in L2)
+  auto turned = [&](int k0) { return k0 + rot < kspan ? k0 + rot : k0 + rot - kspan; };
+  auto fetch_w = [&](int k0, bf16x8 (&wr)[4]) {
+    k0 = turned(k0);
     const bool ok = k0 + kc_mine < width;
 #pragma unroll
     for (int i = 0; i < 4; ++i) wr[i] = ok ? *reinterpret_cast<const bf16x8*>(w_expert + wsrc[i] + k0) : zero;
+  };
+  auto fetch_x = [&](int k0, bf16x8 (&xr)[TL_XPER]) {
+    k0 = turned(k0);
+    const bool ok = k0 + kc_mine < width;
 #pragma unroll
     for (int i = 0; i < TL_XPER; ++i)  // piece i lies in sixteens 2 i and 2 i + 1 (uniform over the workgroup)
       if (2 * i < nblk) xr[i] = ok ? *reinterpret_cast<const bf16x8*>(a + xsrc[i] + k0) : zero;
@@ -125,26 +141,37 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
     }
   };
 
-  fetch(0, wreg[0], xreg[0]);
+  fetch_w(0, wreg[0]);
+  fetch_x(0, xreg[0]);
   stage(wreg[0], xreg[0]);
-  if (TL_K < width) fetch(TL_K, wreg[1], xreg[1]);
-  __syncthreads();
-  // two stages per turn, so that the register sets are named statically
-  for (int k0 = 0; k0 < width; k0 += 2 * TL_K) {
-    if (k0 + 2 * TL_K < width) fetch(k0 + 2 * TL_K, wreg[0], xreg[0]);
-    multiply();  // stage k0
-    __syncthreads();
-    if (k0 + TL_K >= width) break;
-    stage(wreg[1], xreg[1]);
-    __syncthreads();
-    if (k0 + 3 * TL_K < width) fetch(k0 + 3 * TL_K, wreg[1], xreg[1]);
-    multiply();  // stage k0 + 64
-    __syncthreads();
-    if (k0 + 2 * TL_K < width) {
-      stage(wreg[0], xreg[0]);
-      __syncthreads();
-    }
+  if (TL_K < width) {
+    fetch_w(TL_K, wreg[1]);
+    fetch_x(TL_K, xreg[1]);
   }
+  if (2 * TL_K < width) fetch_w(2 * TL_K, wreg[2]);
+  __syncthreads();
+  // One stage s: ask for the weights of stage s + 3 and the activations of stage s + 2 (into the sets that held
+  // stage s, which is in LDS), multiply, then move stage s + 1 into LDS.  Six stages per turn, so that the
+  // register sets (three of weights, two of activations) are named statically.
+#define TL_STAGE(K0, W_FREE, W_NEXT, X_FREE, X_NEXT)                              \
+  {                                                                               \
+    if ((K0) + 3 * TL_K < width) fetch_w((K0) + 3 * TL_K, wreg[W_FREE]);          \
+    if ((K0) + 2 * TL_K < width) fetch_x((K0) + 2 * TL_K, xreg[X_FREE]);          \
+    multiply();                                                                   \
+    __syncthreads();                                                              \
+    if ((K0) + TL_K >= width) break;                                              \
+    stage(wreg[W_NEXT], xreg[X_NEXT]);                                            \
+    __syncthreads();                                                              \
+  }
+  for (int k0 = 0; k0 < width; k0 += 6 * TL_K) {
+    TL_STAGE(k0, 0, 1, 0, 1)
+    TL_STAGE(k0 + TL_K, 1, 2, 1, 0)
+    TL_STAGE(k0 + 2 * TL_K, 2, 0, 0, 1)
+    TL_STAGE(k0 + 3 * TL_K, 0, 1, 1, 0)
+    TL_STAGE(k0 + 4 * TL_K, 1, 2, 0, 1)
+    TL_STAGE(k0 + 5 * TL_K, 2, 0, 1, 0)
+  }
+#undef TL_STAGE
 
   // lane holds weight rows (block) + 4 g + i of activation row row0 + 16 (2 t + xi) + m
   const bool vec = (n_out & 3) == 0;
