@@ -38,16 +38,60 @@ __device__ __forceinline__ float ix_load_rt(const void* base, int dtype, int64_t
                          : ix_bf16_to_f32(static_cast<const uint16_t*>(base)[i]);
 }
 
+// Sum / maximum over the 64 lanes, result in every lane.  Within a row of 16 lanes the partners come through
+// DPP (lanes ^1, ^2, then the half row and the row mirrored: no LDS round trip), across rows through two
+// exchanges.  The order of the additions is fixed.
+template <int CTRL>
+__device__ __forceinline__ float ix_dpp(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+template <int CTRL>
+__device__ __forceinline__ int ix_dpp(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+#define IX_DPP_XOR1 0xB1         // quad_perm [1, 0, 3, 2]
+#define IX_DPP_XOR2 0x4E         // quad_perm [2, 3, 0, 1]
+#define IX_DPP_HALF_MIRROR 0x141  // lane i of 8 <-> lane 7 - i
+#define IX_DPP_MIRROR 0x140       // lane i of 16 <-> lane 15 - i
+
 __device__ __forceinline__ float ix_wave_sum(float v) {
-#pragma unroll
-  for (int off = IX_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, IX_WAVE);
+  v += ix_dpp<IX_DPP_XOR1>(v);
+  v += ix_dpp<IX_DPP_XOR2>(v);
+  v += ix_dpp<IX_DPP_HALF_MIRROR>(v);
+  v += ix_dpp<IX_DPP_MIRROR>(v);
+  v += __shfl_xor(v, 16, IX_WAVE);
+  v += __shfl_xor(v, 32, IX_WAVE);
   return v;
 }
 
 __device__ __forceinline__ float ix_wave_max(float v) {
-#pragma unroll
-  for (int off = IX_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, IX_WAVE));
+  v = fmaxf(v, ix_dpp<IX_DPP_XOR1>(v));
+  v = fmaxf(v, ix_dpp<IX_DPP_XOR2>(v));
+  v = fmaxf(v, ix_dpp<IX_DPP_HALF_MIRROR>(v));
+  v = fmaxf(v, ix_dpp<IX_DPP_MIRROR>(v));
+  v = fmaxf(v, __shfl_xor(v, 16, IX_WAVE));
+  v = fmaxf(v, __shfl_xor(v, 32, IX_WAVE));
   return v;
+}
+
+// The largest value over the 64 lanes and, among equals, the smallest index that comes with it; in every lane.
+__device__ __forceinline__ void ix_wave_argmax(float& v, int& idx) {
+#define IX_ARGMAX_STEP(OV, OI)                               \
+  {                                                          \
+    const float ov = (OV);                                   \
+    const int oi = (OI);                                     \
+    if (ov > v || (ov == v && oi < idx)) {                   \
+      v = ov;                                                \
+      idx = oi;                                              \
+    }                                                        \
+  }
+  IX_ARGMAX_STEP(ix_dpp<IX_DPP_XOR1>(v), ix_dpp<IX_DPP_XOR1>(idx))
+  IX_ARGMAX_STEP(ix_dpp<IX_DPP_XOR2>(v), ix_dpp<IX_DPP_XOR2>(idx))
+  IX_ARGMAX_STEP(ix_dpp<IX_DPP_HALF_MIRROR>(v), ix_dpp<IX_DPP_HALF_MIRROR>(idx))
+  IX_ARGMAX_STEP(ix_dpp<IX_DPP_MIRROR>(v), ix_dpp<IX_DPP_MIRROR>(idx))
+  IX_ARGMAX_STEP(__shfl_xor(v, 16, IX_WAVE), __shfl_xor(idx, 16, IX_WAVE))
+  IX_ARGMAX_STEP(__shfl_xor(v, 32, IX_WAVE), __shfl_xor(idx, 32, IX_WAVE))
+#undef IX_ARGMAX_STEP
 }
 
 // Block-wide sum/max, result in every thread.  `red` holds one float per wave

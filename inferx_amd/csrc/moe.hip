@@ -73,12 +73,7 @@ __device__ __forceinline__ void route_select(float* z, float* red, float* __rest
       const float v = z[e];
       if (v > bv) { bv = v; bi = e; }
     }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) {
-      const float ov = __shfl_xor(bv, off, 64);
-      const int oi = __shfl_xor(bi, off, 64);
-      if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-    }
+    ix_wave_argmax(bv, bi);
     if (bi < 0 || bi >= experts) bi = 0;  // only when every score is NaN
     const float wgt = bv * inv_sum;
     total += wgt;

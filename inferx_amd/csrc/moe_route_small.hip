@@ -21,7 +21,6 @@ moe_select_dispatch_kernel(const float* __restrict__ logits, float* __restrict__
   __shared__ int32_t first_row[SD_MAX_EXPERTS];
   __shared__ int32_t first_tile[SD_MAX_EXPERTS];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  for (int e = tid; e < experts; e += SD_THREADS) counts[e] = 0;
 
   // ---- selection: one wavefront per token ----
   float* z = zs[wave];
@@ -52,12 +51,7 @@ moe_select_dispatch_kernel(const float* __restrict__ logits, float* __restrict__
         const float v = z[e];
         if (v > bv) { bv = v; bi = e; }
       }
-#pragma unroll
-      for (int off = 32; off > 0; off >>= 1) {
-        const float ov = __shfl_xor(bv, off, 64);
-        const int oi = __shfl_xor(bi, off, 64);
-        if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
-      }
+      ix_wave_argmax(bv, bi);
       if (bi < 0 || bi >= experts) bi = 0;  // only when every score is NaN
       const float wgt = bv * inv_sum;
       total += wgt;
@@ -75,39 +69,62 @@ moe_select_dispatch_kernel(const float* __restrict__ logits, float* __restrict__
   }
   __syncthreads();
 
-  // ---- grouping ----
+  // ---- grouping: thread e owns expert e ----
+  // counts: one pass over the assignments per thread (every thread reads the same LDS word: a broadcast)
   const int assignments = tokens * k;
-  int mine = -1, rank = 0;
-  if (tid < assignments) {
-    mine = chosen[tid];
-    for (int b = 0; b < tid; ++b) rank += (chosen[b] == mine) ? 1 : 0;
-    atomicAdd(&counts[mine], 1);  // integer counts: order does not matter
-  }
+  int my_count = 0;
+  if (tid < experts)
+    for (int a = 0; a < assignments; ++a) my_count += (chosen[a] == tid) ? 1 : 0;
+  if (tid < SD_MAX_EXPERTS) counts[tid] = tid < experts ? my_count : 0;
   __syncthreads();
-  if (tid == 0) {
-    int32_t run = 0, tiles = 0;
-    for (int e = 0; e < experts; ++e) {
-      offsets[e] = run;
+  // offsets: exclusive sums over the experts by the first wavefront, four experts per lane
+  if (wave == 0) {
+    int c[4], rows_before = 0, tiles_before = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      c[j] = counts[4 * lane + j];
+      rows_before += c[j];
+      tiles_before += tile_rows > 0 ? (c[j] + tile_rows - 1) / tile_rows : 0;
+    }
+    const int rows_mine = rows_before, tiles_mine = tiles_before;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {  // inclusive sums over the lanes
+      const int r = __shfl_up(rows_before, off, 64), t = __shfl_up(tiles_before, off, 64);
+      if (lane >= off) {
+        rows_before += r;
+        tiles_before += t;
+      }
+    }
+    int run = rows_before - rows_mine, tiles = tiles_before - tiles_mine;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int e = 4 * lane + j;
       first_row[e] = run;
       first_tile[e] = tiles;
-      run += counts[e];
-      if (tile_rows > 0) tiles += (counts[e] + tile_rows - 1) / tile_rows;
+      if (e < experts) offsets[e] = run;
+      run += c[j];
+      tiles += tile_rows > 0 ? (c[j] + tile_rows - 1) / tile_rows : 0;
     }
-    offsets[experts] = run;
-    if (tile_info) tile_info[0] = tiles;
+    if (lane == 63) {
+      offsets[experts] = run;
+      if (tile_info) tile_info[0] = tiles;
+    }
   }
   __syncthreads();
-  if (tid < assignments) {
-    const int32_t r = first_row[mine] + rank;
-    rows[r] = tid / k;
-    dest[tid] = r;
-  }
-  if (tile_rows > 0 && tile_expert) {
-    for (int e = tid; e < experts; e += SD_THREADS) {
-      const int n = (counts[e] + tile_rows - 1) / tile_rows;
+  // placement in the order of the assignments (stable), and the expert's row tiles
+  if (tid < experts) {
+    int r = first_row[tid];
+    for (int a = 0; a < assignments; ++a)
+      if (chosen[a] == tid) {
+        rows[r] = a / k;
+        dest[a] = r;
+        ++r;
+      }
+    if (tile_rows > 0 && tile_expert) {
+      const int n = (my_count + tile_rows - 1) / tile_rows;
       for (int i = 0; i < n; ++i) {
-        tile_expert[first_tile[e] + i] = e;
-        tile_row0[first_tile[e] + i] = first_row[e] + i * tile_rows;
+        tile_expert[first_tile[tid] + i] = tid;
+        tile_row0[first_tile[tid] + i] = first_row[tid] + i * tile_rows;
       }
     }
   }

@@ -23,11 +23,7 @@ __device__ __forceinline__ ArgPair better(ArgPair a, ArgPair b) {
 
 __device__ ArgPair block_argmax(ArgPair p, ArgPair* red) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    ArgPair o{__shfl_xor(p.v, off, 64), __shfl_xor(p.i, off, 64)};
-    p = better(p, o);
-  }
+  ix_wave_argmax(p.v, p.i);
   __syncthreads();
   if (lane == 0) red[wave] = p;
   __syncthreads();
