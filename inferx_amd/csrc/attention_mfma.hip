@@ -36,7 +36,7 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
                  const int32_t* __restrict__ tile_q0, const int32_t* __restrict__ tile_rows,
                  const int32_t* __restrict__ positions, __bf16* __restrict__ out, float* __restrict__ part_o,
                  float* __restrict__ part_ml, int n_tiles, int n_splits, int heads, int kv_heads, int page_size,
-                 int max_blocks, float scale_log2, int window) {
+                 int max_blocks, float scale_log2, int window, int page_shift) {
   constexpr int D = 16 * NB;
   constexpr int NC = (NB + 1) / 2;  // 32-wide chunks of the head dimension
   const int lane = threadIdx.x & 63;
@@ -86,15 +86,18 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
 
   // K fragments for the 32 keys from kb on (two blocks of 16 rows) and V^T fragments
   // (lane (dd = n, g) holds V^T[16 blk + dd][kb + 8 g .. +8])
+  // a page size that is a power of two (page_shift >= 0, the usual case) spares the divisions
+  auto page_of = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
   auto load_kv = [&](int kb, bf16x8 (&kf)[2][NC], bf16x8 (&vf)[NB]) {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
       int key = kb + 8 * (n >> 2) + 4 * b + (n & 3);  // A row n of block b
       key = min(key, hi - 1);                          // rows past the end are masked below
-      int page = table[key / page_size];
+      const int pi = page_of(key);
+      int page = table[pi];
       page = max(page, 0);                             // a page the window has passed: masked below
       const __bf16* kr =
-          k_cache + ((static_cast<int64_t>(page) * kv_heads + kvh) * page_size + key % page_size) * D;
+          k_cache + ((static_cast<int64_t>(page) * kv_heads + kvh) * page_size + (key - pi * page_size)) * D;
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const int d0 = 32 * c + 8 * g;
@@ -105,8 +108,9 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
       }
     }
     int key = min(kb + 8 * g, hi - 1) & ~7;
-    int page = max(table[key / page_size], 0);
-    const __bf16* vr = v_cache + (static_cast<int64_t>(page) * kv_heads + kvh) * D * page_size + key % page_size;
+    const int pi = page_of(key);
+    int page = max(table[pi], 0);
+    const __bf16* vr = v_cache + (static_cast<int64_t>(page) * kv_heads + kvh) * D * page_size + (key - pi * page_size);
 #pragma unroll
     for (int b = 0; b < NB; ++b)
       vf[b] = *reinterpret_cast<const bf16x8*>(vr + static_cast<int64_t>(16 * b + n) * page_size);
@@ -144,36 +148,55 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
       const int my_pos = pos0 + 16 * t + n;
       const bool my_row = 16 * t + n < rows;
       const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
+      // scores stay unscaled: the scale (times log2 e) enters with the reference point in one fused multiply-add
       float sv[8];
       float mx = -INFINITY;
+      // keys that every query of these sixteen sees need no mask (uniform over the wavefront)
+      const bool inner = 16 * t + 16 <= rows && kb + ATTN_KEYS_PER_ITER <= ke && kb + ATTN_KEYS_PER_ITER - 1 <= pos0 + 16 * t &&
+                         (window == 0 || kb > pos0 + 16 * t + 15 - window);
+      if (inner) {
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const int key = kb + 8 * g + j;
-        const bool ok = my_row && key >= my_lo && key <= my_pos && key < ke;
-        sv[j] = ok ? s[j >> 2][j & 3] * scale_log2 : -INFINITY;
-        mx = fmaxf(mx, sv[j]);
+        for (int j = 0; j < 8; ++j) {
+          sv[j] = s[j >> 2][j & 3];
+          mx = fmaxf(mx, sv[j]);
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = kb + 8 * g + j;
+          const bool ok = my_row && key >= my_lo && key <= my_pos && key < ke;
+          sv[j] = ok ? s[j >> 2][j & 3] : -INFINITY;
+          mx = fmaxf(mx, sv[j]);
+        }
       }
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m[t], mx);
-      const float m_safe = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = exp2f(m[t] - m_safe);
+      // The reference point m of the exponentials (in units of log2) follows the running maximum lazily: it moves
+      // only when some query's maximum has outgrown it by more than 2^8, so the accumulators are seldom rescaled.
+      // Any m gives the same quotient; probabilities up to 2^8 keep the relative precision of bfloat16.
+      const float top = mx * scale_log2;
+      if (__any(top > m[t] + 8.f)) {
+        const float m_new = fmaxf(m[t], top);
+        // v_exp_f32 as it is: a result below the smallest normal number may become 0
+        const float alpha = __builtin_amdgcn_exp2f(m[t] - ((m_new == -INFINITY) ? 0.f : m_new));
+        lsum[t] *= alpha;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) o[t][b] *= alpha;
+        m[t] = m_new;
+      }
+      const float m_safe = (m[t] == -INFINITY) ? 0.f : m[t];
       float psum = 0.f;
       bf16x8 pf;
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
-        const float p = exp2f(sv[j] - m_safe);
+        const float p = __builtin_amdgcn_exp2f(fmaf(sv[j], scale_log2, -m_safe));
         psum += p;
         pf[j] = (__bf16)p;
       }
-      lsum[t] = lsum[t] * alpha + psum;
-      m[t] = m_new;
+      lsum[t] += psum;
       // ---- O^T += V^T P^T ----
 #pragma unroll
-      for (int b = 0; b < NB; ++b) {
-        o[t][b] *= alpha;
-        o[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf, o[t][b], 0, 0, 0);
-      }
+      for (int b = 0; b < NB; ++b) o[t][b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[b], pf, o[t][b], 0, 0, 0);
     }
   }
 
@@ -248,9 +271,12 @@ static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void
                         const int32_t* tile_rows, const int32_t* positions, void* out, float* part_o, float* part_ml,
                         int n_tiles, int n_splits, int heads, int kv_heads, int page_size, int max_blocks,
                         float scale_log2, int window) {
+  int page_shift = -1;  // log2 of the page size if it is a power of two
+  for (int b = 4; b < 31; ++b)
+    if (page_size == (1 << b)) page_shift = b;
   hipLaunchKernelGGL((attn_mfma_kernel<NB, QT, PF>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, positions, (__bf16*)out, part_o, part_ml,
-                     n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window);
+                     n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window, page_shift);
 }
 
 // Workspace (when n_splits > 1): part_o float32 [tokens * heads * n_splits * head_dim],

@@ -28,7 +28,8 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-ta
 
 # per source: matrix-core accumulators in ordinary vector registers, where a kernel also rescales them with vector
 # instructions between products (the compiler otherwise copies them to and from accumulation registers every time)
-FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+              "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
 _lib: Optional[ctypes.CDLL] = None
 
