@@ -69,13 +69,18 @@ moe_select_dispatch_kernel(const float* __restrict__ logits, float* __restrict__
   }
   __syncthreads();
 
-  // ---- grouping: thread e owns expert e ----
-  // counts: one pass over the assignments per thread (every thread reads the same LDS word: a broadcast)
+  // ---- grouping: a wavefront per expert (in turn), 64 assignments at a time ----
+  // counts: lanes compare their assignments with the expert, a ballot counts the matches
   const int assignments = tokens * k;
-  int my_count = 0;
-  if (tid < experts)
-    for (int a = 0; a < assignments; ++a) my_count += (chosen[a] == tid) ? 1 : 0;
-  if (tid < SD_MAX_EXPERTS) counts[tid] = tid < experts ? my_count : 0;
+  if (tid >= experts && tid < SD_MAX_EXPERTS) counts[tid] = 0;
+  for (int e = wave; e < experts; e += SD_THREADS / 64) {
+    int count = 0;
+    for (int a0 = 0; a0 < assignments; a0 += 64) {
+      const int a = a0 + lane;
+      count += __popcll(__ballot(a < assignments && chosen[a] == e));
+    }
+    if (lane == 0) counts[e] = count;
+  }
   __syncthreads();
   // offsets: exclusive sums over the experts by the first wavefront, four experts per lane
   if (wave == 0) {
@@ -111,20 +116,27 @@ moe_select_dispatch_kernel(const float* __restrict__ logits, float* __restrict__
     }
   }
   __syncthreads();
-  // placement in the order of the assignments (stable), and the expert's row tiles
-  if (tid < experts) {
-    int r = first_row[tid];
-    for (int a = 0; a < assignments; ++a)
-      if (chosen[a] == tid) {
+  // placement in the order of the assignments (stable): a match's row is the expert's first row plus the matches
+  // before it; and the expert's row tiles
+  const uint64_t below = (uint64_t(1) << lane) - 1;
+  for (int e = wave; e < experts; e += SD_THREADS / 64) {
+    int base = first_row[e];
+    for (int a0 = 0; a0 < assignments; a0 += 64) {
+      const int a = a0 + lane;
+      const bool match = a < assignments && chosen[a] == e;
+      const uint64_t mask = __ballot(match);
+      if (match) {
+        const int r = base + __popcll(mask & below);
         rows[r] = a / k;
         dest[a] = r;
-        ++r;
       }
+      base += __popcll(mask);
+    }
     if (tile_rows > 0 && tile_expert) {
-      const int n = (my_count + tile_rows - 1) / tile_rows;
-      for (int i = 0; i < n; ++i) {
-        tile_expert[first_tile[tid] + i] = tid;
-        tile_row0[first_tile[tid] + i] = first_row[tid] + i * tile_rows;
+      const int n = (counts[e] + tile_rows - 1) / tile_rows;
+      for (int i = lane; i < n; i += 64) {
+        tile_expert[first_tile[e] + i] = e;
+        tile_row0[first_tile[e] + i] = first_row[e] + i * tile_rows;
       }
     }
   }
