@@ -11,6 +11,7 @@ from __future__ import annotations
 from collections import Counter
 from typing import List, Sequence, Tuple
 
+import numpy as np
 import torch
 
 from .. import ops
@@ -58,15 +59,18 @@ class Sampler:
         if all(p.temperature <= 0 for p, _, _ in rows):
             ops.argmax(logits, out)
         else:
-            to_i64 = lambda v: v - (1 << 64) if v >= (1 << 63) else v
-            ops.sample(
-                logits, out,
-                self._dev([p.temperature for p, _, _ in rows], torch.float32),
-                self._dev([p.top_p for p, _, _ in rows], torch.float32),
-                self._dev([p.top_k for p, _, _ in rows], torch.int32),
-                self._dev([p.min_p for p, _, _ in rows], torch.float32),
-                self._dev([to_i64(p.seed % (1 << 64)) for p, _, _ in rows], torch.int64),
-                self._dev([n for _, n, _ in rows], torch.int64))
+            # all per-row settings in one upload: four 32-bit columns, then two 64-bit ones
+            host = np.empty(8 * R, dtype=np.int32)
+            host[0:R].view(np.float32)[:] = [p.temperature for p, _, _ in rows]
+            host[R:2 * R].view(np.float32)[:] = [p.top_p for p, _, _ in rows]
+            host[2 * R:3 * R] = [p.top_k for p, _, _ in rows]
+            host[3 * R:4 * R].view(np.float32)[:] = [p.min_p for p, _, _ in rows]
+            host[4 * R:6 * R].view(np.uint64)[:] = [p.seed % (1 << 64) for p, _, _ in rows]
+            host[6 * R:8 * R].view(np.uint64)[:] = [n for _, n, _ in rows]
+            dev = torch.from_numpy(host).to(self.rt.device)
+            ops.sample(logits, out, dev[0:R].view(torch.float32), dev[R:2 * R].view(torch.float32), dev[2 * R:3 * R],
+                       dev[3 * R:4 * R].view(torch.float32), dev[4 * R:6 * R].view(torch.int64),
+                       dev[6 * R:8 * R].view(torch.int64))
         self.last_logprobs = None
         if any(p.want_logprobs or p.top_logprobs for p, _, _ in rows):
             n_top = max(p.top_logprobs for p, _, _ in rows)

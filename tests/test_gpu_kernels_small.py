@@ -259,6 +259,54 @@ def test_random_settings_stay_in_the_support_and_repeat(settings):
     assert len({draw(logits, 0.8, seed=1, counter=c, **settings)[0] for c in range(40)}) > 1 or len(support) == 1
 
 
+@pytest.mark.parametrize("settings", [dict(top_k=40), dict(top_p=0.9), dict(top_k=500, top_p=0.95, min_p=0.001),
+                                      dict(min_p=0.05), dict(top_k=100000)])
+@pytest.mark.parametrize("spread", [3.0, 1e-3])
+def test_cut_offs_on_a_real_vocabulary(settings, spread):
+    """151,936 logits, broad (the boundary's bin of the first histogram is small) and nearly uniform (all tokens
+    fall into one or two bins, which are cut finer twice): every draw lies in the plain implementation's support,
+    and with many seeds the draws reach beyond the most probable tokens."""
+    V = 151936
+    logits = rnd(2, V, seed=11, scale=spread)
+    supports = [set(pm.sampling_support(logits[r].cpu(), 0.8, **settings)) for r in range(2)]
+    seen = [set(), set()]
+    for seed in range(24):
+        got = draw(logits, 0.8, seed=seed, counter=seed * 7, **settings)
+        assert got == draw(logits, 0.8, seed=seed, counter=seed * 7, **settings)
+        for r in range(2):
+            assert got[r] in supports[r], (settings, spread, seed, r, got[r], len(supports[r]))
+            seen[r].add(got[r])
+    assert all(len(s) > 3 for s in seen)
+
+
+def test_cut_offs_with_many_equal_logits():
+    """Three distinct values, tens of thousands of tokens each: tokens that cannot be told apart stay together, so
+    the support is every token at least as probable as the boundary token (the plain implementation cuts the ties
+    by index)."""
+    V = 90000
+    logits = torch.full((1, V), -2.0, device=DEV)
+    logits[0, 1::3] = 1.0
+    logits[0, 2::3] = 0.5
+    exact = set(pm.sampling_support(logits[0].cpu(), 1.0, top_k=40000))
+    with_ties = set(range(1, V, 3)) | set(range(2, V, 3))  # 30,000 + 30,000: the boundary lies among the second value
+    assert exact < with_ties
+    seen = set()
+    for seed in range(30):
+        tok = draw(logits, 1.0, top_k=40000, seed=seed)[0]
+        assert tok in with_ties
+        seen.add(tok % 3)
+    assert seen == {1, 2}
+    for seed in range(10):
+        assert draw(logits, 1.0, top_k=2000, seed=seed)[0] % 3 == 1  # the rank falls among the first value's tokens
+    # up to 2,048 equal tokens are ranked exactly, by index like the plain implementation
+    few = torch.full((1, 5000), -3.0, device=DEV)
+    few[0, 7::5] = 2.0  # 999 tokens tied at the top
+    exact = set(pm.sampling_support(few[0].cpu(), 1.0, top_k=300))
+    assert exact == set(range(7, 7 + 5 * 300, 5))
+    seen = {draw(few, 1.0, top_k=300, seed=seed)[0] for seed in range(60)}
+    assert seen <= exact and len(seen) > 20
+
+
 def test_sampling_follows_the_distribution():
     logits = torch.tensor([[2.0, 1.0, 0.0, -1.0]], device=DEV)
     p = torch.softmax(logits[0].cpu().double() / 0.9, -1)
