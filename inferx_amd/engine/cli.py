@@ -38,7 +38,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--kv-cache-memory-bytes", type=int, default=None, help="explicit cache budget in bytes")
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.92,
                     help="fraction of GPU memory the engine may use")
-    ap.add_argument("--enforce-eager", action="store_true", help="accepted; the engine launches kernels eagerly")
+    ap.add_argument("--enforce-eager", action="store_true", help="no captured HIP graphs: every step launches its kernels one by one")
     ap.add_argument("--device", default="rocm", choices=["rocm", "cuda"], help="execution backend (one GPU)")
     ap.add_argument("--prompt-ids", action="append", default=[], help="a prompt as token ids, e.g. 1,2,3 (repeatable)")
     ap.add_argument("--prompt-file", help="file with one prompt of token ids per line")
@@ -94,7 +94,7 @@ def main(argv: Optional[List[str]] = None) -> int:
                            max_num_batched_tokens=args.max_num_batched_tokens, block_size=args.block_size,
                            num_gpu_blocks_override=args.num_gpu_blocks_override,
                            kv_cache_memory_bytes=args.kv_cache_memory_bytes,
-                           gpu_memory_utilization=args.gpu_memory_utilization)
+                           gpu_memory_utilization=args.gpu_memory_utilization, enforce_eager=args.enforce_eager)
         params = SamplingParams(max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p,
                                 top_k=args.top_k, min_p=args.min_p, presence_penalty=args.presence_penalty,
                                 frequency_penalty=args.frequency_penalty,

@@ -70,7 +70,8 @@ class LLMEngine:
     def __init__(self, model: str, dtype: str = "bfloat16", *, max_num_seqs: int = 8, max_model_len: int = 2048,
                  max_num_batched_tokens: Optional[int] = None, block_size: int = 16,
                  num_gpu_blocks_override: Optional[int] = None, kv_cache_memory_bytes: Optional[int] = None,
-                 gpu_memory_utilization: float = 0.92, device: str = "cuda:0", runner: Optional[ModelRunner] = None):
+                 gpu_memory_utilization: float = 0.92, device: str = "cuda:0", enforce_eager: bool = False,
+                 runner: Optional[ModelRunner] = None):
         if max_num_batched_tokens is None:
             max_num_batched_tokens = max(2048, max_model_len)  # reference: options.cc:332-336
         if runner is None:
@@ -80,7 +81,7 @@ class LLMEngine:
             weights = load_weights(net, model, rt)
             # page count needs the per-token bytes, which need the cache plan: lay out with one page, then size
             probe = ModelRunner(config, weights, rt, page_size=block_size, num_pages=1, max_requests=max_num_seqs,
-                                max_seq_len=max_model_len, model=net)
+                                max_seq_len=max_model_len, model=net, use_graphs=not enforce_eager)
             block_bytes = probe.kv_bytes_per_token() * block_size
             free, total = torch.cuda.mem_get_info(rt.device)
             pages = resolve_kv_blocks(max(block_bytes, 1), explicit_blocks=num_gpu_blocks_override,

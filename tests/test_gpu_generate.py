@@ -170,6 +170,22 @@ def test_far_key_and_window_edge_show_in_the_logits(tmp_path):
         ru.compare(ru.replay(runner, steps), {"r": whole}, ru.FP32_TOL, "peaked attention")
 
 
+def test_enforce_eager_gives_the_same_tokens_without_graphs(tmp_path):
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_A, 41, str(tmp_path), "bfloat16")
+    cfg, _ = tiny.read_folder(str(tmp_path))
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 70 + n) for n in (5, 18)]
+    outs = []
+    for eager in (False, True):
+        engine = LLMEngine(str(tmp_path), "bfloat16", max_num_seqs=2, max_model_len=64, num_gpu_blocks_override=12,
+                           enforce_eager=eager)
+        assert engine.runner.use_graphs == (not eager)
+        outs.append(engine.generate(prompts, SamplingParams(max_tokens=10)))
+        assert bool(engine.runner._graphs) == (not eager)
+    assert outs[0] == outs[1]
+
+
 def test_command_line(tmp_path):
     tiny.make_folder(tiny.CONFIG_A, 37, str(tmp_path), "float32")
     cfg, weights = tiny.read_folder(str(tmp_path))
