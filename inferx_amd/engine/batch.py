@@ -42,6 +42,7 @@ class StepBatch:
     slots: List[np.ndarray]          # per group [T]
     block_tables: List[np.ndarray]   # per group [S, max_blocks], -1 where no page is held
     request_ids: List[Hashable]
+    laid_out_by_manager: bool = False  # True: the host library built it, so only the token ids are unchecked
 
     @property
     def num_tokens(self) -> int:
@@ -53,14 +54,16 @@ class StepBatch:
 
     def validate(self, vocab_size: int, pages_per_group: Sequence[int], page_size: int) -> None:
         T, S = self.num_tokens, self.num_requests
+        if T and (self.token_ids.min() < 0 or self.token_ids.max() >= vocab_size):
+            bad = self.token_ids[(self.token_ids < 0) | (self.token_ids >= vocab_size)][0]
+            raise BatchError(f"token id {int(bad)} is outside the vocabulary of {vocab_size}")
+        if self.laid_out_by_manager:
+            return
         for name in ("positions", "seq_of_token"):
             if getattr(self, name).shape != (T,):
                 raise BatchError(f"{name} must hold one entry per token")
         if self.q_start.shape != (S + 1,) or self.q_start[0] != 0 or self.q_start[-1] != T:
             raise BatchError("q_start must run from 0 to the number of tokens")
-        if T and (self.token_ids.min() < 0 or self.token_ids.max() >= vocab_size):
-            bad = self.token_ids[(self.token_ids < 0) | (self.token_ids >= vocab_size)][0]
-            raise BatchError(f"token id {int(bad)} is outside the vocabulary of {vocab_size}")
         n = self.q_start[1:].astype(np.int64) - self.q_start[:-1]
         if S and n.min() < 0:
             raise BatchError("q_start must not descend")
@@ -132,4 +135,5 @@ def build_step_batch(cache: CacheManager, entries: Sequence[Entry]) -> StepBatch
             raise OutOfPages(rid, RESERVE_POOL_EMPTY if rc == 1 else RESERVE_CONTEXT_FULL)
         raise BatchError(f"request {rid!r} " + cache._lib.ixh_cache_error(cache._h).decode("utf-8", "replace"))
     return StepBatch(token_ids, positions, seq_of_token, q_start, seq_lens, state_slots, logits_rows,
-                     [slots[g] for g in range(G)], [tables[g] for g in range(G)], [e[0] for e in entries])
+                     [slots[g] for g in range(G)], [tables[g] for g in range(G)], [e[0] for e in entries],
+                     laid_out_by_manager=True)

@@ -31,13 +31,17 @@ from .runtime import CacheBinding, Runtime, StepContext
 N_FIXED = 7  # token_ids, positions, seq_of_token, q_start, seq_lens, state_slots, logits_rows
 
 
-def _pack(batch: StepBatch) -> Tuple[List[int], np.ndarray]:
+def _pack(batch: StepBatch, out: Optional[np.ndarray] = None) -> Tuple[List[int], np.ndarray]:
+    """The batch's arrays one after the other as int32; into `out` if it is given and has their size."""
     parts = [batch.token_ids, batch.positions, batch.seq_of_token, batch.q_start, batch.seq_lens,
              batch.state_slots, batch.logits_rows] + list(batch.slots) + [t.reshape(-1) for t in batch.block_tables]
     sizes = [int(p.size) for p in parts]
     if not sum(sizes):
         return sizes, np.zeros(0, np.int32)
-    return sizes, np.concatenate([np.ascontiguousarray(p, dtype=np.int32).reshape(-1) for p in parts])
+    flat = [np.ascontiguousarray(p, dtype=np.int32).reshape(-1) for p in parts]
+    if out is not None and out.size == sum(sizes):
+        return sizes, np.concatenate(flat, out=out)
+    return sizes, np.concatenate(flat)
 
 
 class ModelRunner:
@@ -215,16 +219,21 @@ class _DecodeGraph:
     def _fill(self, flat: np.ndarray) -> None:
         self.copied.synchronize()  # the pinned buffer is free again
         self.host_np[:] = flat
+        self._send()
+
+    def _send(self) -> None:
         self.dev.copy_(self.host, non_blocking=True)
         self.copied.record()
 
     def run(self, batch: StepBatch) -> torch.Tensor:
-        sizes, flat = _pack(self._with_all_rows(batch))
+        T = batch.num_tokens
+        self.copied.synchronize()  # the pinned buffer is free again
+        sizes, _ = _pack(self._with_all_rows(batch), out=self.host_np)
         if sizes != self.sizes:
             raise RuntimeError("a captured step was given a batch of another shape")
-        self._fill(flat)
+        self._send()
         self.graph.replay()
         rows = batch.logits_rows
-        if len(rows) == batch.num_tokens and np.array_equal(rows, np.arange(batch.num_tokens)):
+        if len(rows) == T and (T == 0 or (rows[0] == 0 and rows[-1] == T - 1 and np.all(rows[1:] > rows[:-1]))):
             return self.logits.clone()
         return self.logits[torch.from_numpy(rows.astype(np.int64)).to(self.logits.device)]
