@@ -29,52 +29,46 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define TL_WROWS 128
 #define TL_K 64
 #define TL_STRIDE 72  // elements per LDS row: 64 + 8 of padding
-#define TL_XPER (TL_ROWS * 8 / 256)  // 16-byte pieces of activations per thread and stage
-#define TL_XBLK (TL_ROWS / 32)       // sixteens of activation rows per wavefront
 
-template <bool GATE_UP>
-__global__ void __launch_bounds__(256)
-moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w, __bf16* __restrict__ out,
-                         const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
-                         const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
-                         const int32_t* __restrict__ tile_info, int n_out, int width) {
-  __shared__ __attribute__((aligned(16))) __bf16 ws[TL_WROWS * TL_STRIDE];
-  __shared__ __attribute__((aligned(16))) __bf16 xs[TL_ROWS * TL_STRIDE];
-  if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
+// One row tile x 128 weight rows.  NP: pairs of sixteens of activation rows the tile holds (1..5); with it a
+// template parameter, and every load unconditional (a stage past the end asks for the last stage again, a piece
+// past the row's end for the row's start, and what comes back is replaced by zero on its way into LDS), the loop is one straight line, so the
+// compiler can count exactly how many loads may stay in flight at each wait.  With branches in the loop it
+// waited for all of them, also those of three stages ahead.
+template <bool GATE_UP, int NP>
+__device__ __forceinline__ void
+tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ rows, int n_out, int width, int e, int row0, int row_end, __bf16* ws,
+           __bf16* xs) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
   const int wi = wave & 1, xi = wave >> 1;
-  const int e = tile_expert[blockIdx.y];
-  const int row0 = tile_row0[blockIdx.y];
-  const int row_end = offsets[e + 1];
-  const int nblk = (min(TL_ROWS, row_end - row0) + 15) >> 4;  // sixteens of rows this tile holds
   constexpr int COLS = GATE_UP ? 64 : 128;  // output columns of this workgroup
   const int n0 = blockIdx.x * COLS;
 
-  // what this thread copies per stage: 4 pieces of 8 weights, up to TL_XPER pieces of 8 activations
+  // what this thread copies per stage: 4 pieces of 8 weights, NP pieces of 8 activations
   const int64_t w_rows = GATE_UP ? 2 * static_cast<int64_t>(n_out) : n_out;
   // (32-bit offsets: the entry point has checked that one expert's weights and the activations stay below 2^31)
   const __bf16* w_expert = w + static_cast<int64_t>(e) * w_rows * width;
+  const int kc_mine = (tid & 7) * 8;  // the same for all of this thread's pieces
   int wsrc[4], wdst[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int c = tid + 256 * i, r = c >> 3, kc = (c & 7) * 8;
+    const int c = tid + 256 * i, r = c >> 3;
     int src_row;
     if (GATE_UP)
       src_row = (r < 64 ? 0 : n_out) + min(n0 + (r & 63), n_out - 1);
     else
       src_row = min(n0 + r, n_out - 1);
-    wsrc[i] = src_row * width + kc;
-    wdst[i] = r * TL_STRIDE + kc;
+    wsrc[i] = src_row * width;
+    wdst[i] = r * TL_STRIDE + kc_mine;
   }
-  int xsrc[TL_XPER];
+  int xsrc[NP];
 #pragma unroll
-  for (int i = 0; i < TL_XPER; ++i) {
+  for (int i = 0; i < NP; ++i) {
     const int r = (tid >> 3) + 32 * i;
     const int gr = min(row0 + r, row_end - 1);  // rows past the end repeat the last one; their results are dropped
-    xsrc[i] = (rows ? rows[gr] : gr) * width + (tid & 7) * 8;
+    xsrc[i] = (rows ? rows[gr] : gr) * width;
   }
-  const int kc_mine = (tid & 7) * 8;  // the same for all of this thread's pieces
   const int xdst = (tid >> 3) * TL_STRIDE + kc_mine;
 
   const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
@@ -82,7 +76,7 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
   // The weights come from memory and are what the kernel waits for: three register sets keep the loads of three
   // stages on their way while a fourth stage is multiplied out of LDS.  The activations are asked for two stages
   // ahead, in two sets.
-  bf16x8 wreg[3][4], xreg[2][TL_XPER];
+  bf16x8 wreg[3][4], xreg[2][NP];
   // Row tiles walk the reduction in the same order but start at different stages (and wrap round): were all
   // workgroups at the same offset of their weight rows at the same time, a row length that is a power of two
   // would send their loads to the same few memory channels (measured with few rows per expert: 4.0 instead of
@@ -92,37 +86,49 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
   const int rot = (width % 512 == 0)  // rows of a multiple of 1,024 bytes; workgroups of one row tile stay together
                       ? static_cast<int>((blockIdx.y * 3u) % static_cast<unsigned>(kspan / TL_K)) * TL_K
                       : 0;         // (they read the same activations, which then stay in L2)
-  auto turned = [&](int k0) { return k0 + rot < kspan ? k0 + rot : k0 + rot - kspan; };
+  // where this thread's pieces of stage k0 start in a row, and whether they exist
+  auto place = [&](int k0, bool& ok) {
+    k0 = min(k0, kspan - TL_K);
+    const int k = (k0 + rot < kspan ? k0 + rot : k0 + rot - kspan) + kc_mine;
+    ok = k < width;
+    return ok ? k : 0;
+  };
   auto fetch_w = [&](int k0, bf16x8 (&wr)[4]) {
-    k0 = turned(k0);
-    const bool ok = k0 + kc_mine < width;
+    bool ok;
+    const int k = place(k0, ok);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) wr[i] = ok ? *reinterpret_cast<const bf16x8*>(w_expert + wsrc[i] + k0) : zero;
+    for (int i = 0; i < 4; ++i) {
+      wr[i] = *reinterpret_cast<const bf16x8*>(w_expert + wsrc[i] + k);
+    }
   };
-  auto fetch_x = [&](int k0, bf16x8 (&xr)[TL_XPER]) {
-    k0 = turned(k0);
-    const bool ok = k0 + kc_mine < width;
+  auto fetch_x = [&](int k0, bf16x8 (&xr)[NP]) {
+    bool ok;
+    const int k = place(k0, ok);
 #pragma unroll
-    for (int i = 0; i < TL_XPER; ++i)  // piece i lies in sixteens 2 i and 2 i + 1 (uniform over the workgroup)
-      if (2 * i < nblk) xr[i] = ok ? *reinterpret_cast<const bf16x8*>(a + xsrc[i] + k0) : zero;
+    for (int i = 0; i < NP; ++i) {
+      xr[i] = *reinterpret_cast<const bf16x8*>(a + xsrc[i] + k);
+    }
   };
-  auto stage = [&](const bf16x8 (&wr)[4], const bf16x8 (&xr)[TL_XPER]) {
+  // (what was loaded for a piece that does not exist becomes zero here, not at the load: the loads' results are
+  // not touched before they are needed)
+  auto stage = [&](int k0, const bf16x8 (&wr)[4], const bf16x8 (&xr)[NP]) {
+    bool ok;
+    place(k0, ok);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + wdst[i]) = wr[i];
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + wdst[i]) = ok ? wr[i] : zero;
 #pragma unroll
-    for (int i = 0; i < TL_XPER; ++i)
-      if (2 * i < nblk) *reinterpret_cast<bf16x8*>(xs + xdst + 32 * i * TL_STRIDE) = xr[i];
+    for (int i = 0; i < NP; ++i) *reinterpret_cast<bf16x8*>(xs + xdst + 32 * i * TL_STRIDE) = ok ? xr[i] : zero;
   };
 
   // weight blocks of this wavefront: gate|up 32 wi + {0, 16} and the same + 64; down 64 wi + 16 j
   int wblock[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) wblock[j] = GATE_UP ? 32 * wi + 16 * (j & 1) + 64 * (j >> 1) : 64 * wi + 16 * j;
-  f32x4 acc[4][TL_XBLK];
+  f32x4 acc[4][NP];
 #pragma unroll
   for (int j = 0; j < 4; ++j)
 #pragma unroll
-    for (int t = 0; t < TL_XBLK; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = 0; t < NP; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   auto multiply = [&]() {
 #pragma unroll
@@ -132,8 +138,7 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
 #pragma unroll
       for (int j = 0; j < 4; ++j) wa[j] = *reinterpret_cast<const bf16x8*>(ws + (wblock[j] + m) * TL_STRIDE + col);
 #pragma unroll
-      for (int t = 0; t < TL_XBLK; ++t) {
-        if (2 * t + xi >= nblk) continue;  // uniform over the wavefront
+      for (int t = 0; t < NP; ++t) {  // sixteen 2 t + xi (an odd count of sixteens: the last one of xi = 1 is idle work)
         const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xs + (16 * (2 * t + xi) + m) * TL_STRIDE + col);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[j], xb, acc[j][t], 0, 0, 0);
@@ -143,27 +148,27 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
 
   fetch_w(0, wreg[0]);
   fetch_x(0, xreg[0]);
-  stage(wreg[0], xreg[0]);
-  if (TL_K < width) {
-    fetch_w(TL_K, wreg[1]);
-    fetch_x(TL_K, xreg[1]);
-  }
-  if (2 * TL_K < width) fetch_w(2 * TL_K, wreg[2]);
+  stage(0, wreg[0], xreg[0]);
+  fetch_w(TL_K, wreg[1]);
+  fetch_x(TL_K, xreg[1]);
+  fetch_w(2 * TL_K, wreg[2]);
   __syncthreads();
   // One stage s: ask for the weights of stage s + 3 and the activations of stage s + 2 (into the sets that held
   // stage s, which is in LDS), multiply, then move stage s + 1 into LDS.  Six stages per turn, so that the
   // register sets (three of weights, two of activations) are named statically.
 #define TL_STAGE(K0, W_FREE, W_NEXT, X_FREE, X_NEXT)                              \
   {                                                                               \
-    if ((K0) + 3 * TL_K < width) fetch_w((K0) + 3 * TL_K, wreg[W_FREE]);          \
-    if ((K0) + 2 * TL_K < width) fetch_x((K0) + 2 * TL_K, xreg[X_FREE]);          \
+    fetch_w((K0) + 3 * TL_K, wreg[W_FREE]);                                       \
+    fetch_x((K0) + 2 * TL_K, xreg[X_FREE]);                                       \
+    __builtin_amdgcn_sched_barrier(0); /* the loads stay ahead of the products */ \
     multiply();                                                                   \
+    __builtin_amdgcn_sched_barrier(0);                                            \
     __syncthreads();                                                              \
     if ((K0) + TL_K >= width) break;                                              \
-    stage(wreg[W_NEXT], xreg[X_NEXT]);                                            \
+    stage((K0) + TL_K, wreg[W_NEXT], xreg[X_NEXT]);                               \
     __syncthreads();                                                              \
   }
-  for (int k0 = 0; k0 < width; k0 += 6 * TL_K) {
+  for (int k0 = 0;; k0 += 6 * TL_K) {
     TL_STAGE(k0, 0, 1, 0, 1)
     TL_STAGE(k0 + TL_K, 1, 2, 1, 0)
     TL_STAGE(k0 + 2 * TL_K, 2, 0, 0, 1)
@@ -176,9 +181,9 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
   // lane holds weight rows (block) + 4 g + i of activation row row0 + 16 (2 t + xi) + m
   const bool vec = (n_out & 3) == 0;
 #pragma unroll
-  for (int t = 0; t < TL_XBLK; ++t) {
+  for (int t = 0; t < NP; ++t) {
     const int r = row0 + 16 * (2 * t + xi) + m;
-    if (2 * t + xi >= nblk || r >= row_end) continue;
+    if (r >= row_end) continue;
     if (GATE_UP) {
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
@@ -214,6 +219,28 @@ moe_grouped_tiled_kernel(const __bf16* __restrict__ a, const __bf16* __restrict_
         }
       }
     }
+  }
+}
+
+template <bool GATE_UP>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
+                         const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
+                         const int32_t* __restrict__ tile_info, int n_out, int width) {
+  __shared__ __attribute__((aligned(16))) __bf16 ws[TL_WROWS * TL_STRIDE];
+  __shared__ __attribute__((aligned(16))) __bf16 xs[TL_ROWS * TL_STRIDE];
+  if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
+  const int e = tile_expert[blockIdx.y];
+  const int row0 = tile_row0[blockIdx.y];
+  const int row_end = offsets[e + 1];
+  const int held = min(TL_ROWS, row_end - row0);
+  if (held <= 0) return;
+  switch ((held + 31) >> 5) {  // pairs of sixteens of rows this tile holds
+    case 1: tiled_body<GATE_UP, 1>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
+    case 2: tiled_body<GATE_UP, 2>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
+    case 3: tiled_body<GATE_UP, 3>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
+    case 4: tiled_body<GATE_UP, 4>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
+    default: tiled_body<GATE_UP, 5>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
   }
 }
 
