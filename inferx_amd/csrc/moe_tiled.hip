@@ -7,11 +7,13 @@
 // kernel's map; with a few hundred tokens that is all rows of the expert, so
 // its weights are read once) x 128 weight rows: for the gate|up product 64 gate
 // rows and the 64 up rows that belong to them (64 output columns after SwiGLU),
-// for the down product 128 output columns.  Only the sixteens of rows that the
-// tile really holds are multiplied.  The reduction runs in stages of 64: the
-// next stage's global loads are issued into registers before the current stage
-// is multiplied out of LDS.  LDS rows are padded to 144 bytes so that the
-// 16-byte operand reads of a wavefront quarter fall on distinct banks.
+// for the down product 128 output columns.  Only the pairs of sixteens of rows
+// that the tile really holds are multiplied.  The reduction runs in stages of
+// 64 through two LDS buffers: while one stage is multiplied, the next one is
+// already in the other buffer, the weights of three further stages and the
+// activations of two are on their way from memory into registers, and one
+// barrier per stage is enough.  LDS rows are 128 bytes with their 16-byte
+// pieces permuted, so that operand reads and writes fall on distinct banks.
 //
 // As in moe_mfma.hip the product is formed transposed (A = weight rows,
 // B = activation rows), so lane l ends up with four consecutive output
@@ -28,7 +30,12 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 #define TL_ROWS 160   // the row-tile map is made for tiles of this many rows
 #define TL_WROWS 128
 #define TL_K 64
-#define TL_STRIDE 72  // elements per LDS row: 64 + 8 of padding
+#define TL_STRIDE 64  // elements per LDS row: no padding; the eight 16-byte pieces of a row are stored permuted
+#define TL_WTILE (TL_WROWS * TL_STRIDE)
+#define TL_XTILE (TL_ROWS * TL_STRIDE)
+// piece p of row r lies at piece p ^ ((r >> 1) & 7): the sixteen rows that a quarter of a wavefront reads at one
+// piece index then fall on sixteen different groups of four banks, as do the pieces that sixteen lanes write
+__device__ __forceinline__ int tl_at(int row, int piece) { return row * TL_STRIDE + ((piece ^ ((row >> 1) & 7)) << 3); }
 
 // One row tile x 128 weight rows.  NP: pairs of sixteens of activation rows the tile holds (1..5); with it a
 // template parameter, and every load unconditional (a stage past the end asks for the last stage again, a piece
@@ -37,20 +44,20 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // waited for all of them, also those of three stages ahead.
 template <bool GATE_UP, int NP>
 __device__ __forceinline__ void
-tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ rows, int n_out, int width, int e, int row0, int row_end, __bf16* ws,
+tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ rows, int n_out, int width, int e, int row0, int row_end, int tile, int col_block, __bf16* ws,
            __bf16* xs) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
   const int wi = wave & 1, xi = wave >> 1;
   constexpr int COLS = GATE_UP ? 64 : 128;  // output columns of this workgroup
-  const int n0 = blockIdx.x * COLS;
+  const int n0 = col_block * COLS;
 
   // what this thread copies per stage: 4 pieces of 8 weights, NP pieces of 8 activations
   const int64_t w_rows = GATE_UP ? 2 * static_cast<int64_t>(n_out) : n_out;
   // (32-bit offsets: the entry point has checked that one expert's weights and the activations stay below 2^31)
   const __bf16* w_expert = w + static_cast<int64_t>(e) * w_rows * width;
   const int kc_mine = (tid & 7) * 8;  // the same for all of this thread's pieces
-  int wsrc[4], wdst[4];
+  int wsrc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const int c = tid + 256 * i, r = c >> 3;
@@ -60,7 +67,6 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
     else
       src_row = min(n0 + r, n_out - 1);
     wsrc[i] = src_row * width;
-    wdst[i] = r * TL_STRIDE + kc_mine;
   }
   int xsrc[NP];
 #pragma unroll
@@ -69,10 +75,8 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
     const int gr = min(row0 + r, row_end - 1);  // rows past the end repeat the last one; their results are dropped
     xsrc[i] = (rows ? rows[gr] : gr) * width;
   }
-  const int xdst = (tid >> 3) * TL_STRIDE + kc_mine;
+  const int xdst = tl_at(tid >> 3, tid & 7);  // rows 32 further on have the same permutation
 
-  const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
-                       (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
   // The weights come from memory and are what the kernel waits for: three register sets keep the loads of three
   // stages on their way while a fourth stage is multiplied out of LDS.  The activations are asked for two stages
   // ahead, in two sets.
@@ -84,9 +88,13 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
   // grid, so results repeat bit for bit.
   const int kspan = ((width + TL_K - 1) / TL_K) * TL_K;
   const int rot = (width % 512 == 0)  // rows of a multiple of 1,024 bytes; workgroups of one row tile stay together
-                      ? static_cast<int>((blockIdx.y * 3u) % static_cast<unsigned>(kspan / TL_K)) * TL_K
+                      ? static_cast<int>((static_cast<unsigned>(tile) * 3u) % static_cast<unsigned>(kspan / TL_K)) * TL_K
                       : 0;         // (they read the same activations, which then stay in L2)
-  // where this thread's pieces of stage k0 start in a row, and whether they exist
+  // Where this thread's pieces of stage k0 start in a row, and whether they exist.  A piece that does not exist
+  // (the reduction width is no multiple of 64) is loaded from the row's start instead and overwritten with
+  // zeros in LDS by the thread that put it there: no loaded value is touched before its use, and the only
+  // branch, in the last stage, holds nothing but LDS writes.
+  const bool ragged = (width & (TL_K - 1)) != 0;
   auto place = [&](int k0, bool& ok) {
     k0 = min(k0, kspan - TL_K);
     const int k = (k0 + rot < kspan ? k0 + rot : k0 + rot - kspan) + kc_mine;
@@ -97,84 +105,111 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
     bool ok;
     const int k = place(k0, ok);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      wr[i] = *reinterpret_cast<const bf16x8*>(w_expert + wsrc[i] + k);
-    }
+    for (int i = 0; i < 4; ++i) wr[i] = *reinterpret_cast<const bf16x8*>(w_expert + wsrc[i] + k);
   };
   auto fetch_x = [&](int k0, bf16x8 (&xr)[NP]) {
     bool ok;
     const int k = place(k0, ok);
 #pragma unroll
-    for (int i = 0; i < NP; ++i) {
-      xr[i] = *reinterpret_cast<const bf16x8*>(a + xsrc[i] + k);
+    for (int i = 0; i < NP; ++i) xr[i] = *reinterpret_cast<const bf16x8*>(a + xsrc[i] + k);
+  };
+  auto stage = [&](int k0, int buf, const bf16x8 (&wr)[4], const bf16x8 (&xr)[NP]) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + buf * TL_WTILE + xdst + 32 * i * TL_STRIDE) = wr[i];
+#pragma unroll
+    for (int i = 0; i < NP; ++i) *reinterpret_cast<bf16x8*>(xs + buf * TL_XTILE + xdst + 32 * i * TL_STRIDE) = xr[i];
+    if (ragged) {
+      bool ok;
+      place(k0, ok);
+      if (!ok) {
+        const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
+                             (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + buf * TL_WTILE + xdst + 32 * i * TL_STRIDE) = zero;
+#pragma unroll
+        for (int i = 0; i < NP; ++i)
+          *reinterpret_cast<bf16x8*>(xs + buf * TL_XTILE + xdst + 32 * i * TL_STRIDE) = zero;
+      }
     }
   };
-  // (what was loaded for a piece that does not exist becomes zero here, not at the load: the loads' results are
-  // not touched before they are needed)
-  auto stage = [&](int k0, const bf16x8 (&wr)[4], const bf16x8 (&xr)[NP]) {
-    bool ok;
-    place(k0, ok);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + wdst[i]) = ok ? wr[i] : zero;
-#pragma unroll
-    for (int i = 0; i < NP; ++i) *reinterpret_cast<bf16x8*>(xs + xdst + 32 * i * TL_STRIDE) = ok ? xr[i] : zero;
-  };
 
-  // weight blocks of this wavefront: gate|up 32 wi + {0, 16} and the same + 64; down 64 wi + 16 j
-  int wblock[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) wblock[j] = GATE_UP ? 32 * wi + 16 * (j & 1) + 64 * (j >> 1) : 64 * wi + 16 * j;
   f32x4 acc[4][NP];
 #pragma unroll
   for (int j = 0; j < 4; ++j)
 #pragma unroll
     for (int t = 0; t < NP; ++t) acc[j][t] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  auto multiply = [&]() {
+  // this lane's operand pieces: row (block) + m, piece 4 kk + g.  Blocks start at multiples of 16 rows, so the
+  // permutation depends on m only and a block is a constant distance from the wavefront's first one.
+  int wat[2], xat[2];
+#pragma unroll
+  for (int kk = 0; kk < 2; ++kk) {
+    wat[kk] = tl_at((GATE_UP ? 32 : 64) * wi + m, 4 * kk + g);
+    xat[kk] = tl_at(16 * xi + m, 4 * kk + g);
+  }
+  auto multiply = [&](int buf) {
+    const __bf16* wt = ws + buf * TL_WTILE;
+    const __bf16* xt = xs + buf * TL_XTILE;
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
-      const int col = 32 * kk + 8 * g;
       bf16x8 wa[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) wa[j] = *reinterpret_cast<const bf16x8*>(ws + (wblock[j] + m) * TL_STRIDE + col);
+      for (int j = 0; j < 4; ++j) {  // gate|up: blocks 32 wi + {0, 16} and the same + 64; down: 64 wi + 16 j
+        const int block = GATE_UP ? 16 * (j & 1) + 64 * (j >> 1) : 16 * j;
+        wa[j] = *reinterpret_cast<const bf16x8*>(wt + wat[kk] + block * TL_STRIDE);
+      }
 #pragma unroll
       for (int t = 0; t < NP; ++t) {  // sixteen 2 t + xi (an odd count of sixteens: the last one of xi = 1 is idle work)
-        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xs + (16 * (2 * t + xi) + m) * TL_STRIDE + col);
+        const bf16x8 xb = *reinterpret_cast<const bf16x8*>(xt + xat[kk] + 32 * t * TL_STRIDE);
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[j][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wa[j], xb, acc[j][t], 0, 0, 0);
       }
     }
   };
 
+  // (the loads are asked for in the order in which the loop leaves them behind, so that the count of loads that
+  // may stay in flight at the loop's first wait is the same on the way in and on the way round)
   fetch_w(0, wreg[0]);
-  fetch_x(0, xreg[0]);
-  stage(0, wreg[0], xreg[0]);
+  __builtin_amdgcn_sched_barrier(0);
   fetch_w(TL_K, wreg[1]);
-  fetch_x(TL_K, xreg[1]);
+  __builtin_amdgcn_sched_barrier(0);
+  fetch_x(0, xreg[0]);
+  __builtin_amdgcn_sched_barrier(0);
   fetch_w(2 * TL_K, wreg[2]);
+  __builtin_amdgcn_sched_barrier(0);
+  fetch_x(TL_K, xreg[1]);
+  __builtin_amdgcn_sched_barrier(0);
+  stage(0, 0, wreg[0], xreg[0]);
+  fetch_w(3 * TL_K, wreg[0]);
+  __builtin_amdgcn_sched_barrier(0);
+  fetch_x(2 * TL_K, xreg[0]);
+  __builtin_amdgcn_sched_barrier(0);
   __syncthreads();
-  // One stage s: ask for the weights of stage s + 3 and the activations of stage s + 2 (into the sets that held
-  // stage s, which is in LDS), multiply, then move stage s + 1 into LDS.  Six stages per turn, so that the
+  // Stage s is in LDS buffer s & 1.  First stage s + 1 goes from its registers into the other buffer (whose last
+  // readers passed the previous barrier); the registers it leaves take the loads of the weights of stage s + 4 and
+  // the activations of stage s + 3; then stage s is multiplied; one barrier.  Six stages per turn, so that the
   // register sets (three of weights, two of activations) are named statically.
-#define TL_STAGE(K0, W_FREE, W_NEXT, X_FREE, X_NEXT)                              \
+#define TL_STAGE(K0, BUF, W_NEXT, X_NEXT)                                         \
   {                                                                               \
-    fetch_w((K0) + 3 * TL_K, wreg[W_FREE]);                                       \
-    fetch_x((K0) + 2 * TL_K, xreg[X_FREE]);                                       \
+    stage((K0) + TL_K, 1 - (BUF), wreg[W_NEXT], xreg[X_NEXT]);                    \
+    fetch_w((K0) + 4 * TL_K, wreg[W_NEXT]);                                       \
+    __builtin_amdgcn_sched_barrier(0);                                            \
+    fetch_x((K0) + 3 * TL_K, xreg[X_NEXT]);                                       \
     __builtin_amdgcn_sched_barrier(0); /* the loads stay ahead of the products */ \
-    multiply();                                                                   \
+    if ((K0) < kspan) multiply(BUF);                                              \
     __builtin_amdgcn_sched_barrier(0);                                            \
     __syncthreads();                                                              \
-    if ((K0) + TL_K >= width) break;                                              \
-    stage((K0) + TL_K, wreg[W_NEXT], xreg[X_NEXT]);                               \
-    __syncthreads();                                                              \
   }
-  for (int k0 = 0;; k0 += 6 * TL_K) {
-    TL_STAGE(k0, 0, 1, 0, 1)
-    TL_STAGE(k0 + TL_K, 1, 2, 1, 0)
-    TL_STAGE(k0 + 2 * TL_K, 2, 0, 0, 1)
-    TL_STAGE(k0 + 3 * TL_K, 0, 1, 1, 0)
-    TL_STAGE(k0 + 4 * TL_K, 1, 2, 0, 1)
-    TL_STAGE(k0 + 5 * TL_K, 2, 0, 1, 0)
+  // Whole turns only, and no way out of a turn's middle: a way out would join the states of the loads of all
+  // stages, and the loop's first wait would have to be for the worst of them.  Stages past the end ask for the
+  // last stage's operands again and multiply nothing (that branch holds no loads).
+  for (int k0 = 0; k0 < kspan; k0 += 6 * TL_K) {
+    TL_STAGE(k0, 0, 1, 1)
+    TL_STAGE(k0 + TL_K, 1, 2, 0)
+    TL_STAGE(k0 + 2 * TL_K, 0, 0, 1)
+    TL_STAGE(k0 + 3 * TL_K, 1, 1, 0)
+    TL_STAGE(k0 + 4 * TL_K, 0, 2, 1)
+    TL_STAGE(k0 + 5 * TL_K, 1, 0, 0)
   }
 #undef TL_STAGE
 
@@ -226,21 +261,25 @@ template <bool GATE_UP>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
 moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
                          const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
-                         const int32_t* __restrict__ tile_info, int n_out, int width) {
-  __shared__ __attribute__((aligned(16))) __bf16 ws[TL_WROWS * TL_STRIDE];
-  __shared__ __attribute__((aligned(16))) __bf16 xs[TL_ROWS * TL_STRIDE];
-  if (static_cast<int>(blockIdx.y) >= tile_info[0]) return;
-  const int e = tile_expert[blockIdx.y];
-  const int row0 = tile_row0[blockIdx.y];
+                         const int32_t* __restrict__ tile_info, int n_out, int width, int n_col_blocks) {
+  __shared__ __attribute__((aligned(16))) __bf16 ws[2 * TL_WTILE];
+  __shared__ __attribute__((aligned(16))) __bf16 xs[2 * TL_XTILE];
+  // Workgroups go to the chip's eight dies in turn, by their number.  All column blocks of a row tile read the
+  // same activations: they are numbered so that they land on one die and share its L2 (tile t on die t % 8).
+  const int slot = blockIdx.x >> 3;
+  const int tile = (slot / n_col_blocks) * 8 + (blockIdx.x & 7), col_block = slot % n_col_blocks;
+  if (tile >= tile_info[0]) return;
+  const int e = tile_expert[tile];
+  const int row0 = tile_row0[tile];
   const int row_end = offsets[e + 1];
   const int held = min(TL_ROWS, row_end - row0);
   if (held <= 0) return;
   switch ((held + 31) >> 5) {  // pairs of sixteens of rows this tile holds
-    case 1: tiled_body<GATE_UP, 1>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
-    case 2: tiled_body<GATE_UP, 2>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
-    case 3: tiled_body<GATE_UP, 3>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
-    case 4: tiled_body<GATE_UP, 4>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
-    default: tiled_body<GATE_UP, 5>(a, w, out, rows, n_out, width, e, row0, row_end, ws, xs); break;
+    case 1: tiled_body<GATE_UP, 1>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 2: tiled_body<GATE_UP, 2>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 3: tiled_body<GATE_UP, 3>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 4: tiled_body<GATE_UP, 4>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    default: tiled_body<GATE_UP, 5>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
   }
 }
 
@@ -257,12 +296,17 @@ extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, con
   IX_REQUIRE(max_tiles <= 65535, "too many row tiles for one launch");
   if (max_tiles == 0) return 0;
   const int cols = gate_up ? 64 : 128;
-  dim3 grid(static_cast<unsigned>((n_out + cols - 1) / cols), max_tiles), block(256);
+  const int n_col_blocks = static_cast<int>((n_out + cols - 1) / cols);
+  const int64_t groups = 8 * static_cast<int64_t>(n_col_blocks) * ((max_tiles + 7) / 8);
+  IX_REQUIRE(groups < (int64_t(1) << 31), "too many workgroups for one launch");
+  dim3 grid(static_cast<unsigned>(groups)), block(256);
   if (gate_up)
     hipLaunchKernelGGL(moe_grouped_tiled_kernel<true>, grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w,
-                       (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width);
+                       (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width,
+                       n_col_blocks);
   else
     hipLaunchKernelGGL(moe_grouped_tiled_kernel<false>, grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w,
-                       (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width);
+                       (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width,
+                       n_col_blocks);
   return ix_check_launch("ix_moe_grouped_tiled");
 }
