@@ -88,14 +88,24 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
   // (lane (dd = n, g) holds V^T[16 blk + dd][kb + 8 g .. +8])
   // a page size that is a power of two (page_shift >= 0, the usual case) spares the divisions
   auto page_of = [&](int key) { return page_shift >= 0 ? key >> page_shift : key / page_size; };
-  auto load_kv = [&](int kb, bf16x8 (&kf)[2][NC], bf16x8 (&vf)[NB]) {
+  // The pages of the 32 keys from kb on, as this lane needs them: for its row of the two key blocks and for its
+  // eight values.  They are looked up one iteration before the keys and values themselves are asked for, so that
+  // no load in the loop has to wait for another one's result.
+  auto ask_pages = [&](int kb, int (&pg)[3]) {
 #pragma unroll
     for (int b = 0; b < 2; ++b) {
-      int key = kb + 8 * (n >> 2) + 4 * b + (n & 3);  // A row n of block b
+      const int key = min(kb + 8 * (n >> 2) + 4 * b + (n & 3), hi - 1);  // A row n of block b
+      pg[b] = table[page_of(key)];
+    }
+    pg[2] = table[page_of(min(kb + 8 * g, hi - 1) & ~7)];
+  };
+  auto load_kv = [&](int kb, const int (&pg)[3], bf16x8 (&kf)[2][NC], bf16x8 (&vf)[NB]) {
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      int key = kb + 8 * (n >> 2) + 4 * b + (n & 3);
       key = min(key, hi - 1);                          // rows past the end are masked below
       const int pi = page_of(key);
-      int page = table[pi];
-      page = max(page, 0);                             // a page the window has passed: masked below
+      const int page = max(pg[b], 0);                  // a page the window has passed: masked below
       const __bf16* kr =
           k_cache + ((static_cast<int64_t>(page) * kv_heads + kvh) * page_size + (key - pi * page_size)) * D;
 #pragma unroll
@@ -107,9 +117,9 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
           for (int j = 0; j < 8; ++j) kf[b][c][j] = (__bf16)0.f;
       }
     }
-    int key = min(kb + 8 * g, hi - 1) & ~7;
+    const int key = min(kb + 8 * g, hi - 1) & ~7;
     const int pi = page_of(key);
-    int page = max(table[pi], 0);
+    const int page = max(pg[2], 0);
     const __bf16* vr = v_cache + (static_cast<int64_t>(page) * kv_heads + kvh) * D * page_size + (key - pi * page_size);
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -117,8 +127,13 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
   };
 
   bf16x8 kf_next[PF ? 2 : 1][PF ? NC : 1], vf_next[PF ? NB : 1];
-  if constexpr (PF) {
-    if (ks < ke) load_kv(ks, kf_next, vf_next);
+  int pg[3], pg_next[3];
+  if (ks < ke) {
+    ask_pages(ks, pg);
+    if constexpr (PF) {
+      ask_pages(ks + ATTN_KEYS_PER_ITER, pg_next);
+      load_kv(ks, pg, kf_next, vf_next);
+    }
   }
   for (int kb = ks; kb < ke; kb += ATTN_KEYS_PER_ITER) {
     bf16x8 kf[2][NC], vf[NB];
@@ -129,9 +144,15 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
         for (int c = 0; c < NC; ++c) kf[b][c] = kf_next[b][c];
 #pragma unroll
       for (int b = 0; b < NB; ++b) vf[b] = vf_next[b];
-      if (kb + ATTN_KEYS_PER_ITER < ke) load_kv(kb + ATTN_KEYS_PER_ITER, kf_next, vf_next);
+      if (kb + ATTN_KEYS_PER_ITER < ke) {
+        load_kv(kb + ATTN_KEYS_PER_ITER, pg_next, kf_next, vf_next);
+        ask_pages(kb + 2 * ATTN_KEYS_PER_ITER, pg_next);
+      }
     } else {
-      load_kv(kb, kf, vf);
+      ask_pages(kb + ATTN_KEYS_PER_ITER, pg_next);
+      load_kv(kb, pg, kf, vf);
+#pragma unroll
+      for (int i = 0; i < 3; ++i) pg[i] = pg_next[i];
     }
 #pragma unroll
     for (int t = 0; t < QT; ++t) {

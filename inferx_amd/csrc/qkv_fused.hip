@@ -14,7 +14,7 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 __global__ void __launch_bounds__(256)
-qkv_rope_skinny_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ w, const void* __restrict__ bias,
+qkv_rope_skinny_kernel(const __bf16* x, const __bf16* w, const void* __restrict__ bias,
                        int bias_dtype, const float2* __restrict__ cs, const int32_t* __restrict__ slots,
                        __bf16* __restrict__ q_out, __bf16* __restrict__ k_cache, __bf16* __restrict__ v_cache,
                        int tokens, int width, int heads, int kv_heads, int head_dim, int page_size,
@@ -35,20 +35,64 @@ qkv_rope_skinny_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ 
   const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
                        (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
   f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
-  for (int k0 = kbegin; k0 < kend; k0 += 128) {
-    bf16x8 fl[4], fh[4], fx[4];
+  // Steps of 128 of the reduction in two register sets: the loads of the next step are on their way while this
+  // one is multiplied.  Every load is unconditional (a piece past the end is read from the range's first piece
+  // instead, and its token values are replaced by zeros when they are used), so that the loop is one straight
+  // line and the compiler lets the younger loads stay in flight at each wait.
+  struct Step { bf16x8 fl[4], fh[4], fx[4]; };
+  Step one, two;
+  auto fetch = [&](int k0, Step& st) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row per load
-      const bool ok = kk < kend;
-      fl[j] = ok ? *reinterpret_cast<const bf16x8*>(wl + kk) : zero;
-      fh[j] = ok ? *reinterpret_cast<const bf16x8*>(wh + kk) : zero;
-      fx[j] = ok ? *reinterpret_cast<const bf16x8*>(xr + kk) : zero;
+      int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row
+      kk = kk < kend ? kk : kbegin + 8 * g;  // (past the end: a piece that was read before, not the next wavefront's)
+      st.fl[j] = *reinterpret_cast<const bf16x8*>(wl + kk);
+      st.fh[j] = *reinterpret_cast<const bf16x8*>(wh + kk);
+      st.fx[j] = *reinterpret_cast<const bf16x8*>(xr + kk);
     }
+  };
+  auto multiply = [&](int k0, const Step& st) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fl[j], fx[j], acc[0], 0, 0, 0);
-      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fh[j], fx[j], acc[1], 0, 0, 0);
+      const bf16x8 xv = (k0 + 32 * j + 8 * g < kend) ? st.fx[j] : zero;
+      acc[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.fl[j], xv, acc[0], 0, 0, 0);
+      acc[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(st.fh[j], xv, acc[1], 0, 0, 0);
+    }
+  };
+  // What the first wavefront needs after the products is asked for now, so that it is there by then.
+  const int t = m, j0 = 16 * jt + 4 * g, col = head * head_dim + j0;
+  const bool is_v = head >= heads + kv_heads;
+  float4 blo = make_float4(0.f, 0.f, 0.f, 0.f), bhi = blo, cs01 = blo, cs23 = blo;
+  uint2 blo16 = make_uint2(0u, 0u), bhi16 = blo16;
+  int slot_t = -1;
+  if (wave == 0 && t < tokens) {
+    if (bias) {
+      if (bias_dtype == IX_BF16) {
+        blo16 = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(bias) + col);
+        bhi16 = *reinterpret_cast<const uint2*>(static_cast<const uint16_t*>(bias) + col + half);
+      } else {
+        blo = *reinterpret_cast<const float4*>(static_cast<const float*>(bias) + col);
+        bhi = *reinterpret_cast<const float4*>(static_cast<const float*>(bias) + col + half);
+      }
+    }
+    if (!is_v && cs) {
+      const float4* c = reinterpret_cast<const float4*>(cs + static_cast<int64_t>(t) * half + j0);
+      cs01 = c[0];
+      cs23 = c[1];
+    }
+    if (slots) slot_t = slots[t];
+  }
+  if (kbegin < kend) {
+    fetch(kbegin, one);
+    for (int k0 = kbegin; k0 < kend; k0 += 256) {
+      fetch(k0 + 128, two);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(k0, one);
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(k0 + 256, one);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(k0 + 128, two);
+      __builtin_amdgcn_sched_barrier(0);
     }
   }
   if (wave > 0) {
@@ -70,10 +114,16 @@ qkv_rope_skinny_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ 
   }
 
   // lane holds features j = 16 jt + 4 g + i (low) and j + half (high) of token m
-  const int t = m;
   if (t >= tokens) return;
-  const int j0 = 16 * jt + 4 * g;
-  const int col = head * head_dim + j0;
+  if (bias && bias_dtype == IX_BF16) {
+    blo = make_float4(__uint_as_float(blo16.x << 16), __uint_as_float(blo16.x & 0xffff0000u),
+                      __uint_as_float(blo16.y << 16), __uint_as_float(blo16.y & 0xffff0000u));
+    bhi = make_float4(__uint_as_float(bhi16.x << 16), __uint_as_float(bhi16.x & 0xffff0000u),
+                      __uint_as_float(bhi16.y << 16), __uint_as_float(bhi16.y & 0xffff0000u));
+  }
+  const float bl[4] = {blo.x, blo.y, blo.z, blo.w}, bh[4] = {bhi.x, bhi.y, bhi.z, bhi.w};
+  const float2 rot[4] = {make_float2(cs01.x, cs01.y), make_float2(cs01.z, cs01.w), make_float2(cs23.x, cs23.y),
+                         make_float2(cs23.z, cs23.w)};
   float lo[4], hi[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
@@ -81,25 +131,23 @@ qkv_rope_skinny_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ 
     lo[i] = ix_bf16_to_f32(ix_f32_to_bf16(acc[0][i]));
     hi[i] = ix_bf16_to_f32(ix_f32_to_bf16(acc[1][i]));
     if (bias) {
-      lo[i] += ix_load_rt(bias, bias_dtype, col + i);
-      hi[i] += ix_load_rt(bias, bias_dtype, col + half + i);
+      lo[i] += bl[i];
+      hi[i] += bh[i];
     }
   }
-  const bool is_v = head >= heads + kv_heads;
   if (!is_v && cs) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const float2 c = cs[static_cast<int64_t>(t) * half + j0 + i];
+      const float2 c = rot[i];
       const float rlo = lo[i] * c.x - hi[i] * c.y;
       const float rhi = hi[i] * c.x + lo[i] * c.y;
       lo[i] = rlo;
       hi[i] = rhi;
     }
   }
-  const int64_t slot = slots ? slots[t] : -1;
-  const bool cache_ok = k_cache != nullptr && slot >= 0 && slot < total_slots;
-  const int64_t page = cache_ok ? slot / page_size : 0;
-  const int off = cache_ok ? static_cast<int>(slot % page_size) : 0;
+  const bool cache_ok = k_cache != nullptr && slot_t >= 0 && slot_t < total_slots;
+  const int64_t page = cache_ok ? slot_t / page_size : 0;  // (slots are 32-bit: a short division)
+  const int off = cache_ok ? slot_t - static_cast<int>(page) * page_size : 0;
   if (is_v) {
     if (!cache_ok) return;
     __bf16* dst = v_cache + ((page * kv_heads + (head - heads - kv_heads)) * head_dim + j0) * page_size + off;
@@ -131,6 +179,9 @@ extern "C" int ix_qkv_rope_skinny(const void* x, const void* w, const void* bias
   IX_REQUIRE(head_dim % 32 == 0 && head_dim <= 256, "head_dim must be a multiple of 32 up to 256");
   IX_REQUIRE(width % 8 == 0 && width < (1 << 30), "the reduction width must be a multiple of 8");
   IX_REQUIRE((k_cache == nullptr) == (v_cache == nullptr), "give both caches or neither");
+  IX_REQUIRE(bias == nullptr || bias_dtype == IX_F32 || bias_dtype == IX_BF16, "the bias must be float32 or bfloat16");
+  IX_REQUIRE(((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(bias) |
+               reinterpret_cast<uintptr_t>(cs)) & 15) == 0, "operands must be aligned to 16 bytes");
   dim3 grid((heads + 2 * kv_heads) * (head_dim / 32)), block(256);
   hipLaunchKernelGGL(qkv_rope_skinny_kernel, grid, block, 0, stream, (const __bf16*)x, (const __bf16*)w, bias,
                      bias_dtype, (const float2*)cs, slots, (__bf16*)q_out, (__bf16*)k_cache, (__bf16*)v_cache, tokens,
