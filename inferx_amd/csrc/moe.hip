@@ -257,70 +257,103 @@ extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dty
 // Also, for the matrix-core product, a map of row tiles: tile i covers rows
 // [tile_row0[i], min(tile_row0[i] + tile_rows, end of its expert)) of expert
 // tile_expert[i]; tile_info[0] = number of tiles.
-__global__ void __launch_bounds__(1024)
-moe_count_scan_kernel(const int32_t* __restrict__ topk_e, int32_t* __restrict__ offsets, int64_t assignments,
-                      int experts, int tile_rows, int32_t* __restrict__ tile_expert,
-                      int32_t* __restrict__ tile_row0, int32_t* __restrict__ tile_info) {
+// Many assignments: one workgroup of sixteen wavefronts per expert, one launch.  Every workgroup counts the
+// assignments of all experts (a sweep over topk_e with integer atomics in LDS: order does not matter), adds up
+// the rows and row tiles of the experts before its own, writes its own offset and tiles, and then places its
+// own assignments in a second sweep: a wavefront takes 512 consecutive assignments of a pass of 8,192, finds
+// its matches by ballot, and their rows follow from the counts of the wavefronts before it.
+#define DW_THREADS 1024
+#define DW_WAVES (DW_THREADS / 64)
+#define DW_ROUNDS 8
+__global__ void __launch_bounds__(DW_THREADS)
+moe_dispatch_wide_kernel(const int32_t* __restrict__ topk_e, int32_t* __restrict__ offsets,
+                         int32_t* __restrict__ rows, int32_t* __restrict__ dest, int64_t assignments, int experts,
+                         int k, int tile_rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
+                         int32_t* __restrict__ tile_info) {
   __shared__ int32_t counts[IX_MAX_EXPERTS];
-  __shared__ int32_t first_row[IX_MAX_EXPERTS];
-  __shared__ int32_t first_tile[IX_MAX_EXPERTS];
-  for (int e = threadIdx.x; e < experts; e += blockDim.x) counts[e] = 0;
-  __syncthreads();
-  for (int64_t a = threadIdx.x; a < assignments; a += blockDim.x) {
-    const int e = topk_e[a];
-    if (e >= 0 && e < experts) atomicAdd(&counts[e], 1);  // integer counts: order does not matter
-  }
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    int32_t run = 0, tiles = 0;
-    for (int e = 0; e < experts; ++e) {
-      offsets[e] = run;
-      first_row[e] = run;
-      first_tile[e] = tiles;
-      run += counts[e];
-      if (tile_rows > 0) tiles += (counts[e] + tile_rows - 1) / tile_rows;
-    }
-    offsets[experts] = run;
-    if (tile_info) tile_info[0] = tiles;
-  }
-  __syncthreads();
-  if (tile_rows > 0 && tile_expert) {
-    for (int e = threadIdx.x; e < experts; e += blockDim.x) {
-      const int n = (counts[e] + tile_rows - 1) / tile_rows;
-      for (int i = 0; i < n; ++i) {
-        tile_expert[first_tile[e] + i] = e;
-        tile_row0[first_tile[e] + i] = first_row[e] + i * tile_rows;
-      }
-    }
-  }
-}
-
-__global__ void __launch_bounds__(256)
-moe_scatter_kernel(const int32_t* __restrict__ topk_e, const int32_t* __restrict__ offsets,
-                   int32_t* __restrict__ rows, int32_t* __restrict__ dest, int64_t assignments, int k) {
-  __shared__ int32_t wave_count[4];
+  __shared__ int32_t wave_count[DW_WAVES];
+  __shared__ int32_t part[2][DW_WAVES];
   const int e = blockIdx.x;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  int32_t next = offsets[e];
-  for (int64_t base = 0; base < assignments; base += 256) {
-    const int64_t a = base + threadIdx.x;
-    const bool mine = a < assignments && topk_e[a] == e;
-    const unsigned long long ballot = __ballot(mine);
-    const int before = __popcll(ballot & ((1ull << lane) - 1ull));
-    __syncthreads();
-    if (lane == 0) wave_count[wave] = __popcll(ballot);
-    __syncthreads();
-    int wave_base = 0, total = 0;
-    for (int w = 0; w < 4; ++w) {
-      if (w < wave) wave_base += wave_count[w];
-      total += wave_count[w];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  for (int i = tid; i < experts; i += DW_THREADS) counts[i] = 0;
+  __syncthreads();
+  for (int64_t a = tid; a < assignments; a += DW_THREADS) {
+    const int v = topk_e[a];
+    if (v >= 0 && v < experts) atomicAdd(&counts[v], 1);
+  }
+  __syncthreads();
+  int rows_before = 0, tiles_before = 0;
+  for (int i = tid; i < e; i += DW_THREADS) {
+    const int c = counts[i];
+    rows_before += c;
+    tiles_before += tile_rows > 0 ? (c + tile_rows - 1) / tile_rows : 0;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    rows_before += __shfl_xor(rows_before, off, 64);
+    tiles_before += __shfl_xor(tiles_before, off, 64);
+  }
+  if (lane == 0) {
+    part[0][wave] = rows_before;
+    part[1][wave] = tiles_before;
+  }
+  __syncthreads();
+  rows_before = tiles_before = 0;
+#pragma unroll
+  for (int w = 0; w < DW_WAVES; ++w) {
+    rows_before += part[0][w];
+    tiles_before += part[1][w];
+  }
+  const int mine = counts[e];
+  const int my_tiles = tile_rows > 0 ? (mine + tile_rows - 1) / tile_rows : 0;
+  if (tid == 0) {
+    offsets[e] = rows_before;
+    if (e == experts - 1) {
+      offsets[experts] = rows_before + mine;
+      if (tile_info) tile_info[0] = tiles_before + my_tiles;
     }
-    if (mine) {
-      const int32_t r = next + wave_base + before;
-      rows[r] = static_cast<int32_t>(a / k);
-      dest[a] = r;
+  }
+  if (tile_expert)
+    for (int i = tid; i < my_tiles; i += DW_THREADS) {
+      tile_expert[tiles_before + i] = e;
+      tile_row0[tiles_before + i] = rows_before + i * tile_rows;
     }
-    next += total;
+  if (mine == 0) return;  // uniform over the workgroup
+
+  const uint64_t below = (uint64_t(1) << lane) - 1;
+  int base = rows_before;
+  for (int64_t p0 = 0; p0 < assignments; p0 += DW_WAVES * DW_ROUNDS * 64) {
+    const int64_t a0 = p0 + static_cast<int64_t>(wave) * DW_ROUNDS * 64 + lane;
+    uint64_t match[DW_ROUNDS];
+    int found = 0;
+#pragma unroll
+    for (int r = 0; r < DW_ROUNDS; ++r) {
+      const int64_t a = a0 + 64 * r;
+      match[r] = __ballot(a < assignments && topk_e[a] == e);
+      found += __popcll(match[r]);
+    }
+    if (lane == 0) wave_count[wave] = found;
+    __syncthreads();
+    int before = 0, total = 0;
+#pragma unroll
+    for (int w = 0; w < DW_WAVES; ++w) {
+      const int c = wave_count[w];
+      before += w < wave ? c : 0;
+      total += c;
+    }
+    int run = base + before;
+#pragma unroll
+    for (int r = 0; r < DW_ROUNDS; ++r) {
+      if ((match[r] >> lane) & 1) {
+        const int64_t a = a0 + 64 * r;
+        const int32_t row = run + __popcll(match[r] & below);
+        rows[row] = static_cast<int32_t>(a / k);
+        dest[a] = row;
+      }
+      run += __popcll(match[r]);
+    }
+    base += total;
+    __syncthreads();
   }
 }
 
@@ -389,11 +422,8 @@ extern "C" int ix_moe_dispatch(const int32_t* topk_e, int32_t* offsets, int32_t*
                        (int)assignments, experts, k, tile_rows, tile_expert, tile_row0, tile_info);
     return ix_check_launch("ix_moe_dispatch");
   }
-  hipLaunchKernelGGL(moe_count_scan_kernel, dim3(1), dim3(1024), 0, stream, topk_e, offsets, assignments, experts,
-                     tile_rows, tile_expert, tile_row0, tile_info);
-  if (assignments > 0)
-    hipLaunchKernelGGL(moe_scatter_kernel, dim3(experts), dim3(256), 0, stream, topk_e, offsets, rows, dest,
-                       assignments, k);
+  hipLaunchKernelGGL(moe_dispatch_wide_kernel, dim3(experts), dim3(DW_THREADS), 0, stream, topk_e, offsets, rows, dest,
+                     assignments, experts, k, tile_rows, tile_expert, tile_row0, tile_info);
   return ix_check_launch("ix_moe_dispatch");
 }
 

@@ -85,7 +85,8 @@ def dispatch(topk_e, E, tile_rows=0):
 
 
 @pytest.mark.parametrize("T,E,k,tile_rows", [(24, 8, 2, 16), (300, 60, 4, 32), (1, 4, 2, 16), (1000, 7, 3, 64),
-                                             (40, 64, 1, 0)])
+                                             (40, 64, 1, 0), (2048, 60, 4, 160), (3000, 60, 4, 160), (500, 200, 3, 32),
+                                             (600, 1024, 2, 16), (4100, 3, 2, 0)])
 def test_dispatch_is_a_stable_bijection(T, E, k, tile_rows):
     # reference: moe_test.cc:277-350
     g = torch.Generator().manual_seed(T)
