@@ -28,7 +28,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // The work of one wavefront (KSPLIT == 1) or workgroup (KSPLIT == 4): rows [row0, row_end) x out-features
 // [n0, n0 + 16) of expert e.  `red`: LDS for the partial sums of a split reduction.
 template <int MT, bool GATE_UP, int KSPLIT, typename TO = __bf16>
-__device__ __forceinline__ void grouped_body(const __bf16* __restrict__ a, const __bf16* __restrict__ w,
+__device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
                                              TO* __restrict__ out, const int32_t* __restrict__ rows, int e,
                                              int row0, int row_end, int n0, int n_out, int width, float* red) {
   constexpr int NACC = GATE_UP ? 2 : 1;
@@ -58,36 +58,60 @@ __device__ __forceinline__ void grouped_body(const __bf16* __restrict__ a, const
 
   const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
                        (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
-  // the loads of the next 128 of K are issued before the products of the present ones, so that a wavefront
-  // always has loads on their way
+  // The loads of the next 128 of K are issued before the products of the present ones, so that a wavefront
+  // always has loads on their way.  Every load is unconditional (a piece past the end of a ragged last round is read from the
+  // range's first piece instead, which is in the cache, and the activations' values are replaced by zeros when they are
+  // used): with no branch in it the loop is one straight line, and the compiler lets the younger loads stay in
+  // flight at each wait instead of waiting for all.
   bf16x8 fw[2][NACC][4], fx[2][MT][4];
   auto fetch = [&](int k0, bf16x8 (&w_)[NACC][4], bf16x8 (&x_)[MT][4]) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row per load
-      const bool ok = kk < kend;
-      w_[0][j] = ok ? *reinterpret_cast<const bf16x8*>(wg + kk) : zero;
-      if (GATE_UP) w_[1][j] = ok ? *reinterpret_cast<const bf16x8*>(wu + kk) : zero;
+      int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row per load
+      kk = kk < kend ? kk : kbegin + 8 * g;
+      w_[0][j] = *reinterpret_cast<const bf16x8*>(wg + kk);
+      if (GATE_UP) w_[1][j] = *reinterpret_cast<const bf16x8*>(wu + kk);
 #pragma unroll
-      for (int t = 0; t < MT; ++t) x_[t][j] = ok ? *reinterpret_cast<const bf16x8*>(xr[t] + kk) : zero;
+      for (int t = 0; t < MT; ++t) x_[t][j] = *reinterpret_cast<const bf16x8*>(xr[t] + kk);
     }
   };
-  auto multiply = [&](const bf16x8 (&w_)[NACC][4], const bf16x8 (&x_)[MT][4]) {
+  auto multiply = [&](int k0, const bf16x8 (&w_)[NACC][4], const bf16x8 (&x_)[MT][4]) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 4; ++j) {
+      const bool ok = k0 + 32 * j + 8 * g < kend;
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
+      for (int t = 0; t < MT; ++t) {
+        const bf16x8 xv = ok ? x_[t][j] : zero;
 #pragma unroll
         for (int u = 0; u < NACC; ++u)
-          acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_[u][j], x_[t][j], acc[u][t], 0, 0, 0);
+          acc[u][t] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(w_[u][j], xv, acc[u][t], 0, 0, 0);
+      }
+    }
   };
-  if (kbegin < kend) fetch(kbegin, fw[0], fx[0]);
-  for (int k0 = kbegin; k0 < kend; k0 += 256) {  // two rounds per turn, so that the register sets are named statically
-    if (k0 + 128 < kend) fetch(k0 + 128, fw[1], fx[1]);
-    multiply(fw[0], fx[0]);
-    if (k0 + 128 >= kend) break;
-    if (k0 + 256 < kend) fetch(k0 + 256, fw[0], fx[0]);
-    multiply(fw[1], fx[1]);
+  // Rounds of 128 in pairs, so that the register sets are named statically; the loop runs while both rounds of a
+  // turn are followed by another one and has no way out of its middle, the last one or two rounds come after it.
+  const int rounds = kbegin < kend ? (kend - kbegin + 127) >> 7 : 0;
+  if (rounds > 0) {
+    fetch(kbegin, fw[0], fx[0]);
+    int k0 = kbegin, left = rounds;
+    for (; left > 2; left -= 2, k0 += 256) {
+      fetch(k0 + 128, fw[1], fx[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(k0, fw[0], fx[0]);
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(k0 + 256, fw[0], fx[0]);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(k0 + 128, fw[1], fx[1]);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    if (left == 2) {
+      fetch(k0 + 128, fw[1], fx[1]);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(k0, fw[0], fx[0]);
+      multiply(k0 + 128, fw[1], fx[1]);
+    } else {
+      multiply(k0, fw[0], fx[0]);
+    }
   }
 
   if (KSPLIT > 1) {
@@ -147,7 +171,7 @@ __device__ __forceinline__ void grouped_body(const __bf16* __restrict__ a, const
 // logits stay float32 (one workgroup per 16 out-features, the reduction split over its four wavefronts).
 template <int MT>
 __global__ void __launch_bounds__(256)
-linear_skinny_f32_kernel(const __bf16* __restrict__ x, const __bf16* __restrict__ w, float* __restrict__ out,
+linear_skinny_f32_kernel(const __bf16* x, const __bf16* w, float* __restrict__ out,
                          int rows, int n_out, int width) {
   __shared__ float red[3 * 64 * MT * 4];
   grouped_body<MT, false, 4, float>(x, w, out, nullptr, 0, 0, rows, blockIdx.x * 16, n_out, width, red);
@@ -155,7 +179,7 @@ linear_skinny_f32_kernel(const __bf16* __restrict__ x, const __bf16* __restrict_
 
 template <int MT, bool GATE_UP, int KSPLIT>
 __global__ void __launch_bounds__(256)
-moe_grouped_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w, __bf16* __restrict__ out,
+moe_grouped_mfma_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ out,
                         const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
                         const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
                         const int32_t* __restrict__ tile_info, int n_out, int width) {
@@ -173,11 +197,11 @@ moe_grouped_mfma_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__
 // workgroups to start set the kernel's end); the rest serve the routed experts' row tiles.
 template <int MT, bool GATE_UP>
 __global__ void __launch_bounds__(256)
-moe_grouped_dual_kernel(const __bf16* __restrict__ a, const __bf16* __restrict__ w, __bf16* __restrict__ out,
+moe_grouped_dual_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ out,
                         const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
                         const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
                         const int32_t* __restrict__ tile_info, int max_tiles, int n_out, int width,
-                        const __bf16* __restrict__ a_s, const __bf16* __restrict__ w_s, __bf16* __restrict__ out_s,
+                        const __bf16* a_s, const __bf16* w_s, __bf16* __restrict__ out_s,
                         int shared_rows, int n_out_s, int width_s) {
   __shared__ float red[3 * 64 * MT * (GATE_UP ? 2 : 1) * 4];
   const int n16_s = (n_out_s + 15) / 16;

@@ -36,9 +36,9 @@ qkv_rope_skinny_kernel(const __bf16* x, const __bf16* w, const void* __restrict_
                        (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
   f32x4 acc[2] = {f32x4{0.f, 0.f, 0.f, 0.f}, f32x4{0.f, 0.f, 0.f, 0.f}};
   // Steps of 128 of the reduction in two register sets: the loads of the next step are on their way while this
-  // one is multiplied.  Every load is unconditional (a piece past the end is read from the range's first piece
-  // instead, and its token values are replaced by zeros when they are used), so that the loop is one straight
-  // line and the compiler lets the younger loads stay in flight at each wait.
+  // one is multiplied.  Every load is unconditional (a piece past the end of a ragged last round is read from
+  // the range's first piece instead, and its token values are replaced by zeros when they are used), so that
+  // the loop is one straight line and the compiler lets the younger loads stay in flight at each wait.
   struct Step { bf16x8 fl[4], fh[4], fx[4]; };
   Step one, two;
   auto fetch = [&](int k0, Step& st) {
@@ -82,9 +82,13 @@ qkv_rope_skinny_kernel(const __bf16* x, const __bf16* w, const void* __restrict_
     }
     if (slots) slot_t = slots[t];
   }
-  if (kbegin < kend) {
+  // rounds in pairs; the loop runs while both rounds of a turn are followed by another one and has no way out of
+  // its middle, the last one or two rounds come after it
+  const int rounds = kbegin < kend ? (kend - kbegin + 127) >> 7 : 0;
+  if (rounds > 0) {
     fetch(kbegin, one);
-    for (int k0 = kbegin; k0 < kend; k0 += 256) {
+    int k0 = kbegin, left = rounds;
+    for (; left > 2; left -= 2, k0 += 256) {
       fetch(k0 + 128, two);
       __builtin_amdgcn_sched_barrier(0);
       multiply(k0, one);
@@ -93,6 +97,14 @@ qkv_rope_skinny_kernel(const __bf16* x, const __bf16* w, const void* __restrict_
       __builtin_amdgcn_sched_barrier(0);
       multiply(k0 + 128, two);
       __builtin_amdgcn_sched_barrier(0);
+    }
+    if (left == 2) {
+      fetch(k0 + 128, two);
+      __builtin_amdgcn_sched_barrier(0);
+      multiply(k0, one);
+      multiply(k0 + 128, two);
+    } else {
+      multiply(k0, one);
     }
   }
   if (wave > 0) {
