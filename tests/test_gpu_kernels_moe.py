@@ -158,7 +158,8 @@ def grouped_reference(a, w, offsets, rows, gate_up):
     return out
 
 
-GROUPED = [(24, 64, 8, 2, 32), (300, 96, 8, 3, 48), (9, 72, 5, 1, 40), (700, 256, 60, 4, 176), (3, 2048, 60, 4, 1408)]
+GROUPED = [(24, 64, 8, 2, 32), (300, 96, 8, 3, 48), (9, 72, 5, 1, 40), (700, 256, 60, 4, 176), (3, 2048, 60, 4, 1408),
+           (20, 1160, 5, 2, 200)]
 
 
 @pytest.mark.parametrize("T,H,E,k,mi", GROUPED)
