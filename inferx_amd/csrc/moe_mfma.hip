@@ -59,10 +59,10 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
   const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
                        (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
   // The loads of the next 128 of K are issued before the products of the present ones, so that a wavefront
-  // always has loads on their way.  Every load is unconditional (a piece past the end of a ragged last round is read from the
-  // range's first piece instead, which is in the cache, and the activations' values are replaced by zeros when they are
-  // used): with no branch in it the loop is one straight line, and the compiler lets the younger loads stay in
-  // flight at each wait instead of waiting for all.
+  // always has loads on their way.  Every load is unconditional (a piece past the end of a ragged last round is
+  // read from the range's first piece instead, which is in the cache, and the activations' values are replaced
+  // by zeros when they are used): with no branch in it the loop is one straight line, and the compiler lets the
+  // younger loads stay in flight at each wait instead of waiting for all.
   bf16x8 fw[2][NACC][4], fx[2][MT][4];
   auto fetch = [&](int k0, bf16x8 (&w_)[NACC][4], bf16x8 (&x_)[MT][4]) {
 #pragma unroll

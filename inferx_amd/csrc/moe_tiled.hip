@@ -37,15 +37,17 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 // piece index then fall on sixteen different groups of four banks, as do the pieces that sixteen lanes write
 __device__ __forceinline__ int tl_at(int row, int piece) { return row * TL_STRIDE + ((piece ^ ((row >> 1) & 7)) << 3); }
 
-// One row tile x 128 weight rows.  NP: pairs of sixteens of activation rows the tile holds (1..5); with it a
+// One row tile x 128 weight rows.  NP: pairs of sixteens of activation rows the tile holds (1..5).  With it a
 // template parameter, and every load unconditional (a stage past the end asks for the last stage again, a piece
-// past the row's end for the row's start, and what comes back is replaced by zero on its way into LDS), the loop is one straight line, so the
-// compiler can count exactly how many loads may stay in flight at each wait.  With branches in the loop it
-// waited for all of them, also those of three stages ahead.
+// past the row's end for the row's start, and zeros are written over it in LDS), the loop is one straight line,
+// so the compiler can count exactly how many loads may stay in flight at each wait.  With branches in the loop
+// it waited for all of them, also those of three stages ahead.
 template <bool GATE_UP, int NP>
 __device__ __forceinline__ void
-tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ rows, int n_out, int width, int e, int row0, int row_end, int tile, int col_block, __bf16* ws,
-           __bf16* xs) {
+tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ rows, int n_out, int width,
+           int e, int row0, int row_end, int tile, int col_block, __bf16* ws, __bf16* xs) {
+  // (a and w are plain pointers on purpose: loads through `const __restrict__` ones may be moved by the
+  // optimiser, which sinks them to their first use and so undoes the prefetch)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
   const int wi = wave & 1, xi = wave >> 1;
@@ -78,8 +80,8 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
   const int xdst = tl_at(tid >> 3, tid & 7);  // rows 32 further on have the same permutation
 
   // The weights come from memory and are what the kernel waits for: three register sets keep the loads of three
-  // stages on their way while a fourth stage is multiplied out of LDS.  The activations are asked for two stages
-  // ahead, in two sets.
+  // stages on their way while one stage is multiplied and the next one lies in the other LDS buffer.  The
+  // activations, which mostly come from L2, are in two sets.
   bf16x8 wreg[3][4], xreg[2][NP];
   // Row tiles walk the reduction in the same order but start at different stages (and wrap round): were all
   // workgroups at the same offset of their weight rows at the same time, a row length that is a power of two
@@ -92,8 +94,8 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
                       : 0;         // (they read the same activations, which then stay in L2)
   // Where this thread's pieces of stage k0 start in a row, and whether they exist.  A piece that does not exist
   // (the reduction width is no multiple of 64) is loaded from the row's start instead and overwritten with
-  // zeros in LDS by the thread that put it there: no loaded value is touched before its use, and the only
-  // branch, in the last stage, holds nothing but LDS writes.
+  // zeros in LDS by the thread that put it there: no loaded value is touched before its use, and the branch
+  // that does it holds nothing but LDS writes.
   const bool ragged = (width & (TL_K - 1)) != 0;
   auto place = [&](int k0, bool& ok) {
     k0 = min(k0, kspan - TL_K);
@@ -259,7 +261,8 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
 
 template <bool GATE_UP>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
-moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
+moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ offsets,
+                         const int32_t* __restrict__ rows,
                          const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
                          const int32_t* __restrict__ tile_info, int n_out, int width, int n_col_blocks) {
   __shared__ __attribute__((aligned(16))) __bf16 ws[2 * TL_WTILE];
