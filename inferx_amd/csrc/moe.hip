@@ -5,6 +5,7 @@
 // Placement is deterministic: no floating-point atomics anywhere, rows of one
 // expert keep token order (reference: ops/moe.h:26-33, moe.cu:130-221).
 #include "common.h"
+#include "moe_route.h"
 
 #define ROUTE_THREADS 256
 #define IX_MAX_TOP_K 32
@@ -18,35 +19,6 @@
 // (reference: RouteTopKKernel, moe.cu:36-127).  Output order: descending score.
 // If `shared_gate_w` is given, sigmoid(x . shared_gate_w) is written too
 // (reference: AddSharedExpertKernel, moe.cu:275-287).
-// x . w[row] over `width`, one wavefront, x as float32 at `xs` (LDS or global)
-__device__ __forceinline__ float route_row_dot(const float* __restrict__ xs, const void* __restrict__ w, int dt,
-                                               int64_t base, int64_t width, int lane) {
-  float dot = 0.f;
-  if (dt == IX_BF16 && (width & 7) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
-    // eight weights per lane and load (16 bytes); the order of additions is fixed by the lane layout
-    const uint16_t* wrow = static_cast<const uint16_t*>(w) + base;
-    for (int64_t i = lane * 8; i < width; i += 512) {
-      const uint4 v = *reinterpret_cast<const uint4*>(wrow + i);
-      const float4 x0 = *reinterpret_cast<const float4*>(xs + i);
-      const float4 x1 = *reinterpret_cast<const float4*>(xs + i + 4);
-      dot += x0.x * __uint_as_float(v.x << 16) + x0.y * __uint_as_float(v.x & 0xffff0000u) +
-             x0.z * __uint_as_float(v.y << 16) + x0.w * __uint_as_float(v.y & 0xffff0000u) +
-             x1.x * __uint_as_float(v.z << 16) + x1.y * __uint_as_float(v.z & 0xffff0000u) +
-             x1.z * __uint_as_float(v.w << 16) + x1.w * __uint_as_float(v.w & 0xffff0000u);
-    }
-  } else if (dt == IX_F32 && (width & 3) == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0) {
-    const float* wrow = static_cast<const float*>(w) + base;
-    for (int64_t i = lane * 4; i < width; i += 256) {
-      const float4 v = *reinterpret_cast<const float4*>(wrow + i);
-      const float4 x0 = *reinterpret_cast<const float4*>(xs + i);
-      dot += x0.x * v.x + x0.y * v.y + x0.z * v.z + x0.w * v.w;
-    }
-  } else {
-    for (int64_t i = lane; i < width; i += 64) dot += xs[i] * ix_load_rt(w, dt, base + i);
-  }
-  return ix_wave_sum(dot);
-}
-
 // softmax over z[0..experts) (LDS, overwritten) and k rounds of argmax, by the whole workgroup
 __device__ __forceinline__ void route_select(float* z, float* red, float* __restrict__ topk_w,
                                              int32_t* __restrict__ topk_e, int64_t t, int experts, int k,

@@ -299,14 +299,26 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
 
 
 SELECT_DISPATCH_MAX_ASSIGNMENTS, SELECT_DISPATCH_MAX_EXPERTS = 1024, 256
+ROUTE_ONE_LAUNCH_TOKENS = 16
+_arrival_counters: dict = {}
+
+
+def _arrival_counter(device: torch.device) -> torch.Tensor:
+    """One int32 per device that the one-launch router's workgroups count themselves off on; every launch
+    leaves it zero.  Launches on one device follow one another on a stream, so they can share it."""
+    c = _arrival_counters.get(device)
+    if c is None:
+        c = _arrival_counters[device] = torch.zeros(1, dtype=torch.int32, device=device)
+    return c
 
 
 def moe_route_dispatch(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor],
                        topk_w: torch.Tensor, topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor],
                        renormalize: bool, scale: float, offsets: torch.Tensor, rows: torch.Tensor,
                        dest: torch.Tensor, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None) -> None:
-    """`moe_route` and `moe_dispatch` for few tokens in two launches: router scores spread over many workgroups,
-    then selection and grouping in one workgroup.  Needs T * k <= 1024 and at most 256 experts."""
+    """`moe_route` and `moe_dispatch` for few tokens: router scores spread over many workgroups, then selection
+    and grouping in one workgroup; up to 16 tokens in one launch (the last workgroup to finish its scores goes
+    on), else in two.  Needs T * k <= 1024 and at most 256 experts."""
     T, H = x.shape
     E = router_w.shape[0]
     k = topk_w.shape[1]
@@ -330,6 +342,14 @@ def moe_route_dispatch(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: O
         _is_i32(tile_map, 2 * mt + 1)
         te, tr, ti = tile_map[:mt], tile_map[mt:2 * mt], tile_map[2 * mt:]
     logits = torch.empty((T, E + 1), dtype=torch.float32, device=x.device)
+    if T <= ROUTE_ONE_LAUNCH_TOKENS and H * 4 <= 40 * 1024:
+        _call("ix_moe_route_dispatch_small", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)),
+              _ptr(shared_gate_w), _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits),
+              _ptr(_arrival_counter(x.device)), _i64(H), _ptr(topk_w), _ptr(topk_e),
+              _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest),
+              _i32(T), _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(tile_rows), _ptr(te),
+              _ptr(tr), _ptr(ti), _stream())
+        return
     _call("ix_moe_route_logits", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
           _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits), _i64(T), _i64(H), _i32(E),
           _stream())

@@ -121,10 +121,12 @@ def test_dispatch_is_a_stable_bijection(T, E, k, tile_rows):
 
 @pytest.mark.parametrize("T,H,E,k,renorm,tile_rows", [(1, 64, 4, 2, False, 16), (8, 2048, 60, 4, False, 16),
                                                        (37, 96, 8, 3, True, 32), (128, 72, 5, 1, False, 0),
-                                                       (32, 200, 256, 32, True, 16)])
+                                                       (32, 200, 256, 32, True, 16), (16, 136, 60, 4, True, 16),
+                                                       (5, 88, 7, 3, False, 0), (13, 200, 256, 8, True, 16)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_route_and_dispatch_in_two_launches(T, H, E, k, renorm, tile_rows, dtype):
-    """The fused selection + grouping gives exactly what the separate kernels give."""
+def test_route_and_dispatch_for_few_tokens(T, H, E, k, renorm, tile_rows, dtype):
+    """The fused selection + grouping (one launch up to 16 tokens, two beyond) gives exactly what the separate
+    kernels give."""
     from inferx_amd import ops
     x, wr, wsg = rnd(T, H, dtype=dtype), rnd(E, H, seed=1, dtype=dtype, scale=0.3), rnd(1, H, seed=2, dtype=dtype, scale=0.1)
     A = T * k
@@ -142,6 +144,28 @@ def test_route_and_dispatch_in_two_launches(T, H, E, k, renorm, tile_rows, dtype
         mt = (tm1.numel() - 1) // 2
         n = int(tm1[2 * mt])
         assert int(tm2[2 * mt]) == n and torch.equal(tm1[:n], tm2[:n]) and torch.equal(tm1[mt:mt + n], tm2[mt:mt + n])
+
+
+def test_route_in_one_launch_again_and_again():
+    """The one-launch router counts its workgroups off on a counter that every launch leaves at zero, and its
+    last workgroup reads what workgroups on other dies wrote: many launches of changing sizes one after the
+    other, without waiting, all agree with the separate kernels."""
+    from inferx_amd import ops
+    mk = lambda *shape, dt=torch.int32: torch.full(shape, -9, dtype=dt, device=DEV)
+    cases, got = [(3, 2048, 60, 4), (16, 136, 60, 4), (1, 64, 4, 2), (9, 200, 256, 8), (8, 2048, 60, 4)] * 40, []
+    for i, (T, H, E, k) in enumerate(cases):
+        x, wr, wsg = (rnd(T, H, seed=i, dtype=torch.bfloat16), rnd(E, H, seed=100 + i, dtype=torch.bfloat16, scale=0.3),
+                      rnd(1, H, seed=200 + i, dtype=torch.bfloat16, scale=0.1))
+        w2, e2, g2 = mk(T, k, dt=torch.float32), mk(T, k), mk(T, dt=torch.float32)
+        o2, r2, d2 = mk(E + 1), mk(T * k), mk(T * k)
+        ops.moe_route_dispatch(x, wr, wsg, w2, e2, g2, True, 1.0, o2, r2, d2, 0, None)
+        got.append((x, wr, wsg, w2, e2, g2, o2, r2, d2))
+    for (T, H, E, k), (x, wr, wsg, w2, e2, g2, o2, r2, d2) in zip(cases, got):
+        w1, e1, g1 = mk(T, k, dt=torch.float32), mk(T, k), mk(T, dt=torch.float32)
+        ops.moe_route(x, wr, wsg, w1, e1, g1, True, 1.0)
+        o1, r1, d1, _ = dispatch(e1, E, 0)
+        assert torch.equal(e1, e2) and torch.equal(o1, o2) and torch.equal(r1, r2) and torch.equal(d1, d2)
+        assert rel_err(w2, w1) < 1e-6 and rel_err(g2, g1) < 1e-6
 
 
 def grouped_reference(a, w, offsets, rows, gate_up):
