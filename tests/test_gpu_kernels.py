@@ -113,7 +113,7 @@ def tiles_for(q_lens, tile=16):
 
 
 @pytest.mark.parametrize("tile", [16, 32, -16])  # -16: tiles of 16 with prefetch
-@pytest.mark.parametrize("n_splits", [1, 3, 8])
+@pytest.mark.parametrize("n_splits", [1, 3, 8, 70])
 @pytest.mark.parametrize("case", ATTN_CASES)
 def test_attention_mfma(case, n_splits, tile):
     from inferx_amd import ops
