@@ -37,7 +37,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
   constexpr int NC = (NB + 1) / 2;          // 32-wide chunks of the head dimension
   constexpr int KS = 128;                   // elements per LDS row of the key tile: sixteen 16-byte pieces,
                                             // piece p of row r kept at place p ^ swz(r) (see key_place)
-  constexpr int VS = PF_KEYS + 8;           // elements per LDS row of the value tile
+  constexpr int VS = PF_KEYS;               // elements per LDS row of the value tile: eight 16-byte pieces,
+                                            // piece p of row r kept at place p ^ ((r >> 1) & 7)
   constexpr int K_CHUNKS = PF_KEYS * 2 * NB;  // 16-byte pieces of a key tile
   constexpr int V_CHUNKS = D * (PF_KEYS / 8);
   constexpr int K_PER = (K_CHUNKS + 255) / 256, V_PER = (V_CHUNKS + 255) / 256;
@@ -107,9 +108,12 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
 #pragma unroll
   for (int i = 0; i < V_PER; ++i) {
     const int c = min(tid + 256 * i, V_CHUNKS - 1), w = c % GROUP_CHUNKS;
+    // sixteen lanes take the same half (8 keys) of sixteen rows: with the permutation below they write to, and a
+    // quarter wavefront later reads from, sixteen different groups of four banks
+    const int half = (w >> 4) & 1, dd = (w & 15) | ((w >> 5) << 4);
     v_grp[i] = c / GROUP_CHUNKS;
-    v_src[i] = (w >> 1) * page_size + (w & 1) * 8;
-    v_dst[i] = (w >> 1) * VS + (c / GROUP_CHUNKS) * 16 + (w & 1) * 8;
+    v_src[i] = dd * page_size + half * 8;
+    v_dst[i] = dd * VS + (((2 * (c / GROUP_CHUNKS) + half) ^ ((dd >> 1) & 7)) << 3);
   }
   const int64_t page_elems = static_cast<int64_t>(kv_heads) * page_size * D;
   const __bf16* k_head = k_cache + static_cast<int64_t>(kvh) * page_size * D;
@@ -207,7 +211,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
         }
       }
 #pragma unroll
-      for (int b = 0; b < NB; ++b) vf[b] = *reinterpret_cast<const bf16x8*>(vs + (16 * b + n) * VS + 32 * h2 + 8 * g);
+      for (int b = 0; b < NB; ++b)  // row 16 b + n, piece 4 h2 + g; (row >> 1) & 7 = (n >> 1) & 7
+        vf[b] = *reinterpret_cast<const bf16x8*>(vs + (16 * b + n) * VS + (((4 * h2 + g) ^ ((n >> 1) & 7)) << 3));
 #pragma unroll
       for (int t = 0; t < QT; ++t) {
         if (wq0 + 16 * t >= rows || kb2 > pos0 + wq0 + 16 * t + 15) continue;
