@@ -68,7 +68,7 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row per load
-      kk = kk < kend ? kk : kbegin + 8 * g;
+      kk = kk < kend ? kk : kbegin;  // (the range's first piece: it exists, kbegin + 8 g need not)
       w_[0][j] = *reinterpret_cast<const bf16x8*>(wg + kk);
       if (GATE_UP) w_[1][j] = *reinterpret_cast<const bf16x8*>(wu + kk);
 #pragma unroll

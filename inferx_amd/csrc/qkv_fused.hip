@@ -45,7 +45,7 @@ qkv_rope_skinny_kernel(const __bf16* x, const __bf16* w, const void* __restrict_
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row
-      kk = kk < kend ? kk : kbegin + 8 * g;  // (past the end: a piece that was read before, not the next wavefront's)
+      kk = kk < kend ? kk : kbegin;  // (past the end: the range's first piece, which exists and was read before)
       st.fl[j] = *reinterpret_cast<const bf16x8*>(wl + kk);
       st.fh[j] = *reinterpret_cast<const bf16x8*>(wh + kk);
       st.fx[j] = *reinterpret_cast<const bf16x8*>(xr + kk);

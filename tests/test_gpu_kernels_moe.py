@@ -255,6 +255,34 @@ def test_grouped_tiled(T, H, E, k, mi):
         assert rel_err(act, act2) < 1e-2 and rel_err(y, y2) < 1e-2
 
 
+@pytest.mark.parametrize("T,N,K", [(3, 40, 264), (16, 33, 1160), (2, 16, 8), (5, 48, 520)])
+def test_streaming_kernels_read_nothing_past_their_operands(T, N, K):
+    """Reduction widths that leave a wavefront a ragged last round: what lies behind the last row of the weights
+    and of the activations (here NaN) must not reach a result, not even multiplied by zero."""
+    from inferx_amd import ops
+    xbuf = torch.full((T + 1, K), float("nan"), dtype=torch.bfloat16, device=DEV)
+    wbuf = torch.full((2 * N + 1, K), float("nan"), dtype=torch.bfloat16, device=DEV)
+    xbuf[:T] = rnd(T, K, dtype=torch.bfloat16)
+    wbuf[:2 * N] = rnd(2 * N, K, seed=1, dtype=torch.bfloat16, scale=K ** -0.5)
+    x, w = xbuf[:T], wbuf[:N]
+    out = torch.full((T, N), float("nan"), device=DEV)
+    ops.linear_skinny_f32(x, w, out)
+    want = x.double().cpu() @ w.double().cpu().t()
+    assert torch.isfinite(out).all() and rel_err(out, want) < 1e-5
+    # the grouped product, one expert: gate|up over both halves of the weights, then a plain product
+    offsets = torch.tensor([0, T], dtype=torch.int32, device=DEV)
+    tile_map = torch.tensor([0, 0, 0, 0, 1], dtype=torch.int32, device=DEV)  # one tile of expert 0 from row 0
+    for k_split in (1, 4):
+        act = torch.full((T, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.moe_grouped_mfma(x, wbuf[:2 * N].unsqueeze(0), act, offsets, None, tile_map, 16, True, k_split)
+        z = x.double().cpu() @ wbuf[:2 * N].double().cpu().t()
+        assert torch.isfinite(act).all()
+        assert rel_err(act, torch.nn.functional.silu(z[:, :N]) * z[:, N:]) < 1.5e-2
+        y = torch.full((T, N), float("nan"), dtype=torch.bfloat16, device=DEV)
+        ops.moe_grouped_mfma(x, w.unsqueeze(0), y, offsets, None, tile_map, 16, False, k_split)
+        assert torch.isfinite(y).all() and rel_err(y, want) < 1.5e-2
+
+
 @pytest.mark.parametrize("T,N,K", [(1, 301, 72), (8, 151936, 2048), (16, 384, 96), (33, 1000, 64), (64, 256, 40)])
 def test_linear_skinny_f32(T, N, K):
     from inferx_amd import ops
