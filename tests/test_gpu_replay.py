@@ -121,3 +121,24 @@ def test_mixed_with_few_pages(folders, name, dtype):
     ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"mixed {name} {dtype}",
                ties_for(folders, name, dtype))
     assert all(p.used_pages == 0 for p in runner.cache.pools)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("seed", [1, 2, 3, 5, 8, 13, 19, 34])
+def test_random_configurations(tmp_path, seed, dtype):
+    """Configurations drawn at random from what the architecture allows (head sizes up to 256 and some that are no
+    multiple of 16, odd widths, up to 130 experts, pages of 16 to 64, windows): portions of changing size and
+    mixed steps against the plain implementation."""
+    from inferx_amd.engine.runner import ModelRunner
+    cfg = tiny.random_config(seed)
+    page = cfg.pop("_page_size")
+    tiny.make_folder(cfg, seed=seed, out_dir=str(tmp_path), dtype=dtype)
+    raw, weights = tiny.read_folder(str(tmp_path))
+    prompts = {f"r{i}": tiny.random_tokens(n, cfg["vocab_size"], seed=7 * seed + i) for i, n in enumerate((5, 37, 70, 150))}
+    want = ru.expected_logits(raw, weights, prompts)
+    skip = ru.near_ties(raw, weights, prompts) if dtype == "bfloat16" else set()
+    for how, steps in (("whole", ru.whole(prompts)), ("portions", ru.chunked(prompts)),
+                       ("mixed", ru.mixed(prompts, seed=seed, max_live=4))):
+        runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=page, num_pages=4 * (160 // page + 2),
+                                            max_requests=4, max_seq_len=256)
+        ru.compare(ru.replay(runner, steps), want, (ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL), f"seed {seed} {dtype} {how}", skip=skip)

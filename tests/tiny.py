@@ -68,3 +68,37 @@ def read_folder(model_dir: str):
 def random_tokens(n: int, vocab: int, seed: int):
     g = torch.Generator().manual_seed(seed)
     return torch.randint(0, vocab, (n,), generator=g).tolist()
+
+
+def random_config(seed: int) -> dict:
+    """A tiny configuration drawn from the sizes the architecture allows: any number of heads and groups, head sizes
+    in steps of 16 up to 256 and a few that are no multiple of 16, widths and vocabularies that are no power of
+    two, up to 130 experts, pages of 16 to 64 (returned under the key "_page_size", which is no config key)."""
+    import random
+    rnd = random.Random(seed)
+    kv = rnd.choice([1, 2, 3, 4, 5])
+    heads = kv * rnd.choice([1, 2, 3, 4])
+    head_dim = 16 * rnd.randint(1, 16) if rnd.random() < 0.7 else rnd.choice([24, 40, 72])
+    experts = rnd.choice([2, 3, 5, 8, 16, 60, 130])
+    layers = rnd.randint(1, 4)
+    cfg = {
+        "architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "num_hidden_layers": layers,
+        "hidden_size": rnd.choice([64, 72, 88, 96, 100, 136, 200, 264]), "num_attention_heads": heads,
+        "num_key_value_heads": kv, "head_dim": head_dim, "num_experts": experts,
+        "num_experts_per_tok": rnd.randint(1, min(experts, 8)),
+        "moe_intermediate_size": rnd.choice([24, 32, 40, 56, 72, 136]),
+        "shared_expert_intermediate_size": rnd.choice([0, 28, 64, 88]),
+        "intermediate_size": rnd.choice([52, 96, 104, 160]), "decoder_sparse_step": rnd.choice([1, 1, 2]),
+        "mlp_only_layers": [rnd.randrange(layers)] if (layers > 1 and rnd.random() < 0.4) else [],
+        "norm_topk_prob": rnd.random() < 0.5, "vocab_size": rnd.choice([131, 256, 301, 1000]),
+        "rope_theta": rnd.choice([1e4, 1e6]), "rms_norm_eps": rnd.choice([1e-5, 1e-6]),
+        "max_position_embeddings": 512, "use_sliding_window": rnd.random() < 0.5,
+        "sliding_window": rnd.choice([8, 16, 24, 40]), "max_window_layers": rnd.randrange(layers + 1),
+        "tie_word_embeddings": rnd.random() < 0.3, "qkv_bias": rnd.random() < 0.7,
+        "_page_size": rnd.choice([16, 16, 32, 64]),
+    }
+    sparse = [l for l in range(layers)
+              if (l + 1) % cfg["decoder_sparse_step"] == 0 and l not in cfg["mlp_only_layers"]]
+    if not sparse:  # the architecture wants at least one layer of experts
+        cfg["decoder_sparse_step"], cfg["mlp_only_layers"] = 1, []
+    return cfg
