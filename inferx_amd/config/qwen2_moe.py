@@ -66,6 +66,9 @@ class Qwen2MoeConfig:
     initializer_range: float = 0.02
     torch_dtype: str = "bfloat16"
     hidden_act: str = "silu"
+    # ids that end a generation unless the request asks to generate through them (the reference takes the id
+    # from its tokenizer and adds it to a request's stop tokens, src/engine/engine.cc:819-823)
+    eos_token_ids: List[int] = field(default_factory=list)
 
     architecture = ARCHITECTURE
 
@@ -91,6 +94,10 @@ class Qwen2MoeConfig:
         mlp_only = raw.get("mlp_only_layers") or []
         if not isinstance(mlp_only, list) or any(isinstance(x, bool) or not isinstance(x, int) for x in mlp_only):
             raise ConfigError("config.json: mlp_only_layers must be a list of integers")
+        eos = raw.get("eos_token_id")
+        eos = [] if eos is None else (eos if isinstance(eos, list) else [eos])
+        if any(isinstance(x, bool) or not isinstance(x, int) for x in eos):
+            raise ConfigError("config.json: eos_token_id must be an integer or a list of integers")
         bias = raw.get("qkv_bias", raw.get("attention_bias"))
         if bias is None:
             bias = True
@@ -122,10 +129,14 @@ class Qwen2MoeConfig:
             initializer_range=_get(raw, "initializer_range", float, 0.02),
             torch_dtype=_get(raw, "torch_dtype", str, "bfloat16"),
             hidden_act=_get(raw, "hidden_act", str, "silu"),
+            eos_token_ids=list(eos),
         )
 
     def to_dict(self) -> Dict[str, Any]:
         d = asdict(self)
+        eos = d.pop("eos_token_ids")
+        if eos:
+            d["eos_token_id"] = eos[0] if len(eos) == 1 else eos
         d["architectures"] = [ARCHITECTURE]
         d["model_type"] = "qwen2_moe"
         return d
@@ -162,6 +173,8 @@ class Qwen2MoeConfig:
         need(all(0 <= l < self.num_hidden_layers for l in self.mlp_only_layers),
              "mlp_only_layers names a layer the model does not have")
         need(self.max_position_embeddings >= 0, "max_position_embeddings must not be negative")
+        need(all(0 <= t < self.vocab_size for t in self.eos_token_ids),
+             "eos_token_id names a token outside the vocabulary")
         if self.use_sliding_window:
             need(self.sliding_window > 0, "use_sliding_window is set but sliding_window is not positive")
             need(0 <= self.max_window_layers, "max_window_layers must not be negative")

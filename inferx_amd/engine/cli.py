@@ -51,6 +51,10 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--frequency-penalty", type=float, default=0.0)
     ap.add_argument("--repetition-penalty", type=float, default=1.0)
     ap.add_argument("--stop-token-ids", default="", help="comma-separated token ids that end a sequence")
+    ap.add_argument("--min-tokens", type=int, default=0, help="stop tokens do not end a sequence before this many")
+    ap.add_argument("--ignore-eos", action="store_true", help="generate through the model's end-of-sequence ids")
+    ap.add_argument("--logprobs", type=int, default=None, metavar="N",
+                    help="report each token's log-probability and those of the N most probable (0 to 20)")
     ap.add_argument("--seed", type=int, default=0, help="fixes the sampling draws")
     return ap
 
@@ -98,13 +102,19 @@ def main(argv: Optional[List[str]] = None) -> int:
         params = SamplingParams(max_tokens=args.max_tokens, temperature=args.temperature, top_p=args.top_p,
                                 top_k=args.top_k, min_p=args.min_p, presence_penalty=args.presence_penalty,
                                 frequency_penalty=args.frequency_penalty,
-                                repetition_penalty=args.repetition_penalty, stop_tokens=stop, seed=args.seed)
+                                repetition_penalty=args.repetition_penalty, stop_tokens=stop, seed=args.seed,
+                                min_tokens=args.min_tokens, ignore_eos=args.ignore_eos,
+                                want_logprobs=args.logprobs is not None, top_logprobs=args.logprobs or 0)
         results = engine.generate(prompts, params, with_reasons=True)
     except (ConfigError, CheckpointError, ValueError, OSError) as e:
         print(f"inferx-generate: {e}", file=sys.stderr)
         return 1
     for i, (tokens, reason) in enumerate(results):
-        print(json.dumps({"prompt": i, "output_token_ids": tokens, "finish_reason": reason}), flush=True)
+        line = {"prompt": i, "output_token_ids": tokens, "finish_reason": reason}
+        if args.logprobs is not None:
+            line["logprobs"] = [{"logprob": chosen, "top": [[t, lp] for t, lp in top]}
+                                for chosen, top in engine.last_completions[i].logprobs]
+        print(json.dumps(line), flush=True)
     return 0
 
 

@@ -11,6 +11,8 @@ ids out: tokenizers and servers are not part of this engine.
 """
 from __future__ import annotations
 
+import dataclasses
+
 import time
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Union
@@ -108,6 +110,12 @@ class LLMEngine:
         if request_id is None:
             request_id = self._next_id
             self._next_id += 1
+        # the model's end-of-sequence ids join the request's stop tokens unless it asks to generate through them
+        # (reference: src/engine/engine.cc:819-823)
+        params = params or SamplingParams()
+        eos = [t for t in getattr(self.runner.config, "eos_token_ids", []) if t not in params.stop_tokens]
+        if eos and not params.ignore_eos:
+            params = dataclasses.replace(params, stop_tokens=list(params.stop_tokens) + eos)
         self.scheduler.add_request(request_id, [int(t) for t in prompt_token_ids], params)
         return request_id
 

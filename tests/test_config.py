@@ -66,6 +66,8 @@ def test_which_layer_is_which():
     ({"mlp_only_layers": list(range(24))}, "no layer is sparse"),
     ({"decoder_sparse_step": 0}, "decoder_sparse_step"),
     ({"use_sliding_window": True, "sliding_window": 0}, "sliding_window"),
+    ({"eos_token_id": 151936}, "outside the vocabulary"),
+    ({"eos_token_id": "2"}, "eos_token_id"),
     ({"hidden_size": "2048"}, "must be int"),
     ({"num_hidden_layers": True}, "must be an integer"),
 ])
@@ -94,9 +96,15 @@ def test_not_json():
 
 
 def test_round_trip_through_to_dict():
-    for raw in tiny.CONFIGS.values():
+    for raw in list(tiny.CONFIGS.values()) + [{**tiny.CONFIG_A, "eos_token_id": 7}, {**tiny.CONFIG_B, "eos_token_id": [1, 2]}]:
         c = config_from_dict(raw)
         assert config_from_dict(c.to_dict()) == c
+
+
+def test_end_of_sequence_ids():
+    assert config_from_dict(A27B).eos_token_ids == []
+    assert config_from_dict({**A27B, "eos_token_id": 151643}).eos_token_ids == [151643]
+    assert config_from_dict({**A27B, "eos_token_id": [151645, 151643]}).eos_token_ids == [151645, 151643]
 
 
 def test_registering_another_architecture():

@@ -128,6 +128,27 @@ def test_stop_token_and_context_limit(tmp_path):
     assert out[0][1] == "context_limit" and len(out[0][0]) == 32 - 6 + 1
 
 
+def test_end_of_sequence_ids_of_the_model_stop_a_request_unless_it_ignores_them(tmp_path):
+    """config.json's eos_token_id joins every request's stop tokens (reference: src/engine/engine.cc:819-823)."""
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_A, 34, str(tmp_path / "plain"), "float32")
+    cfg, weights = tiny.read_folder(str(tmp_path / "plain"))
+    prompt = tiny.random_tokens(6, cfg["vocab_size"], 70)
+    want, _ = plain_greedy(cfg, weights, prompt, 8)
+    eos = want[2]
+    first = want.index(eos)
+    tiny.make_folder({**tiny.CONFIG_A, "eos_token_id": eos}, 34, str(tmp_path / "eos"), "float32")  # same weights
+    engine = LLMEngine(str(tmp_path / "eos"), "float32", max_num_seqs=2, max_model_len=32, num_gpu_blocks_override=8)
+    out = engine.generate([prompt], SamplingParams(max_tokens=8), with_reasons=True)
+    assert out[0] == (want[:first + 1], "stop_token")
+    out = engine.generate([prompt], SamplingParams(max_tokens=8, ignore_eos=True), with_reasons=True)
+    assert out[0] == (want, "max_tokens")
+    # before min_tokens the stop tokens are masked out of the choice: another token is taken in their place
+    got = engine.generate([prompt], SamplingParams(max_tokens=8, min_tokens=first + 2))[0]
+    assert got[:first] == want[:first] and eos not in got[:first + 2] and len(got) >= first + 2
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_decoding_and_first_tokens(tmp_path, dtype):
     """300 tokens one by one after a two-token start (graphs, page edges, the window), and every
@@ -198,6 +219,13 @@ def test_command_line(tmp_path):
     assert out.returncode == 0, out.stderr
     rec = json.loads(out.stdout.strip().splitlines()[-1])
     assert rec["output_token_ids"] == want and rec["finish_reason"] == "max_tokens"
+    more = subprocess.run(cmd + ["--logprobs", "2", "--ignore-eos", "--min-tokens", "1"], capture_output=True, text=True,
+                          timeout=300)
+    assert more.returncode == 0, more.stderr
+    rec = json.loads(more.stdout.strip().splitlines()[-1])
+    assert rec["output_token_ids"] == want and len(rec["logprobs"]) == 5
+    assert all(len(lp["top"]) == 2 and lp["logprob"] <= 0.0 and lp["top"][0][1] >= lp["top"][1][1] for lp in rec["logprobs"])
+    assert [lp["top"][0][0] for lp in rec["logprobs"]] == want  # greedy: the chosen token is the most probable one
     bad = subprocess.run(cmd[:2] + ["--no-such-flag"], capture_output=True, text=True, timeout=60)
     assert bad.returncode == 2
     missing = subprocess.run(cmd[:2] + ["--model", os.path.join(str(tmp_path), "nothing"), "--prompt-ids", "1"],
