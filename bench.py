@@ -2,8 +2,8 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B]
 
-A step is one decode step of the whole batch through the model runner (batch
-build, upload, every kernel, greedy choice of the next tokens).  Prints ONE
+A step is one decode step of the whole batch through the engine (scheduler,
+batch layout, upload, every kernel, greedy choice of the next tokens).  Prints ONE
 JSON line: decoded tokens a second at the default batch, the prefill of one
 2,048-token prompt, the decode step's HBM roofline fraction, and decode at
 batch 1 and 64.  One GPU only.
@@ -80,10 +80,11 @@ def main() -> int:
 
     import torch
     from inferx_amd.config import config_from_dict
+    from inferx_amd.engine.engine import LLMEngine
     from inferx_amd.engine.runner import ModelRunner
     from inferx_amd.engine.runtime import Runtime
     from inferx_amd.parts import build_model
-    from inferx_amd.sampling import Sampler, SamplingParams
+    from inferx_amd.sampling import SamplingParams
     from inferx_amd.weights import random_tensors
 
     raw = dict(SHAPE)
@@ -103,40 +104,35 @@ def main() -> int:
                          max_seq_len=CONTEXT, model=model)
     torch.cuda.synchronize()
     log(f"model ready in {time.time() - t0:.1f}s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB on the device")
-    sampler = Sampler(rt)
-    greedy = SamplingParams()
     gen = torch.Generator().manual_seed(1234)
 
     def prompt():
         return torch.randint(0, cfg.vocab_size, (PROMPT,), generator=gen).tolist()
 
     def run_decode(batch, steps, warmup):
-        """Prefill `batch` prompts of PROMPT tokens, then time `steps` decode steps."""
-        ids = [f"b{batch}_{i}" for i in range(batch)]
-        nxt = {}
-        for n, rid in enumerate(ids):
-            runner.add_request(rid)
-            logits = runner.run_entries([(rid, prompt(), [PROMPT - 1])])
-            nxt[rid] = sampler.sample(logits, [(greedy, 0, [])])[0]
-            if n % 8 == 7:
-                log(f"  prefilled {n + 1}/{batch}")
-
-        def one_step():
-            logits = runner.run_entries([(rid, [nxt[rid]], [0]) for rid in ids])
-            toks = sampler.sample(logits, [(greedy, 0, [])] * batch)
-            for rid, t in zip(ids, toks):
-                nxt[rid] = t
-
+        """`batch` requests with prompts of PROMPT tokens through the engine (scheduler, step function, sampler):
+        first their prompts, then `warmup` untimed and `steps` timed decode steps of the whole batch."""
+        engine = LLMEngine("", runner=runner, max_num_seqs=batch, max_model_len=CONTEXT, max_num_batched_tokens=PROMPT)
+        # (requests decode while the later prompts are still being read: room for those tokens too)
+        params = SamplingParams(max_tokens=warmup + steps + 3 * batch + 16, ignore_eos=True)
+        ids = [engine.add_request(prompt(), params) for _ in range(batch)]
+        while any(engine.scheduler.sequence(i).generated() == 0 for i in ids):  # the prompts, one a step
+            engine.step()
         for _ in range(warmup):
-            one_step()
+            engine.step()
         torch.cuda.synchronize()
+        before = engine.stats.tokens_out
         t = time.perf_counter()
         for _ in range(steps):
-            one_step()
+            engine.step()
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
-        for rid in ids:
-            runner.end_request(rid)
+        assert engine.stats.tokens_out - before == batch * steps, "a timed step was not a decode step of the whole batch"
+        for i in ids:
+            engine.cancel(i)
+        while engine.has_unfinished():
+            engine.step()
+        assert runner.cache.pools[0].used_pages == 0
         return dt
 
     # ---- prefill of one 2,048-token prompt ---------------------------------

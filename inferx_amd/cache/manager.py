@@ -76,6 +76,10 @@ def host_lib():
             "ixh_sched_plan_tokens": (i64, [vp]),
             "ixh_sched_plan": (None, [vp, i64p, i64p, i32p, i32p, i32p]),
             "ixh_sched_commit": (ci, [vp, i32p, ci]),
+            "ixh_sched_launched": (ci, [vp]),
+            "ixh_sched_resolve": (ci, [vp, i32p, ci]),
+            "ixh_sched_is_planned": (ci, [vp]),
+            "ixh_sched_plan_token_values": (None, [vp, i32p]),
             "ixh_sched_num_completed": (ci, [vp]),
             "ixh_sched_completed": (None, [vp, ci, i64p, i32p, i32p]),
             "ixh_sched_completed_tokens": (None, [vp, ci, i32p]),

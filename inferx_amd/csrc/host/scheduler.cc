@@ -46,6 +46,9 @@ struct Seq {
   int64_t max_tokens = 0, min_tokens = 0;
   std::vector<int32_t> stop;
   bool cancelled = false;
+  bool pending = false;  // its last token stands for a value that is still being sampled (see launched / resolve)
+  bool closing = false;  // it ends when that value arrives, whatever it is: plans leave it out
+  int close_reason = 0;
   int64_t draws = 0;  // sampled tokens so far: the counter of this request's random stream
   int64_t generated() const { return static_cast<int64_t>(tokens.size()) - prompt_len; }
 };
@@ -72,6 +75,8 @@ struct Sched {
   std::vector<Done> completed;
   std::vector<Part> plan;
   bool planned = false;
+  std::vector<Seq*> inflight;  // the sampling sequences of the step that was launched and not yet resolved
+  bool launched_step = false;
   int64_t preemptions = 0;
   std::string error;
 
@@ -80,6 +85,18 @@ struct Sched {
   void retire(std::unique_ptr<Seq> s, int reason) {
     completed.push_back({s->rid, reason, std::vector<int32_t>(s->tokens.begin() + s->prompt_len, s->tokens.end())});
     if (ixh_cache_contains(cache, s->rid)) ixh_cache_free(cache, s->rid);
+  }
+
+  // A sequence whose sampled value is still on its way cannot be let go yet: it is marked and ends at resolve.
+  void retire_or_close(size_t index, int reason) {
+    if (running[index]->pending) {
+      running[index]->closing = true;
+      running[index]->close_reason = reason;
+      return;
+    }
+    std::unique_ptr<Seq> gone = std::move(running[index]);
+    running.erase(running.begin() + static_cast<std::ptrdiff_t>(index));
+    retire(std::move(gone), reason);
   }
 
   void preempt(size_t index) {
@@ -93,6 +110,7 @@ struct Sched {
   void admit() {
     while (!waiting.empty() && static_cast<int>(running.size()) < max_running) {
       Seq& s = *waiting.front();
+      if (s.pending) return;  // preempted while its sampled value was on its way: it waits for that
       if (s.cancelled || static_cast<int64_t>(s.tokens.size()) > max_seq_len) {
         const int reason = s.cancelled ? kCancelled : kOutOfMemory;
         std::unique_ptr<Seq> gone = std::move(waiting.front());
@@ -115,7 +133,7 @@ struct Sched {
     std::vector<int64_t> t(running.size(), 0), pend(running.size(), 0);
     int64_t budget = max_batch_tokens;
     for (size_t i = 0; i < running.size(); ++i) {
-      pend[i] = pending(*running[i]);
+      pend[i] = running[i]->closing ? 0 : pending(*running[i]);
       if (budget > 0 && pend[i] == 1) {
         t[i] = 1;
         --budget;
@@ -136,10 +154,10 @@ struct Sched {
       return -1;
     }
     for (size_t i = 0; i < running.size();) {
-      if (running[i]->cancelled) {
-        std::unique_ptr<Seq> gone = std::move(running[i]);
-        running.erase(running.begin() + static_cast<std::ptrdiff_t>(i));
-        retire(std::move(gone), kCancelled);
+      if (running[i]->cancelled && !running[i]->closing) {
+        const size_t before = running.size();
+        retire_or_close(i, kCancelled);
+        if (running.size() == before) ++i;  // it is in flight and stays until its value has arrived
       } else {
         ++i;
       }
@@ -157,16 +175,12 @@ struct Sched {
         const int status = ixh_cache_reserve(cache, s.rid, ixh_cache_cached(cache, s.rid) + t[i]);
         if (status == kOk) continue;
         if (status == kContextFull) {
-          std::unique_ptr<Seq> gone = std::move(running[i]);
-          running.erase(running.begin() + static_cast<std::ptrdiff_t>(i));
-          retire(std::move(gone), kContext);
+          retire_or_close(i, kContext);
         } else {
           size_t victim = running.size() - 1;
           if (victim == i) {
             if (running.size() == 1) {
-              std::unique_ptr<Seq> gone = std::move(running[i]);
-              running.erase(running.begin());
-              retire(std::move(gone), kOutOfMemory);
+              retire_or_close(i, kOutOfMemory);
               replan = true;
               break;
             }
@@ -192,6 +206,99 @@ struct Sched {
     return static_cast<int>(plan.size());
   }
 
+  // The step has been handed to the device: what it wrote to the cache counts from now on, and every sequence that
+  // samples gets a place for the value that is on its way.  Another step may be planned (prepare) before that
+  // value is known; it is launched only after resolve.  Returns the number of values resolve will want.
+  int launched() {
+    if (!planned) {
+      error = "launched without prepare_step";
+      return -1;
+    }
+    if (launched_step) {
+      error = "launched twice without resolve";
+      return -2;
+    }
+    planned = false;
+    launched_step = true;
+    inflight.clear();
+    for (const Part& p : plan) {
+      Seq& s = *p.seq;
+      ixh_cache_commit(cache, s.rid, p.count);
+      if (!p.samples) continue;
+      s.tokens.push_back(-1);
+      ++s.draws;
+      s.pending = true;
+      if (!s.closing && s.generated() >= s.max_tokens) {
+        s.closing = true;
+        s.close_reason = kLength;
+      }
+      inflight.push_back(&s);
+    }
+    plan.clear();
+    return static_cast<int>(inflight.size());
+  }
+
+  // The sampled values of the launched step, in the order of its sampling sequences.  Sequences that end (stop
+  // token, length, or an ending put off while they were in flight) are let go.  Returns 1 if a step planned
+  // meanwhile named one of them (that plan is dropped: prepare again), 0 otherwise.
+  int resolve(const int32_t* sampled, int n) {
+    if (!launched_step) {
+      error = "resolve without a launched step";
+      return -1;
+    }
+    if (n != static_cast<int>(inflight.size())) {
+      error = std::to_string(n) + " sampled tokens for " + std::to_string(inflight.size()) + " sampling rows";
+      return -2;
+    }
+    launched_step = false;
+    std::vector<std::pair<Seq*, int>> finished;
+    for (int i = 0; i < n; ++i) {
+      Seq& s = *inflight[static_cast<size_t>(i)];
+      const int32_t token = sampled[i];
+      s.tokens.back() = token;
+      s.pending = false;
+      const bool is_stop = std::find(s.stop.begin(), s.stop.end(), token) != s.stop.end();
+      if (is_stop && s.generated() > s.min_tokens)
+        finished.push_back({&s, kStop});
+      else if (s.generated() >= s.max_tokens)
+        finished.push_back({&s, kLength});
+      else if (s.closing)
+        finished.push_back({&s, s.close_reason});
+      s.closing = false;
+    }
+    inflight.clear();
+    int stale = 0;
+    if (planned)
+      for (auto& f : finished)
+        for (const Part& p : plan)
+          if (p.seq == f.first) stale = 1;
+    if (stale) {
+      planned = false;
+      plan.clear();
+    }
+    for (auto& f : finished) {
+      bool gone_from_running = false;
+      for (size_t i = 0; i < running.size(); ++i)
+        if (running[i].get() == f.first) {
+          std::unique_ptr<Seq> gone = std::move(running[i]);
+          running.erase(running.begin() + static_cast<std::ptrdiff_t>(i));
+          retire(std::move(gone), f.second);
+          gone_from_running = true;
+          break;
+        }
+      if (gone_from_running) continue;
+      for (size_t i = 0; i < waiting.size(); ++i)  // it was preempted while its value was on its way
+        if (waiting[i].get() == f.first) {
+          std::unique_ptr<Seq> gone = std::move(waiting[i]);
+          waiting.erase(waiting.begin() + static_cast<std::ptrdiff_t>(i));
+          retire(std::move(gone), f.second);
+          break;
+        }
+    }
+    return stale;
+  }
+
+  // launched and resolve in one: the step has run and its values are known
   int commit(const int32_t* sampled, int n) {
     if (!planned) {
       error = "commit_step without prepare_step";
@@ -203,32 +310,9 @@ struct Sched {
       error = std::to_string(n) + " sampled tokens for " + std::to_string(want) + " sampling rows";
       return -2;
     }
-    planned = false;
-    std::vector<std::pair<Seq*, int>> finished;
-    int next = 0;
-    for (const Part& p : plan) {
-      Seq& s = *p.seq;
-      ixh_cache_commit(cache, s.rid, p.count);
-      if (!p.samples) continue;
-      const int32_t token = sampled[next++];
-      s.tokens.push_back(token);
-      ++s.draws;
-      const bool is_stop = std::find(s.stop.begin(), s.stop.end(), token) != s.stop.end();
-      if (is_stop && s.generated() > s.min_tokens)
-        finished.push_back({&s, kStop});
-      else if (s.generated() >= s.max_tokens)
-        finished.push_back({&s, kLength});
-    }
-    plan.clear();
-    for (auto& f : finished)
-      for (size_t i = 0; i < running.size(); ++i)
-        if (running[i].get() == f.first) {
-          std::unique_ptr<Seq> gone = std::move(running[i]);
-          running.erase(running.begin() + static_cast<std::ptrdiff_t>(i));
-          retire(std::move(gone), f.second);
-          break;
-        }
-    return 0;
+    const int rc = launched();
+    if (rc < 0) return rc;
+    return resolve(sampled, n) < 0 ? -3 : 0;
   }
 
   Seq* find(int64_t rid) {
@@ -300,6 +384,17 @@ void ixh_sched_plan(void* h, int64_t* rids, int64_t* first, int32_t* counts, int
   }
 }
 int ixh_sched_commit(void* h, const int32_t* sampled, int n) { return S(h)->commit(sampled, n); }
+int ixh_sched_launched(void* h) { return S(h)->launched(); }
+int ixh_sched_resolve(void* h, const int32_t* sampled, int n) { return S(h)->resolve(sampled, n); }
+int ixh_sched_is_planned(void* h) { return S(h)->planned ? 1 : 0; }
+// the tokens of the planned step again (flat, as ixh_sched_plan gives them): after resolve they are all known
+void ixh_sched_plan_token_values(void* h, int32_t* tokens) {
+  size_t at = 0;
+  for (const Part& p : S(h)->plan) {
+    std::copy(p.seq->tokens.begin() + p.first, p.seq->tokens.begin() + p.first + p.count, tokens + at);
+    at += static_cast<size_t>(p.count);
+  }
+}
 
 int ixh_sched_num_completed(void* h) { return static_cast<int>(S(h)->completed.size()); }
 void ixh_sched_completed(void* h, int i, int64_t* rid, int32_t* reason, int32_t* n_out) {

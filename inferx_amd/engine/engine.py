@@ -99,6 +99,8 @@ class LLMEngine:
         self.sampler = Sampler(runner.rt)
         self.stats = Stats()
         self._next_id = 0
+        self.plan_ahead = True  # plan and lay out the next step while the device runs this one
+        self._ahead = None      # (plan, batch) made that way
 
     # ---- requests -----------------------------------------------------------
     def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,
@@ -127,19 +129,35 @@ class LLMEngine:
 
     # ---- the loop -------------------------------------------------------------
     def step(self) -> List[Completion]:
-        """One scheduler step.  Returns the requests that finished in it."""
-        plan = self.scheduler.prepare_step()
-        if plan is None:
-            return self.scheduler.take_completed()
+        """One scheduler step.  Returns the requests that finished in it.
+
+        While the device runs the step, the host already plans and lays out the next one (the scheduler takes a
+        step in two halves: `launched` and `resolve`); when the sampled tokens arrive they are written into that
+        layout, which is then ready to go.  If one of its sequences has just ended the plan is dropped and made
+        again at the next call."""
+        if self._ahead is not None:
+            plan, batch = self._ahead
+            self._ahead = None
+        else:
+            plan = self.scheduler.prepare_step()
+            if plan is None:
+                return self.scheduler.take_completed()
+            batch = build_step_batch(self.runner.cache, plan.entries())
         t0 = time.perf_counter()
-        batch = build_step_batch(self.runner.cache, plan.entries())
         logits = self.runner.step(batch)
-        rows = []
-        for c in plan.contributions:
-            if c.samples:
-                rows.append(self.scheduler.sequence(c.rid).sampling_row())
-        sampled = self.sampler.sample(logits, rows)
-        self.scheduler.commit_step(sampled, self.sampler.last_logprobs)
+        rows = [self.scheduler.sequence(c.rid).sampling_row() for c in plan.contributions if c.samples]
+        pending = self.sampler.launch(logits, rows)
+        self.scheduler.launched()
+        nxt = nbatch = None
+        if self.plan_ahead:
+            nxt = self.scheduler.prepare_step()
+            if nxt is not None:
+                nbatch = build_step_batch(self.runner.cache, nxt.entries())
+        sampled = pending.result()
+        dropped = self.scheduler.resolve(sampled, self.sampler.last_logprobs)
+        if nxt is not None and not dropped:
+            nbatch.token_ids[:] = self.scheduler.plan_token_values(nxt)
+            self._ahead = (nxt, nbatch)
         self.stats.steps += 1
         self.stats.tokens_in += plan.num_tokens
         self.stats.tokens_out += len(sampled)

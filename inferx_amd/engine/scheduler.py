@@ -140,6 +140,7 @@ class Scheduler:
             raise RuntimeError("the scheduler could not be created")
         self._params: Dict[Hashable, SamplingParams] = {}
         self._logprobs: Dict[Hashable, List] = {}
+        self._in_flight: Optional[List[Hashable]] = None
         self._plan: Optional[StepPlan] = None
 
     def __del__(self):
@@ -245,19 +246,61 @@ class Scheduler:
 
     def commit_step(self, sampled: List[int], logprobs: Optional[List] = None) -> None:
         """`sampled`: one token per contribution that samples, in order; `logprobs`: what the sampler reported
-        for those rows (or None)."""
-        plan, self._plan = self._plan, None
+        for those rows (or None).  `launched` and `resolve` in one."""
+        plan = self._plan
         if plan is None:
             raise RuntimeError("commit_step without prepare_step")
-        arr = np.asarray([int(t) for t in sampled], dtype=np.int32)
-        rc = self._lib.ixh_sched_commit(self._h, _p32(arr) if len(arr) else None, len(arr))
-        if rc == -2:
+        want = sum(1 for c in plan.contributions if c.samples)
+        if len(sampled) != want:
+            raise ValueError(f"{len(sampled)} sampled tokens for {want} sampling rows")
+        self.launched()
+        self.resolve(sampled, logprobs)
+
+    # ---- a step in two halves: the next one can be planned while this one runs -----------------
+    def launched(self) -> None:
+        """The planned step has been handed to the device.  Its tokens count as cached from now on, and every
+        sequence that samples holds a place for the value that is on its way; `prepare_step` may be called
+        before `resolve` brings the values (the new plan's tokens of such places read -1 until then)."""
+        plan, self._plan = self._plan, None
+        if plan is None:
+            raise RuntimeError("launched without prepare_step")
+        rc = self._lib.ixh_sched_launched(self._h)
+        if rc < 0:
             self._plan = plan
+            raise RuntimeError(self._error())
+        self._in_flight = [c.rid for c in plan.contributions if c.samples]
+
+    def resolve(self, sampled: List[int], logprobs: Optional[List] = None) -> bool:
+        """The sampled values of the launched step.  True if a step planned meanwhile was dropped because one of
+        its sequences has just ended: plan again."""
+        rows, self._in_flight = self._in_flight, None
+        if rows is None:
+            raise RuntimeError("resolve without a launched step")
+        arr = np.asarray([int(t) for t in sampled], dtype=np.int32)
+        rc = self._lib.ixh_sched_resolve(self._h, _p32(arr) if len(arr) else None, len(arr))
+        if rc == -2:
+            self._in_flight = rows
             raise ValueError(self._error())
-        if rc != 0:
+        if rc < 0:
             raise RuntimeError(self._error())
         if logprobs is not None:
-            rows = [c.rid for c in plan.contributions if c.samples]
             for rid, lp in zip(rows, logprobs):
                 if lp is not None and rid in self._logprobs:
                     self._logprobs[rid].append(lp)
+        if rc == 1:
+            self._plan = None
+        return rc == 1
+
+    def plan_token_values(self, plan: StepPlan) -> np.ndarray:
+        """The tokens of the planned step, flat in the order of its contributions, as they are now (after `resolve`
+        no place is open any more); the plan's contributions are brought up to date too."""
+        if self._plan is not plan or not self._lib.ixh_sched_is_planned(self._h):
+            raise RuntimeError("this plan is not the planned step")
+        tokens = np.empty(plan.num_tokens, np.int32)
+        self._lib.ixh_sched_plan_token_values(self._h, _p32(tokens))
+        at, flat = 0, tokens.tolist()
+        for c in plan.contributions:
+            n = len(c.tokens)
+            c.tokens = flat[at:at + n]
+            at += n
+        return tokens

@@ -32,11 +32,16 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, rows: List[Row]) -> List[int]:
         """logits float32 [R, V] on the device (changed in place when penalties apply)."""
+        return self.launch(logits, rows).result()
+
+    def launch(self, logits: torch.Tensor, rows: List[Row]) -> "PendingSample":
+        """Queue the kernels that choose the rows' tokens; `result()` of what is returned waits for them and brings
+        the tokens to the host.  The caller can do other host work in between."""
         R = logits.shape[0]
         if R != len(rows):
             raise ValueError(f"{R} logits rows for {len(rows)} sampling rows")
         if R == 0:
-            return []
+            return PendingSample(self, None, rows, None)
         out = self.rt.empty((R,), torch.int32)
         masks = [list(p.stop_tokens) if len(gen) < p.min_tokens else [] for p, _, gen in rows]
         if any(p.needs_penalties for p, _, _ in rows) or any(masks):
@@ -71,15 +76,33 @@ class Sampler:
             ops.sample(logits, out, dev[0:R].view(torch.float32), dev[R:2 * R].view(torch.float32), dev[2 * R:3 * R],
                        dev[3 * R:4 * R].view(torch.float32), dev[4 * R:6 * R].view(torch.int64),
                        dev[6 * R:8 * R].view(torch.int64))
-        self.last_logprobs = None
+        lp = None
         if any(p.want_logprobs or p.top_logprobs for p, _, _ in rows):
             n_top = max(p.top_logprobs for p, _, _ in rows)
             chosen_lp = self.rt.empty((R,), torch.float32)
             top_ids = self.rt.empty((R, n_top), torch.int32)
             top_lp = self.rt.empty((R, n_top), torch.float32)
             ops.logprobs(logits, out, chosen_lp, top_ids, top_lp)
+            lp = (chosen_lp, top_ids, top_lp)
+        return PendingSample(self, out, rows, lp)
+
+
+class PendingSample:
+    """Tokens that the device is choosing."""
+
+    def __init__(self, sampler: Sampler, out, rows: List[Row], logprob_tensors):
+        self._sampler, self._out, self._rows, self._lp = sampler, out, rows, logprob_tensors
+
+    def result(self) -> List[int]:
+        """Waits for the device; also sets the sampler's `last_logprobs`."""
+        self._sampler.last_logprobs = None
+        if self._out is None:
+            return []
+        tokens = self._out.tolist()
+        if self._lp is not None:
+            chosen_lp, top_ids, top_lp = self._lp
             lp, ids, tlp = chosen_lp.tolist(), top_ids.tolist(), top_lp.tolist()
-            self.last_logprobs = [
+            self._sampler.last_logprobs = [
                 (lp[r], list(zip(ids[r][:p.top_logprobs], tlp[r][:p.top_logprobs])))
-                if (p.want_logprobs or p.top_logprobs) else None for r, (p, _, _) in enumerate(rows)]
-        return out.tolist()
+                if (p.want_logprobs or p.top_logprobs) else None for r, (p, _, _) in enumerate(self._rows)]
+        return tokens

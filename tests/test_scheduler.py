@@ -269,3 +269,80 @@ def test_random_arrivals_scarce_pages(seed):
             assert tight[r].output_tokens == free[r].output_tokens[:len(tight[r].output_tokens)]
         else:
             assert tight[r].reason == FINISH_LENGTH and tight[r].output_tokens == free[r].output_tokens
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_a_step_planned_while_the_last_one_runs(seed):
+    """The step in two halves: `launched` when it is handed to the device, `resolve` when its sampled values
+    arrive, and the next step planned and laid out in between.  With tokens a function of the position, stop
+    tokens that do occur, scarce pages (preemption while a value is on its way), cancellations and arrivals at
+    random steps, every request ends exactly once with the output and the reason of the run that plans one step
+    at a time; no page is lost; a plan that names a sequence which has just ended is dropped."""
+    import random
+    rng = random.Random(1000 + seed)
+    n_req = 14
+    prompts = {r: [rng.randrange(1000) for _ in range(rng.randrange(1, 40))] for r in range(n_req)}
+    limits = {r: rng.randrange(1, 30) for r in range(n_req)}
+    arrive = {r: rng.randrange(0, 25) for r in range(n_req)}
+    # a stop token that the request will meet (the token sampled at position p is fake_token(p))
+    stops = {r: [fake_token(len(prompts[r]) - 1 + rng.randrange(limits[r]))] if rng.random() < 0.5 else []
+             for r in range(n_req)}
+    min_tokens = {r: rng.randrange(0, 4) for r in range(n_req)}
+    cancel_at = {r: arrive[r] + rng.randrange(0, 12) for r in rng.sample(range(n_req), 3)}
+
+    def sampled_for(plan, batch):
+        return [fake_token(int(batch.positions[r])) for r in batch.logits_rows]
+
+    def run(pipelined, pages, budget, cancels):
+        sched, cache = make(pages=pages, page_size=4, max_running=4, budget=budget, max_seq_len=60)
+        done, step, dropped, ahead = [], 0, 0, None
+        while step < 60 or sched.has_work():
+            for r in range(n_req):
+                if arrive[r] == step:
+                    sched.add_request(r, prompts[r], P(limits[r], stop_tokens=stops[r], min_tokens=min_tokens[r]))
+                if cancels and cancel_at.get(r) == step:
+                    sched.cancel(r)
+            if ahead is None:
+                plan = sched.prepare_step()
+                batch = build_step_batch(cache, plan.entries()) if plan is not None else None
+            else:
+                plan, batch = ahead
+            ahead = None
+            if plan is not None:
+                assert 0 < plan.num_tokens <= budget and len(plan.contributions) <= 4
+                assert all(t >= 0 for t in batch.token_ids.tolist())  # no open place reaches the device
+                batch.validate(10 ** 6, [p.num_pages for p in cache.pools], cache.page_size)
+                values = sampled_for(plan, batch)
+                if not pipelined:
+                    sched.commit_step(values)
+                else:
+                    sched.launched()
+                    nxt = sched.prepare_step()  # while the device works
+                    nbatch = build_step_batch(cache, nxt.entries()) if nxt is not None else None
+                    stale = sched.resolve(values)
+                    if nxt is not None and not stale:
+                        nbatch.token_ids[:] = sched.plan_token_values(nxt)
+                        ahead = (nxt, nbatch)
+                    elif nxt is not None:
+                        dropped += 1
+            done += sched.take_completed()
+            cache.check()
+            step += 1
+            assert step < 5000
+        assert all(p.used_pages == 0 for p in cache.pools) and not cache.live_requests()
+        assert len(done) == n_req and len({c.rid for c in done}) == n_req
+        return {c.rid: c for c in done}, sched.preemptions, dropped
+
+    for pages, budget, cancels in ((400, 4096, False), (22, 24, True), (17, 9, False)):
+        one, _, _ = run(False, pages, budget, cancels)
+        two, preemptions, dropped = run(True, pages, budget, cancels)
+        for r in range(n_req):
+            if cancels and r in cancel_at:  # when a cancellation takes hold depends on the step it falls into
+                short, long = sorted((one[r].output_tokens, two[r].output_tokens), key=len)
+                assert long[:len(short)] == short
+            else:
+                assert (two[r].output_tokens, two[r].reason) == (one[r].output_tokens, one[r].reason), r
+        if pages == 400:
+            assert any(c.reason == FINISH_STOP for c in two.values()) and dropped > 0
+        else:
+            assert preemptions > 0
