@@ -207,6 +207,33 @@ def test_enforce_eager_gives_the_same_tokens_without_graphs(tmp_path):
     assert outs[0] == outs[1]
 
 
+def test_planning_the_next_step_ahead_changes_no_output(tmp_path):
+    """The engine plans and lays out the next step while the device runs this one.  With it and without it: the
+    same tokens and reasons, under stop tokens, min_tokens, seeded temperature sampling with cut-offs, penalties
+    and scarce pages (float32, so that a change of batch composition cannot flip a draw)."""
+    import random
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_B, 41, str(tmp_path), "float32")
+    vocab = tiny.CONFIG_B["vocab_size"]
+    rnd = random.Random(5)
+    prompts = [tiny.random_tokens(rnd.randint(1, 50), vocab, seed=300 + i) for i in range(9)]
+    params = [SamplingParams(max_tokens=rnd.randint(1, 18), temperature=rnd.choice([0.0, 0.7, 1.3]),
+                             top_p=rnd.choice([1.0, 0.9]), top_k=rnd.choice([0, 5]), seed=rnd.randrange(1000),
+                             stop_tokens=[rnd.randrange(vocab) for _ in range(rnd.choice([0, 20, 60]))],
+                             min_tokens=rnd.choice([0, 2]), repetition_penalty=rnd.choice([1.0, 1.2]),
+                             presence_penalty=rnd.choice([0.0, 0.5])) for _ in prompts]
+    outs = []
+    for ahead in (False, True):
+        engine = LLMEngine(str(tmp_path), "float32", max_num_seqs=4, max_model_len=80, max_num_batched_tokens=48,
+                           num_gpu_blocks_override=9)
+        engine.plan_ahead = ahead
+        outs.append(engine.generate(prompts, params, with_reasons=True))
+        assert engine.runner.cache.pools[0].used_pages == 0
+    assert outs[0] == outs[1]
+    assert any(r == "stop_token" for _, r in outs[1]) and any(r == "max_tokens" for _, r in outs[1])
+
+
 def test_command_line(tmp_path):
     tiny.make_folder(tiny.CONFIG_A, 37, str(tmp_path), "float32")
     cfg, weights = tiny.read_folder(str(tmp_path))
