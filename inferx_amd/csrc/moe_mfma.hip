@@ -27,11 +27,13 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // The work of one wavefront (KSPLIT == 1) or workgroup (KSPLIT == 4): rows [row0, row_end) x out-features
 // [n0, n0 + 16) of expert e.  `red`: LDS for the partial sums of a split reduction.
-template <int MT, bool GATE_UP, int KSPLIT, typename TO = __bf16>
+// PAIR: two blocks of 16 out-features side by side ([n0, n0 + 32)), so that the rows are read once for both.
+template <int MT, bool GATE_UP, int KSPLIT, typename TO = __bf16, bool PAIR = false>
 __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
                                              TO* __restrict__ out, const int32_t* __restrict__ rows, int e,
                                              int row0, int row_end, int n0, int n_out, int width, float* red) {
-  constexpr int NACC = GATE_UP ? 2 : 1;
+  static_assert(!(GATE_UP && PAIR), "the gate|up product already holds two blocks");
+  constexpr int NACC = (GATE_UP || PAIR) ? 2 : 1;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m = lane & 15, g = lane >> 4;
   const int kper = KSPLIT > 1 ? (((width + KSPLIT - 1) / KSPLIT + 127) & ~127) : width;
@@ -41,7 +43,8 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
   const int64_t w_rows = GATE_UP ? 2 * static_cast<int64_t>(n_out) : n_out;
   const int wrow = min(n0 + m, n_out - 1);  // rows past the end are computed and not stored
   const __bf16* wg = w + (static_cast<int64_t>(e) * w_rows + wrow) * width;
-  const __bf16* wu = wg + static_cast<int64_t>(n_out) * width;
+  const __bf16* wu = PAIR ? w + (static_cast<int64_t>(e) * w_rows + min(n0 + 16 + m, n_out - 1)) * width
+                          : wg + static_cast<int64_t>(n_out) * width;
 
   const __bf16* xr[MT];
 #pragma unroll
@@ -70,7 +73,7 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
       int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row per load
       kk = kk < kend ? kk : kbegin;  // (the range's first piece: it exists, kbegin + 8 g need not)
       w_[0][j] = *reinterpret_cast<const bf16x8*>(wg + kk);
-      if (GATE_UP) w_[1][j] = *reinterpret_cast<const bf16x8*>(wu + kk);
+      if (NACC == 2) w_[1][j] = *reinterpret_cast<const bf16x8*>(wu + kk);
 #pragma unroll
       for (int t = 0; t < MT; ++t) x_[t][j] = *reinterpret_cast<const bf16x8*>(xr[t] + kk);
     }
@@ -139,42 +142,46 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
     }
   }
 
-  // lane holds out-features n0 + 4 g + i of row row0 + 16 t + m
-  const int nb = n0 + 4 * g;
+  // lane holds out-features n0 + 4 g + i (and, of a pair, n0 + 16 + 4 g + i) of row row0 + 16 t + m
 #pragma unroll
-  for (int t = 0; t < MT; ++t) {
-    const int r = row0 + 16 * t + m;
-    if (r >= row_end) continue;
-    float v[4];
+  for (int u = 0; u < (PAIR ? 2 : 1); ++u) {
+    const int nb = n0 + 16 * u + 4 * g;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      v[i] = acc[0][t][i];
-      if (GATE_UP) v[i] = v[i] / (1.0f + __expf(-v[i])) * acc[1][t][i];
-    }
-    TO* dst = out + static_cast<int64_t>(r) * n_out + nb;
-    if (nb + 4 <= n_out && (n_out & 3) == 0) {
-      if constexpr (sizeof(TO) == 4) {
-        *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
-      } else {
-        bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
-        *reinterpret_cast<bf16x4*>(dst) = o;
+    for (int t = 0; t < MT; ++t) {
+      const int r = row0 + 16 * t + m;
+      if (r >= row_end) continue;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[i] = acc[u][t][i];
+        if (GATE_UP) v[i] = v[i] / (1.0f + __expf(-v[i])) * acc[1][t][i];
       }
-    } else {
+      TO* dst = out + static_cast<int64_t>(r) * n_out + nb;
+      if (nb + 4 <= n_out && (n_out & 3) == 0) {
+        if constexpr (sizeof(TO) == 4) {
+          *reinterpret_cast<f32x4*>(dst) = f32x4{v[0], v[1], v[2], v[3]};
+        } else {
+          bf16x4 o = {(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+          *reinterpret_cast<bf16x4*>(dst) = o;
+        }
+      } else {
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
-        if (nb + i < n_out) dst[i] = (TO)v[i];
+        for (int i = 0; i < 4; ++i)
+          if (nb + i < n_out) dst[i] = (TO)v[i];
+      }
     }
   }
 }
 
 // x [rows <= 16 * MT, width] . w[n_out, width]^T -> float32 [rows, n_out]: the head of a decoding step, whose
-// logits stay float32 (one workgroup per 16 out-features, the reduction split over its four wavefronts).
+// logits stay float32 (one workgroup per 32 out-features, so that the rows, which every workgroup reads, weigh
+// less beside the weights; the reduction split over its four wavefronts).
 template <int MT>
 __global__ void __launch_bounds__(256)
 linear_skinny_f32_kernel(const __bf16* x, const __bf16* w, float* __restrict__ out,
                          int rows, int n_out, int width) {
-  __shared__ float red[3 * 64 * MT * 4];
-  grouped_body<MT, false, 4, float>(x, w, out, nullptr, 0, 0, rows, blockIdx.x * 16, n_out, width, red);
+  __shared__ float red[3 * 64 * MT * 2 * 4];
+  grouped_body<MT, false, 4, float, true>(x, w, out, nullptr, 0, 0, rows, blockIdx.x * 32, n_out, width, red);
 }
 
 template <int MT, bool GATE_UP, int KSPLIT>
@@ -292,7 +299,7 @@ extern "C" int ix_linear_skinny_f32(const void* x, const void* w, float* out, in
   IX_REQUIRE(rows > 0 && rows <= 64 && n_out > 0 && width > 0, "between 1 and 64 rows, positive sizes");
   IX_REQUIRE(width % 8 == 0, "the reduction width must be a multiple of 8");
   IX_REQUIRE(n_out < (1ll << 31) - 16 && width < (1 << 30), "sizes too large");
-  dim3 grid(static_cast<unsigned>((n_out + 15) / 16)), block(256);
+  dim3 grid(static_cast<unsigned>((n_out + 31) / 32)), block(256);
   if (rows <= 16)
     hipLaunchKernelGGL(linear_skinny_f32_kernel<1>, grid, block, 0, stream, (const __bf16*)x, (const __bf16*)w, out,
                        rows, (int)n_out, (int)width);
