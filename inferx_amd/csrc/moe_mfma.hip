@@ -27,13 +27,12 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // The work of one wavefront (KSPLIT == 1) or workgroup (KSPLIT == 4): rows [row0, row_end) x out-features
 // [n0, n0 + 16) of expert e.  `red`: LDS for the partial sums of a split reduction.
-// PAIR: two blocks of 16 out-features side by side ([n0, n0 + 32)), so that the rows are read once for both.
-template <int MT, bool GATE_UP, int KSPLIT, typename TO = __bf16, bool PAIR = false>
+// NB: blocks of 16 out-features side by side ([n0, n0 + 16 NB)), so that the rows are read once for all of them.
+template <int MT, bool GATE_UP, int KSPLIT, typename TO = __bf16, int NB = 1>
 __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
                                              TO* __restrict__ out, const int32_t* __restrict__ rows, int e,
                                              int row0, int row_end, int n0, int n_out, int width, float* red) {
-  static_assert(!(GATE_UP && PAIR), "the gate|up product already holds two blocks");
-  constexpr int NACC = (GATE_UP || PAIR) ? 2 : 1;
+  constexpr int NACC = NB * (GATE_UP ? 2 : 1);  // accumulator b + NB h: block b of the gate (h = 0) or up (1) rows
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m = lane & 15, g = lane >> 4;
   const int kper = KSPLIT > 1 ? (((width + KSPLIT - 1) / KSPLIT + 127) & ~127) : width;
@@ -41,10 +40,12 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
   const int kend = min(width, kbegin + kper);
 
   const int64_t w_rows = GATE_UP ? 2 * static_cast<int64_t>(n_out) : n_out;
-  const int wrow = min(n0 + m, n_out - 1);  // rows past the end are computed and not stored
-  const __bf16* wg = w + (static_cast<int64_t>(e) * w_rows + wrow) * width;
-  const __bf16* wu = PAIR ? w + (static_cast<int64_t>(e) * w_rows + min(n0 + 16 + m, n_out - 1)) * width
-                          : wg + static_cast<int64_t>(n_out) * width;
+  const __bf16* wp[NACC];
+#pragma unroll
+  for (int u = 0; u < NACC; ++u) {
+    const int wrow = min(n0 + 16 * (u % NB) + m, n_out - 1);  // rows past the end are computed and not stored
+    wp[u] = w + (static_cast<int64_t>(e) * w_rows + (u / NB) * static_cast<int64_t>(n_out) + wrow) * width;
+  }
 
   const __bf16* xr[MT];
 #pragma unroll
@@ -72,8 +73,8 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
     for (int j = 0; j < 4; ++j) {
       int kk = k0 + 32 * j + 8 * g;  // the four lane groups cover 64 contiguous bytes of a row per load
       kk = kk < kend ? kk : kbegin;  // (the range's first piece: it exists, kbegin + 8 g need not)
-      w_[0][j] = *reinterpret_cast<const bf16x8*>(wg + kk);
-      if (NACC == 2) w_[1][j] = *reinterpret_cast<const bf16x8*>(wu + kk);
+#pragma unroll
+      for (int u = 0; u < NACC; ++u) w_[u][j] = *reinterpret_cast<const bf16x8*>(wp[u] + kk);
 #pragma unroll
       for (int t = 0; t < MT; ++t) x_[t][j] = *reinterpret_cast<const bf16x8*>(xr[t] + kk);
     }
@@ -142,9 +143,9 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
     }
   }
 
-  // lane holds out-features n0 + 4 g + i (and, of a pair, n0 + 16 + 4 g + i) of row row0 + 16 t + m
+  // lane holds out-features n0 + 16 u + 4 g + i of row row0 + 16 t + m
 #pragma unroll
-  for (int u = 0; u < (PAIR ? 2 : 1); ++u) {
+  for (int u = 0; u < NB; ++u) {
     const int nb = n0 + 16 * u + 4 * g;
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
@@ -154,7 +155,7 @@ __device__ __forceinline__ void grouped_body(const __bf16* a, const __bf16* w,
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         v[i] = acc[u][t][i];
-        if (GATE_UP) v[i] = v[i] / (1.0f + __expf(-v[i])) * acc[1][t][i];
+        if constexpr (GATE_UP) v[i] = v[i] / (1.0f + __expf(-v[i])) * acc[NB + u][t][i];
       }
       TO* dst = out + static_cast<int64_t>(r) * n_out + nb;
       if (nb + 4 <= n_out && (n_out & 3) == 0) {
@@ -181,7 +182,7 @@ __global__ void __launch_bounds__(256)
 linear_skinny_f32_kernel(const __bf16* x, const __bf16* w, float* __restrict__ out,
                          int rows, int n_out, int width) {
   __shared__ float red[3 * 64 * MT * 2 * 4];
-  grouped_body<MT, false, 4, float, true>(x, w, out, nullptr, 0, 0, rows, blockIdx.x * 32, n_out, width, red);
+  grouped_body<MT, false, 4, float, 2>(x, w, out, nullptr, 0, 0, rows, blockIdx.x * 32, n_out, width, red);
 }
 
 template <int MT, bool GATE_UP, int KSPLIT>
@@ -202,7 +203,7 @@ moe_grouped_mfma_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ o
 // n16_s * shared_tiles workgroups serve the shared expert, which is one more "expert" over all `shared_rows`
 // tokens with weights and sizes of its own (first, because its reduction may be the longer one and the last
 // workgroups to start set the kernel's end); the rest serve the routed experts' row tiles.
-template <int MT, bool GATE_UP>
+template <int MT, bool GATE_UP, int NB>
 __global__ void __launch_bounds__(256)
 moe_grouped_dual_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ out,
                         const int32_t* __restrict__ offsets, const int32_t* __restrict__ rows,
@@ -210,22 +211,23 @@ moe_grouped_dual_kernel(const __bf16* a, const __bf16* w, __bf16* __restrict__ o
                         const int32_t* __restrict__ tile_info, int max_tiles, int n_out, int width,
                         const __bf16* a_s, const __bf16* w_s, __bf16* __restrict__ out_s,
                         int shared_rows, int n_out_s, int width_s) {
-  __shared__ float red[3 * 64 * MT * (GATE_UP ? 2 : 1) * 4];
-  const int n16_s = (n_out_s + 15) / 16;
+  __shared__ float red[3 * 64 * MT * NB * (GATE_UP ? 2 : 1) * 4];
+  const int n16_s = (n_out_s + 16 * NB - 1) / (16 * NB);  // column blocks of 16 NB out-features
   const int shared_blocks = n16_s * ((shared_rows + 16 * MT - 1) / (16 * MT));
   int idx = blockIdx.x;
   if (idx < shared_blocks) {
     const int tile = idx / n16_s;
-    grouped_body<MT, GATE_UP, 4>(a_s, w_s, out_s, nullptr, 0, tile * 16 * MT, shared_rows, (idx - tile * n16_s) * 16,
+    grouped_body<MT, GATE_UP, 4, __bf16, NB>(a_s, w_s, out_s, nullptr, 0, tile * 16 * MT, shared_rows,
+                                             (idx - tile * n16_s) * 16 * NB,
                                  n_out_s, width_s, red);
   } else {
     idx -= shared_blocks;
-    const int n16_e = (n_out + 15) / 16;
+    const int n16_e = (n_out + 16 * NB - 1) / (16 * NB);
     const int tile = idx / n16_e;
     if (tile >= tile_info[0]) return;
     const int e = tile_expert[tile];
-    grouped_body<MT, GATE_UP, 4>(a, w, out, rows, e, tile_row0[tile], offsets[e + 1], (idx - tile * n16_e) * 16, n_out,
-                                 width, red);
+    grouped_body<MT, GATE_UP, 4, __bf16, NB>(a, w, out, rows, e, tile_row0[tile], offsets[e + 1],
+                                             (idx - tile * n16_e) * 16 * NB, n_out, width, red);
   }
 }
 
@@ -274,20 +276,23 @@ extern "C" int ix_moe_grouped_dual(const void* a, const void* w, void* out, cons
   IX_REQUIRE(width % 8 == 0 && width_s % 8 == 0, "the reduction widths must be multiples of 8");
   IX_REQUIRE(n_out < (1 << 24) && width < (1 << 30) && n_out_s < (1 << 24) && width_s < (1 << 30), "sizes too large");
   IX_REQUIRE(tile_rows == 16 || tile_rows == 32 || tile_rows == 64, "tile_rows must be 16, 32 or 64");
-  const int64_t n16_e = (n_out + 15) / 16, n16_s = (n_out_s + 15) / 16;
+  // one column block per workgroup: two (the rows read once for 32 out-features) measured slower at every tile
+  // height, 64 against 60 us for the gate|up product of a decoding step, for want of wavefronts in flight
+  const int nb = 1;
+  const int64_t n16_e = (n_out + 16 * nb - 1) / (16 * nb), n16_s = (n_out_s + 16 * nb - 1) / (16 * nb);
   const int64_t shared_tiles = (shared_rows + tile_rows - 1) / tile_rows;
   const int64_t blocks = n16_e * max_tiles + n16_s * shared_tiles;
   IX_REQUIRE(blocks < (1ll << 31), "too many workgroups");
   dim3 grid(static_cast<unsigned>(blocks)), block(256);
-#define LAUNCH(MT, GU)                                                                                            \
-  hipLaunchKernelGGL((moe_grouped_dual_kernel<MT, GU>), grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w, \
+#define LAUNCH(MT, GU, NB)                                                                                        \
+  hipLaunchKernelGGL((moe_grouped_dual_kernel<MT, GU, NB>), grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w, \
                      (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, max_tiles, (int)n_out,        \
                      (int)width, (const __bf16*)a_s, (const __bf16*)w_s, (__bf16*)out_s, shared_rows, (int)n_out_s, \
                      (int)width_s)
-#define PICK(MT)               \
-  if (gate_up) LAUNCH(MT, true); \
-  else LAUNCH(MT, false);
-  if (tile_rows == 16) { PICK(1) } else if (tile_rows == 32) { PICK(2) } else { PICK(4) }
+#define PICK(MT, NB)                 \
+  if (gate_up) LAUNCH(MT, true, NB); \
+  else LAUNCH(MT, false, NB);
+  if (tile_rows == 16) { PICK(1, 1) } else if (tile_rows == 32) { PICK(2, 1) } else { PICK(4, 1) }
 #undef PICK
 #undef LAUNCH
   return ix_check_launch("ix_moe_grouped_dual");
