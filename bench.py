@@ -170,7 +170,7 @@ def main() -> int:
         pts[f"decode_b{b}"] = round(b * steps / d, 1)
 
     line = {
-        "metric": "Qwen1.5-MoE-A2.7B decode tok/s @ batch 8 (2048-token prompts)",
+        "metric": f"Qwen1.5-MoE-A2.7B decode tok/s @ batch {args.batch} (2048-token prompts)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if elt == 2 else "fp32", "data": "synthetic: seeded random weights and token ids",

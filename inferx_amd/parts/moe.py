@@ -133,7 +133,7 @@ class MoeFeedForward(FeedForward):
     def route_and_dispatch(self, ctx, x, tile_rows: int):
         """`route` then `dispatch`; for few tokens the selection and the grouping share one launch."""
         rt, T, k, E = ctx.rt, x.shape[0], self.top_k, self.num_experts
-        if T * k > ops.SELECT_DISPATCH_MAX_ASSIGNMENTS or E > ops.SELECT_DISPATCH_MAX_EXPERTS:
+        if T * k > ops.SELECT_DISPATCH_PAYS_ASSIGNMENTS or E > ops.SELECT_DISPATCH_MAX_EXPERTS:
             topk_w, topk_e, gate = self.route(ctx, x)
             return (topk_w, topk_e, gate) + self.dispatch(ctx, topk_e, tile_rows)
         topk_w = rt.empty((T, k), torch.float32)
