@@ -329,58 +329,6 @@ moe_dispatch_wide_kernel(const int32_t* __restrict__ topk_e, int32_t* __restrict
   }
 }
 
-// Few assignments (decoding): one workgroup does counts, offsets, the stable placement and the tile map.
-// rank of assignment a within its expert = number of earlier assignments of the same expert.
-#define DISPATCH_SMALL_MAX 1024
-__global__ void __launch_bounds__(1024)
-moe_dispatch_small_kernel(const int32_t* __restrict__ topk_e, int32_t* __restrict__ offsets,
-                          int32_t* __restrict__ rows, int32_t* __restrict__ dest, int assignments, int experts, int k,
-                          int tile_rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
-                          int32_t* __restrict__ tile_info) {
-  __shared__ int32_t chosen[DISPATCH_SMALL_MAX];
-  __shared__ int32_t counts[IX_MAX_EXPERTS];
-  __shared__ int32_t first_row[IX_MAX_EXPERTS];
-  __shared__ int32_t first_tile[IX_MAX_EXPERTS];
-  const int tid = threadIdx.x;
-  for (int e = tid; e < experts; e += blockDim.x) counts[e] = 0;
-  if (tid < assignments) chosen[tid] = topk_e[tid];
-  __syncthreads();
-  int mine = -1, rank = 0;
-  if (tid < assignments) {
-    mine = chosen[tid];
-    for (int b = 0; b < tid; ++b) rank += (chosen[b] == mine) ? 1 : 0;
-    if (mine >= 0 && mine < experts) atomicAdd(&counts[mine], 1);  // integer counts: order does not matter
-  }
-  __syncthreads();
-  if (tid == 0) {
-    int32_t run = 0, tiles = 0;
-    for (int e = 0; e < experts; ++e) {
-      offsets[e] = run;
-      first_row[e] = run;
-      first_tile[e] = tiles;
-      run += counts[e];
-      if (tile_rows > 0) tiles += (counts[e] + tile_rows - 1) / tile_rows;
-    }
-    offsets[experts] = run;
-    if (tile_info) tile_info[0] = tiles;
-  }
-  __syncthreads();
-  if (tid < assignments && mine >= 0 && mine < experts) {
-    const int32_t r = first_row[mine] + rank;
-    rows[r] = tid / k;
-    dest[tid] = r;
-  }
-  if (tile_rows > 0 && tile_expert) {
-    for (int e = tid; e < experts; e += blockDim.x) {
-      const int n = (counts[e] + tile_rows - 1) / tile_rows;
-      for (int i = 0; i < n; ++i) {
-        tile_expert[first_tile[e] + i] = e;
-        tile_row0[first_tile[e] + i] = first_row[e] + i * tile_rows;
-      }
-    }
-  }
-}
-
 // tile_expert / tile_row0 need room for min(A, ceil(A / tile_rows) + E) entries; tile_rows 0 skips the map.
 extern "C" int ix_moe_dispatch(const int32_t* topk_e, int32_t* offsets, int32_t* rows, int32_t* dest,
                                int64_t assignments, int experts, int k, int tile_rows, int32_t* tile_expert,
@@ -389,11 +337,6 @@ extern "C" int ix_moe_dispatch(const int32_t* topk_e, int32_t* offsets, int32_t*
   IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
   IX_REQUIRE(tile_rows >= 0, "tile_rows must not be negative");
   IX_REQUIRE(tile_rows == 0 || (tile_expert && tile_row0 && tile_info), "tile map buffers needed");
-  if (assignments > 0 && assignments <= DISPATCH_SMALL_MAX) {
-    hipLaunchKernelGGL(moe_dispatch_small_kernel, dim3(1), dim3(1024), 0, stream, topk_e, offsets, rows, dest,
-                       (int)assignments, experts, k, tile_rows, tile_expert, tile_row0, tile_info);
-    return ix_check_launch("ix_moe_dispatch");
-  }
   hipLaunchKernelGGL(moe_dispatch_wide_kernel, dim3(experts), dim3(DW_THREADS), 0, stream, topk_e, offsets, rows, dest,
                      assignments, experts, k, tile_rows, tile_expert, tile_row0, tile_info);
   return ix_check_launch("ix_moe_dispatch");
@@ -563,27 +506,4 @@ extern "C" int ix_moe_combine(const void* y, int dtype, const int32_t* dest, con
   else
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_moe_combine");
-}
-
-// Router scores only: logits float32 [tokens, experts + 1] (the last column is the shared expert's gate score,
-// written when shared_gate_w is given).  For few tokens; selection and grouping then happen in
-// ix_moe_select_dispatch (moe_route_small.hip).
-extern "C" int ix_moe_route_logits(const void* x, int dtype, const void* wr, int wr_dtype, const void* shared_gate_w,
-                                   int sg_dtype, float* logits, int64_t tokens, int64_t width, int experts,
-                                   hipStream_t stream) {
-  IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
-  IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
-  IX_REQUIRE(dtype == IX_F32 || dtype == IX_BF16, "dtype must be float32 or bfloat16");
-  const size_t xs_bytes = ((width + 3) & ~3) * sizeof(float);
-  IX_REQUIRE(xs_bytes <= 60 * 1024, "hidden width too large for the router kernel (limit about 15000)");
-  if (tokens == 0) return 0;
-  const int rows = experts + (shared_gate_w ? 1 : 0);
-  dim3 grid(tokens, (rows + ROUTE_THREADS / 64 - 1) / (ROUTE_THREADS / 64)), block(ROUTE_THREADS);
-  if (dtype == IX_F32)
-    hipLaunchKernelGGL(moe_route_logits_kernel<float>, grid, block, xs_bytes, stream, (const float*)x, wr, wr_dtype,
-                       shared_gate_w, sg_dtype, logits, width, experts);
-  else
-    hipLaunchKernelGGL(moe_route_logits_kernel<bf16_t>, grid, block, xs_bytes, stream, (const bf16_t*)x, wr,
-                       wr_dtype, shared_gate_w, sg_dtype, logits, width, experts);
-  return ix_check_launch("ix_moe_route_logits");
 }

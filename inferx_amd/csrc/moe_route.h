@@ -38,9 +38,9 @@ __device__ __forceinline__ float route_row_dot(const float* __restrict__ xs, con
 // Selection and grouping for few tokens by ONE workgroup of NW wavefronts: softmax and top-k of every
 // token's router scores, then counts, offsets, the stable placement and the row-tile map.
 // `logits` float32 [tokens, experts + 1]; tokens * k <= SD_MAX_ASSIGN, experts <= SD_MAX_EXPERTS.
-// ACROSS: the scores were written by other workgroups of the same launch (with device-scope stores):
-// they are read with device-scope loads, which do not take a stale line from this die's L2.
-template <int NW, bool ACROSS>
+// The scores were written by other workgroups of the same launch (with device-scope stores): they are read with
+// device-scope loads, which do not take a stale line from this die's L2.
+template <int NW>
 __device__ __forceinline__ void
 select_dispatch_body(const float* logits, float* __restrict__ topk_w, int32_t* __restrict__ topk_e,
                      float* __restrict__ shared_gate, int32_t* __restrict__ offsets, int32_t* __restrict__ rows,
@@ -48,9 +48,7 @@ select_dispatch_body(const float* logits, float* __restrict__ topk_w, int32_t* _
                      int tile_rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
                      int32_t* __restrict__ tile_info) {
   static_assert(NW >= SD_MAX_EXPERTS / 64, "a thread per possible expert clears the counts");
-  auto fresh = [](const float* p) {
-    return ACROSS ? __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : *p;
-  };
+  auto fresh = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
   __shared__ float zs[NW][SD_MAX_EXPERTS];
   __shared__ int32_t chosen[SD_MAX_ASSIGN];
   __shared__ int32_t counts[SD_MAX_EXPERTS];

@@ -1,23 +1,10 @@
-// Selection and grouping for few tokens (decoding) in ONE workgroup: softmax and
-// top-k of every token's router scores, then counts, offsets, the stable
-// placement and the row-tile map.  Same arithmetic and tie rule as
-// moe_route_kernel / moe_dispatch_small_kernel in moe.hip (reference:
-// RouteTopKKernel src/backends/cuda/ops/moe.cu:36-127, MoeBuildDispatch :452-513).
+// Router scores, selection and grouping for up to 16 tokens (decoding) in ONE launch:
+// softmax and top-k of every token's router scores, then counts, offsets, the stable
+// placement and the row-tile map.  Same arithmetic and tie rule as moe_route_kernel /
+// moe_dispatch_wide_kernel in moe.hip (reference: RouteTopKKernel
+// src/backends/cuda/ops/moe.cu:36-127, MoeBuildDispatch :452-513).
 #include "common.h"
 #include "moe_route.h"
-
-#define SD_THREADS 1024
-
-__global__ void __launch_bounds__(SD_THREADS)
-moe_select_dispatch_kernel(const float* __restrict__ logits, float* __restrict__ topk_w, int32_t* __restrict__ topk_e,
-                           float* __restrict__ shared_gate, int32_t* __restrict__ offsets, int32_t* __restrict__ rows,
-                           int32_t* __restrict__ dest, int tokens, int experts, int k, int renormalize, float scale,
-                           int tile_rows, int32_t* __restrict__ tile_expert, int32_t* __restrict__ tile_row0,
-                           int32_t* __restrict__ tile_info) {
-  select_dispatch_body<SD_THREADS / 64, false>(logits, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens,
-                                               experts, k, renormalize, scale, tile_rows, tile_expert, tile_row0,
-                                               tile_info);
-}
 
 // At most 16 tokens: scores, selection and grouping in ONE launch.  The router rows are spread over many
 // workgroups, one row per wavefront, as in moe_route_logits_kernel (moe.hip); every workgroup counts itself
@@ -61,7 +48,7 @@ moe_route_dispatch_small_kernel(const T* __restrict__ x, const void* __restrict_
   __syncthreads();
   if (!is_last) return;
   if (tid == 0) __hip_atomic_store(arrived, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  select_dispatch_body<RF_THREADS / 64, true>(logits, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens,
+  select_dispatch_body<RF_THREADS / 64>(logits, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens,
                                               experts, k, renormalize, scale, tile_rows, tile_expert, tile_row0,
                                               tile_info);
 }
@@ -95,21 +82,4 @@ extern "C" int ix_moe_route_dispatch_small(const void* x, int dtype, const void*
                        wr_dtype, shared_gate_w, sg_dtype, logits, arrived, width, topk_w, topk_e, shared_gate, offsets,
                        rows, dest, tokens, experts, k, renormalize, scale, tile_rows, tile_expert, tile_row0, tile_info);
   return ix_check_launch("ix_moe_route_dispatch_small");
-}
-
-// logits float32 [tokens, experts + 1] from ix_moe_route_logits.  tokens * k <= 1024, experts <= 256, k <= 32.
-extern "C" int ix_moe_select_dispatch(const float* logits, float* topk_w, int32_t* topk_e, float* shared_gate,
-                                      int32_t* offsets, int32_t* rows, int32_t* dest, int tokens, int experts, int k,
-                                      int renormalize, float scale, int tile_rows, int32_t* tile_expert,
-                                      int32_t* tile_row0, int32_t* tile_info, hipStream_t stream) {
-  IX_REQUIRE(tokens > 0 && experts > 0 && k > 0, "sizes must be positive");
-  IX_REQUIRE(experts <= SD_MAX_EXPERTS, "at most 256 experts for the one-workgroup selection");
-  IX_REQUIRE(k <= experts && k <= 32, "top_k must be between 1 and min(experts, 32)");
-  IX_REQUIRE(static_cast<int64_t>(tokens) * k <= SD_MAX_ASSIGN, "at most 1024 assignments for the one-workgroup selection");
-  IX_REQUIRE(tile_rows >= 0, "tile_rows must not be negative");
-  IX_REQUIRE(tile_rows == 0 || (tile_expert && tile_row0 && tile_info), "tile map buffers needed");
-  hipLaunchKernelGGL(moe_select_dispatch_kernel, dim3(1), dim3(SD_THREADS), 0, stream, logits, topk_w, topk_e,
-                     shared_gate, offsets, rows, dest, tokens, experts, k, renormalize, scale, tile_rows, tile_expert,
-                     tile_row0, tile_info);
-  return ix_check_launch("ix_moe_select_dispatch");
 }

@@ -304,10 +304,8 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
           _i32(1 if renormalize else 0), _f32(scale), _stream())
 
 
-SELECT_DISPATCH_MAX_ASSIGNMENTS, SELECT_DISPATCH_MAX_EXPERTS = 1024, 256
-# Up to here one workgroup selects and groups as fast as a wavefront per token and a workgroup per expert in two
-# launches do (16.9 against 16.6 us at 32 tokens of 4 experts each out of 60; 26.6 against 18.9 us at 64 tokens)
-SELECT_DISPATCH_PAYS_ASSIGNMENTS = 128
+# the one-launch router: at most this many tokens, experts and bytes of one token as float32
+ROUTE_ONE_LAUNCH_EXPERTS, ROUTE_ONE_LAUNCH_ROW_BYTES = 256, 40 * 1024
 ROUTE_ONE_LAUNCH_TOKENS = 16
 _arrival_counters: dict = {}
 
@@ -321,19 +319,24 @@ def _arrival_counter(device: torch.device) -> torch.Tensor:
     return c
 
 
+def route_one_launch_fits(tokens: int, width: int, experts: int) -> bool:
+    """Whether `moe_route_dispatch` takes these sizes.  Beyond 16 tokens `moe_route` and `moe_dispatch` are as
+    fast (12.4 us both at 16 tokens of 4 experts each out of 60, 11.2 against 12.3 us at 8)."""
+    return (0 < tokens <= ROUTE_ONE_LAUNCH_TOKENS and experts <= ROUTE_ONE_LAUNCH_EXPERTS
+            and width * 4 <= ROUTE_ONE_LAUNCH_ROW_BYTES)
+
+
 def moe_route_dispatch(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor],
                        topk_w: torch.Tensor, topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor],
                        renormalize: bool, scale: float, offsets: torch.Tensor, rows: torch.Tensor,
                        dest: torch.Tensor, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None) -> None:
-    """`moe_route` and `moe_dispatch` for few tokens: router scores spread over many workgroups, then selection
-    and grouping in one workgroup; up to 16 tokens in one launch (the last workgroup to finish its scores goes
-    on), else in two.  Needs T * k <= 1024 and at most 256 experts."""
+    """`moe_route` and `moe_dispatch` for up to 16 tokens in one launch: the router scores are spread over many
+    workgroups, and the last one to finish its scores selects and groups (`route_one_launch_fits`)."""
     T, H = x.shape
     E = router_w.shape[0]
     k = topk_w.shape[1]
     A = T * k
-    _need(A <= SELECT_DISPATCH_MAX_ASSIGNMENTS and E <= SELECT_DISPATCH_MAX_EXPERTS and T > 0,
-          "too many assignments or experts for the fused selection")
+    _need(route_one_launch_fits(T, H, E), "too many tokens or experts, or too wide, for the one-launch router")
     _need(router_w.shape == (E, H), "router weight must be [experts, hidden]")
     _need(topk_w.shape == (T, k) and topk_w.dtype == torch.float32, "topk_w must be float32 [T, k]")
     _need(topk_e.shape == (T, k) and topk_e.dtype == torch.int32, "topk_e must be int32 [T, k]")
@@ -351,21 +354,12 @@ def moe_route_dispatch(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: O
         _is_i32(tile_map, 2 * mt + 1)
         te, tr, ti = tile_map[:mt], tile_map[mt:2 * mt], tile_map[2 * mt:]
     logits = torch.empty((T, E + 1), dtype=torch.float32, device=x.device)
-    if T <= ROUTE_ONE_LAUNCH_TOKENS and H * 4 <= 40 * 1024:
-        _call("ix_moe_route_dispatch_small", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)),
-              _ptr(shared_gate_w), _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits),
-              _ptr(_arrival_counter(x.device)), _i64(H), _ptr(topk_w), _ptr(topk_e),
-              _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest),
-              _i32(T), _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(tile_rows), _ptr(te),
-              _ptr(tr), _ptr(ti), _stream())
-        return
-    _call("ix_moe_route_logits", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
-          _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits), _i64(T), _i64(H), _i32(E),
-          _stream())
-    _call("ix_moe_select_dispatch", _ptr(logits), _ptr(topk_w), _ptr(topk_e),
-          _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest), _i32(T),
-          _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(tile_rows), _ptr(te), _ptr(tr), _ptr(ti),
-          _stream())
+    _call("ix_moe_route_dispatch_small", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)),
+          _ptr(shared_gate_w), _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits),
+          _ptr(_arrival_counter(x.device)), _i64(H), _ptr(topk_w), _ptr(topk_e),
+          _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest),
+          _i32(T), _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(tile_rows), _ptr(te),
+          _ptr(tr), _ptr(ti), _stream())
 
 
 def moe_dispatch(topk_e: torch.Tensor, offsets: torch.Tensor, rows: torch.Tensor, dest: torch.Tensor,

@@ -131,9 +131,9 @@ class MoeFeedForward(FeedForward):
         return rt.linear(rt.gated_linear(x, self.w_shared_gate_up), self.w_shared_down)
 
     def route_and_dispatch(self, ctx, x, tile_rows: int):
-        """`route` then `dispatch`; for few tokens the selection and the grouping share one launch."""
+        """`route` then `dispatch`; for the few tokens of a decoding step in one launch."""
         rt, T, k, E = ctx.rt, x.shape[0], self.top_k, self.num_experts
-        if T * k > ops.SELECT_DISPATCH_PAYS_ASSIGNMENTS or E > ops.SELECT_DISPATCH_MAX_EXPERTS:
+        if not ops.route_one_launch_fits(T, self.hidden_size, E):
             topk_w, topk_e, gate = self.route(ctx, x)
             return (topk_w, topk_e, gate) + self.dispatch(ctx, topk_e, tile_rows)
         topk_w = rt.empty((T, k), torch.float32)
