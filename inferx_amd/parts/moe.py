@@ -76,14 +76,17 @@ class MoeFeedForward(FeedForward):
         ops.moe_route(x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate, self.renormalize, self.routed_scale)
         return topk_w, topk_e, gate
 
-    def _tile_rows(self, x) -> int:
+    def _tile_rows(self, ctx, x) -> int:
         """Rows per tile of the matrix-core product, or 0 where it does not take the shapes (then the plain one runs)."""
         ok = (x.dtype == torch.bfloat16 and self.w13.dtype == torch.bfloat16 and self.w2.dtype == torch.bfloat16
               and self.hidden_size % 8 == 0 and self.expert_width % 8 == 0)
         if not ok:
             return 0
+        # A decoding step, or few rows per expert: 16-row tiles, the weights streamed by every wavefront for itself.
+        # From about three rows per expert on the LDS-staged kernel is faster (60 experts, 4 per token: 174 against
+        # 173 us for both products at 48 tokens, 209 against 189 at 96, 316 against 195 at 256).
         per_expert = x.shape[0] * self.top_k / self.num_experts
-        return 16 if per_expert <= 16 else (32 if per_expert <= 32 else ops.MOE_TILED_ROWS)
+        return 16 if (x.shape[0] <= ctx.rt.SKINNY_ROWS or per_expert <= 3) else ops.MOE_TILED_ROWS
 
     def dispatch(self, ctx, topk_e, tile_rows: int = 0):
         rt, A = ctx.rt, topk_e.numel()
@@ -104,9 +107,9 @@ class MoeFeedForward(FeedForward):
             ops.moe_grouped_tiled(x, self.w13, act, offsets, rows, tile_map, True)
             ops.moe_grouped_tiled(act, self.w2, y, offsets, None, tile_map, False)
         elif tile_rows:
-            k_split = 4 if A <= 1024 else 1  # few rows: the weights are the traffic, split the reduction
-            ops.moe_grouped_mfma(x, self.w13, act, offsets, rows, tile_map, tile_rows, True, k_split)
-            ops.moe_grouped_mfma(act, self.w2, y, offsets, None, tile_map, tile_rows, False, k_split)
+            # few rows: the weights are the traffic, the reduction is split over a workgroup's four wavefronts
+            ops.moe_grouped_mfma(x, self.w13, act, offsets, rows, tile_map, tile_rows, True, 4)
+            ops.moe_grouped_mfma(act, self.w2, y, offsets, None, tile_map, tile_rows, False, 4)
         else:
             ops.moe_grouped_plain(x, self.w13, act, offsets, rows, gate_up=True)
             ops.moe_grouped_plain(act, self.w2, y, offsets, None, gate_up=False)
@@ -114,7 +117,7 @@ class MoeFeedForward(FeedForward):
 
     def _one_launch(self, ctx, x, tile_rows: int) -> bool:
         """Few tokens (decoding): routed and shared experts go into one launch per product."""
-        return (tile_rows in (16, 32) and self.shared_width > 0 and self.shared_width % 8 == 0
+        return (tile_rows == 16 and self.shared_width > 0 and self.shared_width % 8 == 0
                 and x.shape[0] <= ctx.rt.SKINNY_ROWS and self.w_shared_gate_up.dtype == torch.bfloat16
                 and self.w_shared_down.dtype == torch.bfloat16)
 
@@ -148,7 +151,7 @@ class MoeFeedForward(FeedForward):
         return topk_w, topk_e, gate, offsets, rows, dest, tile_map
 
     def forward(self, ctx, x):
-        tile_rows = self._tile_rows(x)
+        tile_rows = self._tile_rows(ctx, x)
         topk_w, topk_e, gate, offsets, rows, dest, tile_map = self.route_and_dispatch(ctx, x, tile_rows)
         if self._one_launch(ctx, x, tile_rows):
             y, shared = self.experts_and_shared(ctx, x, offsets, rows, tile_map, tile_rows)
