@@ -311,11 +311,12 @@ _arrival_counters: dict = {}
 
 
 def _arrival_counter(device: torch.device) -> torch.Tensor:
-    """One int32 per device that the one-launch router's workgroups count themselves off on; every launch
-    leaves it zero.  Launches on one device follow one another on a stream, so they can share it."""
+    """Counters (one for the launch and one per token) per device that the one-launch router's workgroups count
+    themselves off on; every launch leaves them zero.  Launches on one device follow one another on a stream, so
+    they can share them."""
     c = _arrival_counters.get(device)
     if c is None:
-        c = _arrival_counters[device] = torch.zeros(1, dtype=torch.int32, device=device)
+        c = _arrival_counters[device] = torch.zeros(1 + ROUTE_ONE_LAUNCH_TOKENS, dtype=torch.int32, device=device)
     return c
 
 
@@ -326,12 +327,24 @@ def route_one_launch_fits(tokens: int, width: int, experts: int) -> bool:
             and width * 4 <= ROUTE_ONE_LAUNCH_ROW_BYTES)
 
 
-def moe_route_dispatch(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor],
+def moe_route_dispatch(x: Optional[torch.Tensor], router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor],
                        topk_w: torch.Tensor, topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor],
                        renormalize: bool, scale: float, offsets: torch.Tensor, rows: torch.Tensor,
-                       dest: torch.Tensor, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None) -> None:
+                       dest: torch.Tensor, tile_rows: int = 0, tile_map: Optional[torch.Tensor] = None,
+                       norm: Optional[tuple] = None) -> None:
     """`moe_route` and `moe_dispatch` for up to 16 tokens in one launch: the router scores are spread over many
-    workgroups, and the last one to finish its scores selects and groups (`route_one_launch_fits`)."""
+    workgroups, and the last one to finish its scores selects and groups (`route_one_launch_fits`).
+
+    With `norm` = (h, delta, weight, eps, x_out) the norm before the feed-forward is part of the launch too
+    (`x` is None then): x_out = rmsnorm(h + delta) * weight is written and routed, and h += delta."""
+    if norm is not None:
+        h, delta, gamma, eps, x_out = norm
+        _need(x is None, "x is made by the norm")
+        _need(h.dtype == torch.float32 and h.dim() == 2, "the residual stream is float32 [T, H]")
+        _need(delta.shape == h.shape and x_out.shape == h.shape and delta.dtype == x_out.dtype,
+              "delta and x_out must have the shape of h and one type")
+        _need(gamma.numel() == h.shape[1], "the norm weight must hold `hidden` numbers")
+        x = x_out
     T, H = x.shape
     E = router_w.shape[0]
     k = topk_w.shape[1]
@@ -354,12 +367,17 @@ def moe_route_dispatch(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: O
         _is_i32(tile_map, 2 * mt + 1)
         te, tr, ti = tile_map[:mt], tile_map[mt:2 * mt], tile_map[2 * mt:]
     logits = torch.empty((T, E + 1), dtype=torch.float32, device=x.device)
-    _call("ix_moe_route_dispatch_small", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)),
-          _ptr(shared_gate_w), _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits),
-          _ptr(_arrival_counter(x.device)), _i64(H), _ptr(topk_w), _ptr(topk_e),
-          _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest),
-          _i32(T), _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(tile_rows), _ptr(te),
-          _ptr(tr), _ptr(ti), _stream())
+    router = (_ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
+              _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(logits),
+              _ptr(_arrival_counter(x.device)), _i64(H), _ptr(topk_w), _ptr(topk_e),
+              _ptr(shared_gate if shared_gate_w is not None else None), _ptr(offsets), _ptr(rows), _ptr(dest),
+              _i32(T), _i32(E), _i32(k), _i32(1 if renormalize else 0), _f32(scale), _i32(tile_rows), _ptr(te),
+              _ptr(tr), _ptr(ti), _stream())
+    if norm is not None:
+        _call("ix_moe_norm_route_dispatch_small", _ptr(h), _ptr(delta), _i32(_dt(x_out)), _ptr(gamma),
+              _i32(_dt(gamma)), _f32(eps), _ptr(x_out), *router)
+    else:
+        _call("ix_moe_route_dispatch_small", _ptr(x), _i32(_dt(x)), *router)
 
 
 def moe_dispatch(topk_e: torch.Tensor, offsets: torch.Tensor, rows: torch.Tensor, dest: torch.Tensor,

@@ -72,6 +72,30 @@ def resolve_delta(ctx, delta):
     return delta.materialize(ctx) if isinstance(delta, LazyDelta) else delta
 
 
+class LazyNorm:
+    """What a block may hand to a feed-forward that says `takes_lazy_norm`, instead of the normalised tensor: the
+    norm and its operands, not applied yet, so that the feed-forward's first kernel can apply it (and update the
+    residual stream) on its way.  A feed-forward that does not fuse this case calls `materialize` and goes on
+    with the tensor; either way h has had `delta` added when the feed-forward returns."""
+
+    def __init__(self, norm, h, delta):
+        self.norm, self.h, self.delta = norm, h, delta
+
+    def materialize(self, ctx):
+        return self.norm.forward(ctx, self.h, self.delta)
+
+    def rms_operands(self):
+        """(weight, eps) if the norm is y = v * rsqrt(mean(v^2) + eps) * weight and `delta` is a tensor, else None."""
+        if isinstance(self.delta, LazyDelta) or self.delta is None:
+            return None
+        return self.norm.rms_operands()
+
+
+def resolve_input(ctx, x):
+    """A tensor whatever `x` is."""
+    return x.materialize(ctx) if isinstance(x, LazyNorm) else x
+
+
 class Part:
     # True if `forward` only launches work on the current stream (no host reads of device data, no host-side
     # planning from the batch), so that a step can be captured into a HIP graph
@@ -85,6 +109,10 @@ class Part:
 
 
 class Norm(Part):
+    def rms_operands(self):
+        """(weight, eps) if this is a plain RMS norm that another kernel may apply, else None."""
+        return None
+
     def forward(self, ctx, h, delta=None, rows=None):
         raise NotImplementedError
 
@@ -106,6 +134,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_lazy_norm = False  # True: `x` may be a LazyNorm (see there)
+
     def forward(self, ctx, x):
         raise NotImplementedError
 

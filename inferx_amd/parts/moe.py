@@ -15,7 +15,7 @@ from typing import List
 import torch
 
 from .. import ops
-from .base import FeedForward, LazyDelta, ParamSpec, register_part
+from .base import FeedForward, LazyDelta, LazyNorm, ParamSpec, register_part
 from .dense_mlp import stack_rows
 
 
@@ -133,10 +133,12 @@ class MoeFeedForward(FeedForward):
         rt = ctx.rt
         return rt.linear(rt.gated_linear(x, self.w_shared_gate_up), self.w_shared_down)
 
-    def route_and_dispatch(self, ctx, x, tile_rows: int):
-        """`route` then `dispatch`; for the few tokens of a decoding step in one launch."""
+    def route_and_dispatch(self, ctx, x, tile_rows: int, norm=None):
+        """`route` then `dispatch`; for the few tokens of a decoding step in one launch, and the norm before the
+        feed-forward with them: `norm` = (h, delta, weight, eps, x), x still to be filled."""
         rt, T, k, E = ctx.rt, x.shape[0], self.top_k, self.num_experts
         if not ops.route_one_launch_fits(T, self.hidden_size, E):
+            assert norm is None
             topk_w, topk_e, gate = self.route(ctx, x)
             return (topk_w, topk_e, gate) + self.dispatch(ctx, topk_e, tile_rows)
         topk_w = rt.empty((T, k), torch.float32)
@@ -146,13 +148,24 @@ class MoeFeedForward(FeedForward):
         rows = rt.empty((T * k,), torch.int32)
         dest = rt.empty((T * k,), torch.int32)
         tile_map = rt.empty((2 * ops.moe_max_tiles(T * k, E, tile_rows) + 1,), torch.int32) if tile_rows else None
-        ops.moe_route_dispatch(x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate, self.renormalize,
-                               self.routed_scale, offsets, rows, dest, tile_rows, tile_map)
+        ops.moe_route_dispatch(None if norm else x, self.w_router, self.w_shared_gate, topk_w, topk_e, gate,
+                               self.renormalize, self.routed_scale, offsets, rows, dest, tile_rows, tile_map, norm)
         return topk_w, topk_e, gate, offsets, rows, dest, tile_map
 
+    takes_lazy_norm = True
+
     def forward(self, ctx, x):
+        norm = None
+        if isinstance(x, LazyNorm):
+            # a decoding step: the norm is applied by the router's kernel, which every token's row passes anyway
+            rms = x.rms_operands()
+            if rms is not None and ops.route_one_launch_fits(x.h.shape[0], self.hidden_size, self.num_experts):
+                lazy, x = x, ctx.rt.empty(tuple(x.h.shape))
+                norm = (lazy.h, lazy.delta, rms[0], rms[1], x)
+            else:
+                x = x.materialize(ctx)
         tile_rows = self._tile_rows(ctx, x)
-        topk_w, topk_e, gate, offsets, rows, dest, tile_map = self.route_and_dispatch(ctx, x, tile_rows)
+        topk_w, topk_e, gate, offsets, rows, dest, tile_map = self.route_and_dispatch(ctx, x, tile_rows, norm)
         if self._one_launch(ctx, x, tile_rows):
             y, shared = self.experts_and_shared(ctx, x, offsets, rows, tile_map, tile_rows)
         else:

@@ -24,6 +24,9 @@ class RMSNorm(Norm):
     def bind(self, tensors, rt) -> None:
         self.weight = tensors["weight"].contiguous()
 
+    def rms_operands(self):
+        return self.weight, self.eps
+
     def forward(self, ctx, h, delta=None, rows=None):
         """h [T, width] float32 is updated in place with `delta` (unless `rows`
         picks rows out); returns the normalised rows in the run's type."""

@@ -310,3 +310,34 @@ def test_gather_then_combine_is_the_identity(dtype):
     assert rel_err(out, x.double() + gate.double()[:, None] * shared.double()) < (1e-6 if dtype == torch.float32 else 1e-2)
     ops.moe_combine(y, dest, topk_w, shared, None, out)  # an ungated shared expert adds exactly its output
     assert rel_err(out, x.double() + shared.double()) < (1e-6 if dtype == torch.float32 else 1e-2)
+
+
+@pytest.mark.parametrize("T,H,E,k", [(1, 64, 4, 2), (8, 2048, 60, 4), (16, 136, 60, 4), (5, 88, 7, 3), (13, 200, 256, 8)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_route_and_dispatch_in_one_launch(T, H, E, k, dtype):
+    """The norm before the feed-forward as part of the one-launch router: the residual stream is brought up to
+    date exactly, the normalised rows are those of the separate norm kernel up to the rounding of one sum, and
+    the routing is exactly that of the separate kernels on the rows it wrote."""
+    from inferx_amd import ops
+    mk = lambda *shape, dt=torch.int32: torch.full(shape, -9, dtype=dt, device=DEV)
+    h0, delta = rnd(T, H, seed=3, dtype=torch.float32, scale=2.0), rnd(T, H, seed=4, dtype=dtype)
+    gamma = (1.0 + rnd(H, seed=5, dtype=torch.float32, scale=0.2)).to(dtype)
+    wr, wsg = rnd(E, H, seed=1, dtype=dtype, scale=0.3), rnd(1, H, seed=2, dtype=dtype, scale=0.1)
+    eps = 1e-5
+    h1, x1 = h0.clone(), torch.empty(T, H, dtype=dtype, device=DEV)
+    ops.add_rmsnorm(h1, delta, gamma, x1, eps)
+    for tile_rows in (0, 16):
+        h2, x2 = h0.clone(), torch.full((T, H), 7.0, dtype=dtype, device=DEV)
+        w2, e2, g2 = mk(T, k, dt=torch.float32), mk(T, k), mk(T, dt=torch.float32)
+        o2, r2, d2 = mk(E + 1), mk(T * k), mk(T * k)
+        tm2 = mk(2 * ops.moe_max_tiles(T * k, E, tile_rows) + 1) if tile_rows else None
+        ops.moe_route_dispatch(None, wr, wsg, w2, e2, g2, True, 1.0, o2, r2, d2, tile_rows, tm2,
+                               norm=(h2, delta, gamma, eps, x2))
+        assert torch.equal(h2, h1)
+        ulp = 2.0 ** -7 if dtype == torch.bfloat16 else 2.0 ** -21
+        assert ((x2.float() - x1.float()).abs() <= ulp * x1.float().abs() + 1e-30).all()
+        w1, e1, g1 = mk(T, k, dt=torch.float32), mk(T, k), mk(T, dt=torch.float32)
+        ops.moe_route(x2, wr, wsg, w1, e1, g1, True, 1.0)
+        o1, r1, d1, tm1 = dispatch(e1, E, tile_rows)
+        assert torch.equal(e1, e2) and torch.equal(o1, o2) and torch.equal(r1, r2) and torch.equal(d1, d2)
+        assert rel_err(w2, w1) < 1e-6 and rel_err(g2, g1) < 1e-6
