@@ -184,7 +184,7 @@ def test_layer_order_is_data(tmp_path, dtype, tol):
 def define_toy_routed():
     from inferx_amd.config import ModelSpec, PartSpec, ScheduleEntry, register_architecture
     from inferx_amd.config.spec import LayerSpec
-    from inferx_amd.parts import FeedForward, ParamSpec, PositionEncoding, register_part
+    from inferx_amd.parts import FeedForward, LazyNorm, ParamSpec, PositionEncoding, register_part, resolve_input
 
     class StretchedRotary(PositionEncoding):
         def __init__(self, theta, rotary_dim, stretch):
@@ -213,7 +213,11 @@ def define_toy_routed():
         def bind(self, tensors, rt):
             self.wr, self.w1, self.w2 = (tensors[n].float() for n in ("router.weight", "w1", "w2"))
 
+        takes_lazy_norm = True  # the block hands the norm before this part over unapplied; it is applied here
+
         def forward(self, ctx, x):
+            assert isinstance(x, LazyNorm)
+            x = resolve_input(ctx, x)
             xf = x.float()
             e = torch.argmax(xf @ self.wr.T, dim=-1)
             hidden = torch.relu(torch.einsum("twh,th->tw", self.w1[e], xf))
