@@ -298,6 +298,27 @@ qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __rest
   const bool cache_ok = k_cache != nullptr && slot >= 0 && slot < total_slots;
   const int64_t page = cache_ok ? slot / page_size : 0;
   const int off = cache_ok ? static_cast<int>(slot % page_size) : 0;
+  // eight bias values from column c on (c is a multiple of 8): one or two 16-byte loads where the bias allows it
+  const bool bias_vec = (reinterpret_cast<uintptr_t>(bias) & 15) == 0;
+  auto add_bias8 = [&](float (&v)[8], int c) {
+    if (bias_vec && bias_dtype == IX_BF16) {
+      const uint4 b = *reinterpret_cast<const uint4*>(static_cast<const uint16_t*>(bias) + c);
+      const uint32_t w[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        v[2 * i] += __uint_as_float(w[i] << 16);
+        v[2 * i + 1] += __uint_as_float(w[i] & 0xffff0000u);
+      }
+    } else if (bias_vec && bias_dtype == IX_F32) {
+      const float4 a = *reinterpret_cast<const float4*>(static_cast<const float*>(bias) + c);
+      const float4 b = *reinterpret_cast<const float4*>(static_cast<const float*>(bias) + c + 4);
+      v[0] += a.x; v[1] += a.y; v[2] += a.z; v[3] += a.w;
+      v[4] += b.x; v[5] += b.y; v[6] += b.z; v[7] += b.w;
+    } else {
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v[i] += ix_load_rt(bias, bias_dtype, c + i);
+    }
+  };
   for (int p = blockIdx.y * blockDim.x + threadIdx.x; p < items; p += gridDim.y * blockDim.x) {
     const int head = p / per_head, j = (p - head * per_head) * 8;
     const int col = head * head_dim + j;
@@ -313,21 +334,21 @@ qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __rest
       hi[2 * i + 1] = __uint_as_float(hw[i] & 0xffff0000u);
     }
     if (bias) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        lo[i] += ix_load_rt(bias, bias_dtype, col + i);
-        hi[i] += ix_load_rt(bias, bias_dtype, col + half + i);
-      }
+      add_bias8(lo, col);
+      add_bias8(hi, col + half);
     }
     const bool is_v = head >= heads + kv_heads;
     if (!is_v && cs) {
+      // eight (cos, sin) pairs are 64 contiguous bytes (the table is float32 [T, half, 2], a row a multiple of 64 bytes)
+      const float4* c4 = reinterpret_cast<const float4*>(cs + t * half + j);
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float2 c = cs[t * half + j + i];
-        const float rlo = lo[i] * c.x - hi[i] * c.y;
-        const float rhi = hi[i] * c.x + lo[i] * c.y;
-        lo[i] = rlo;
-        hi[i] = rhi;
+      for (int i = 0; i < 4; ++i) {
+        const float4 c = c4[i];
+        const float l0 = lo[2 * i], h0 = hi[2 * i], l1 = lo[2 * i + 1], h1 = hi[2 * i + 1];
+        lo[2 * i] = l0 * c.x - h0 * c.y;
+        hi[2 * i] = h0 * c.x + l0 * c.y;
+        lo[2 * i + 1] = l1 * c.z - h1 * c.w;
+        hi[2 * i + 1] = h1 * c.z + l1 * c.w;
       }
     }
     uint16_t lb[8], hb[8];
@@ -420,7 +441,7 @@ extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, 
     hipLaunchKernelGGL(qkv_rope_append_kernel<float>, grid, block, 0, stream, (const float*)qkv, bias, bias_dtype,
                        (const float2*)cs, slots, (float*)q_out, (float*)k_cache, (float*)v_cache, heads, kv_heads,
                        head_dim, page_size, total_slots);
-  else if (dtype == IX_BF16 && head_dim % 16 == 0) {
+  else if (dtype == IX_BF16 && head_dim % 16 == 0 && (reinterpret_cast<uintptr_t>(cs) & 15) == 0) {
     // from a few dozen tokens on, the values go through the kernel that turns tiles of them
     const int skip_v = (tokens >= 2 * V_TILE_TOKENS && v_cache != nullptr && slots != nullptr && kv_heads <= 65535) ? 1 : 0;
     const int items8 = (heads + (skip_v ? 1 : 2) * kv_heads) * (head_dim / 16);
