@@ -42,10 +42,34 @@ class Runtime:
         ops.lib()  # fail now, loudly, if the HIP library cannot be had
         self._mm_out_dtype_ok: Optional[bool] = None
         self._skinny_plans: Dict[int, Any] = {}
+        self._side_stream: Optional[torch.cuda.Stream] = None
 
     @property
     def is_fp32(self) -> bool:
         return self.dtype == torch.float32
+
+    # ---- work beside the main stream ------------------------------------------------------------------
+    def can_run_beside(self) -> bool:
+        """Not while a graph is being captured: a captured step stays on one stream."""
+        return not torch.cuda.is_current_stream_capturing()
+
+    def run_beside(self, fn):
+        """Runs fn() on a second stream (of the default priority) that starts from the main stream's present
+        state, and returns (fn's tensor, join): the main stream goes on at once, and `join()` makes it wait for
+        fn's work.  What fn allocates belongs to the second stream; the tensor it returns is marked as used by
+        the main stream too, so that its memory is not given out again before the main stream is done with it."""
+        main = torch.cuda.current_stream(self.device)
+        if self._side_stream is None:
+            self._side_stream = torch.cuda.Stream(self.device)
+        side = self._side_stream
+        side.wait_stream(main)
+        with torch.cuda.stream(side):
+            out = fn()
+        out.record_stream(main)
+
+        def join():
+            main.wait_stream(side)
+        return out, join
 
     def empty(self, shape, dtype=None) -> torch.Tensor:
         return torch.empty(shape, dtype=dtype or self.dtype, device=self.device)

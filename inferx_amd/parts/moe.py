@@ -19,6 +19,9 @@ from .base import FeedForward, LazyDelta, LazyNorm, ParamSpec, register_part
 from .dense_mlp import stack_rows
 
 
+SHARED_BESIDE_TOKENS = 256  # from here on the shared expert runs on a second stream beside the routed ones
+
+
 class MoeFeedForward(FeedForward):
     graph_safe = True
 
@@ -165,12 +168,22 @@ class MoeFeedForward(FeedForward):
             else:
                 x = x.materialize(ctx)
         tile_rows = self._tile_rows(ctx, x)
+        one_launch = self._one_launch(ctx, x, tile_rows)
+        shared = join = None
+        if (not one_launch and self.shared_width > 0 and tile_rows == ops.MOE_TILED_ROWS
+                and x.shape[0] >= SHARED_BESIDE_TOKENS and ctx.rt.can_run_beside()):
+            # a prompt portion: the shared expert's library products are bound by the matrix cores, the routed
+            # experts' kernels by memory, so the two run beside each other on two streams
+            shared, join = ctx.rt.run_beside(lambda: self.shared(ctx, x))
         topk_w, topk_e, gate, offsets, rows, dest, tile_map = self.route_and_dispatch(ctx, x, tile_rows, norm)
-        if self._one_launch(ctx, x, tile_rows):
+        if one_launch:
             y, shared = self.experts_and_shared(ctx, x, offsets, rows, tile_map, tile_rows)
         else:
             y = self.experts(ctx, x, offsets, rows, tile_map, tile_rows)
-            shared = self.shared(ctx, x) if self.shared_width > 0 else None
+            if join is not None:
+                join()
+            elif self.shared_width > 0:
+                shared = self.shared(ctx, x)
         return MoeSum(y, dest, topk_w, shared, gate, self.hidden_size)
 
 

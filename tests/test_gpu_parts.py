@@ -168,6 +168,46 @@ def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated, T):
                        again.view(torch.int16 if dtype == "bfloat16" else torch.int32))
 
 
+def test_shared_expert_beside_the_routed_ones():
+    """A prompt portion: the shared expert runs on a second stream beside the routed experts.  The sum is bit for
+    bit that of one stream, also when the calls follow one another without a wait (memory of one call is given
+    out again to the next) and under work that keeps the main stream busy."""
+    from inferx_amd.config import PartSpec
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_part, moe, resolve_delta
+    rt = Runtime("bfloat16")
+    H, T = 136, 640
+    part = build_part("feed_forward", PartSpec("moe", {
+        "hidden_size": H, "num_experts": 8, "top_k": 2, "expert_width": 72, "shared_width": 200,
+        "shared_gated": True, "renormalize": False, "init_std": 0.15}))
+    part.bind({n: v.to(DEV) for n, v in tensors_for(part, rt, seed=3).items()}, rt)
+    ctx, _ = make_ctx(rt, [T], [T], 16, 41)
+    xs = [torch.randn(T, H, generator=torch.Generator().manual_seed(s)).to(rt.dtype).to(DEV) for s in range(6)]
+    assert part._tile_rows(ctx, xs[0]) == ops_tiled_rows() and rt.can_run_beside()
+    threshold = moe.SHARED_BESIDE_TOKENS
+    try:
+        moe.SHARED_BESIDE_TOKENS = 1 << 30
+        want = [resolve_delta(ctx, part.forward(ctx, x)) for x in xs]
+        moe.SHARED_BESIDE_TOKENS = 256
+        assert rt._side_stream is None
+        busy = torch.randn(2048, 2048, device=DEV)
+        got = []
+        for x in xs:  # no wait between the calls
+            busy = busy @ busy * 1e-3
+            got.append(resolve_delta(ctx, part.forward(ctx, x)))
+        assert rt._side_stream is not None
+    finally:
+        moe.SHARED_BESIDE_TOKENS = threshold
+    torch.cuda.synchronize()
+    for g, w in zip(got, want):
+        assert torch.equal(g.view(torch.int16), w.view(torch.int16))
+
+
+def ops_tiled_rows():
+    from inferx_amd import ops
+    return ops.MOE_TILED_ROWS
+
+
 @pytest.mark.parametrize("dtype,tol", PARAMS)
 def test_norm_fuses_the_expert_sum(dtype, tol):
     """The norm forms a lazy expert sum itself: same stream and same output as sum, add, norm one after the other."""
