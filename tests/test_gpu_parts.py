@@ -132,7 +132,7 @@ def test_dense_mlp_part(dtype, tol):
 @pytest.mark.parametrize("H,E,k,mi,si,renorm,gated", [(64, 4, 2, 32, 64, False, True), (96, 8, 3, 48, 80, True, True),
                                                       (72, 5, 1, 40, 0, False, True), (64, 6, 6, 32, 48, True, False),
                                                       (64, 1, 1, 32, 0, False, True)])
-@pytest.mark.parametrize("T", [29, 7])  # 7: the few-token path (experts and shared expert in one launch)
+@pytest.mark.parametrize("T", [40, 29, 7])  # 7, 29: the few-token path (experts and shared expert in one launch)
 def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated, T):
     from inferx_amd.config import PartSpec
     from inferx_amd.engine.runtime import Runtime
