@@ -7,6 +7,12 @@ batch layout, upload, every kernel, greedy choice of the next tokens).  Prints O
 JSON line: decoded tokens a second at the default batch, the prefill of one
 2,048-token prompt, the decode step's HBM roofline fraction, and decode at
 batch 1 and 64.  One GPU only.
+
+Two further workloads at the Qwen2-57B-A14B shape, each with a JSON line of the same form:
+
+    python bench.py --workload mixed [--layers L]   # 32 decodes at a context of 4,096 beside 2 prompt portions of 512
+    python bench.py --workload long [--layers L]    # batch 8, prompts of 16,384 to 32,000 tokens in portions of
+                                                    # 2,048, then --steps decode steps (default there: 256)
 """
 from __future__ import annotations
 
@@ -26,6 +32,15 @@ SHAPE = {
     "num_experts_per_tok": 4, "moe_intermediate_size": 1408, "shared_expert_intermediate_size": 5632,
     "intermediate_size": 5632, "decoder_sparse_step": 1, "mlp_only_layers": [], "norm_topk_prob": False,
     "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 8192,
+    "use_sliding_window": False, "tie_word_embeddings": False,
+}
+# Qwen2-57B-A14B's sizes
+SHAPE_57B = {
+    "architectures": ["Qwen2MoeForCausalLM"], "num_hidden_layers": 28, "hidden_size": 3584,
+    "num_attention_heads": 28, "num_key_value_heads": 4, "head_dim": 128, "num_experts": 64,
+    "num_experts_per_tok": 8, "moe_intermediate_size": 2560, "shared_expert_intermediate_size": 20480,
+    "intermediate_size": 18944, "decoder_sparse_step": 1, "mlp_only_layers": [], "norm_topk_prob": False,
+    "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6, "max_position_embeddings": 32768,
     "use_sliding_window": False, "tie_word_embeddings": False,
 }
 CONTEXT = 4096
@@ -62,13 +77,165 @@ def prefill_flops(cfg, tokens):
     return linear + attention
 
 
+def step_bytes(cfg, tokens, cache_tokens, elt):
+    """Bytes a step of `tokens` tokens has to read: every weight it uses once, and `cache_tokens` of cache."""
+    H, L = cfg.hidden_size, cfg.num_hidden_layers
+    qd, kvd = cfg.q_dim, cfg.kv_dim
+    E, k, mi, si = cfg.num_experts, cfg.num_experts_per_tok, cfg.moe_intermediate_size, cfg.shared_expert_intermediate_size
+    distinct = E * (1.0 - (1.0 - k / E) ** tokens)
+    per_layer = (qd + 2 * kvd) * H + (qd + 2 * kvd) + H * qd + 2 * H + E * H + distinct * 3 * mi * H + 3 * si * H + H
+    return (L * per_layer + H + cfg.vocab_size * H + L * 2 * kvd * cache_tokens) * elt
+
+
+def linear_flops(cfg, tokens, head_rows):
+    H, L = cfg.hidden_size, cfg.num_hidden_layers
+    qd, kvd = cfg.q_dim, cfg.kv_dim
+    E, k, mi, si = cfg.num_experts, cfg.num_experts_per_tok, cfg.moe_intermediate_size, cfg.shared_expert_intermediate_size
+    per_token = (qd + 2 * kvd) * H + H * qd + E * H + k * 3 * mi * H + 3 * si * H + H
+    return 2.0 * tokens * L * per_token + 2.0 * head_rows * cfg.vocab_size * H
+
+
+def attention_flops(cfg, new, before):
+    """QK^T and PV of `new` tokens that follow `before` cached ones (causal)."""
+    return cfg.num_hidden_layers * 2.0 * 2.0 * cfg.q_dim * (new * before + new * (new + 1) / 2.0)
+
+
+def run_57b(args) -> int:
+    """The two workloads at the Qwen2-57B-A14B shape (see the module's docstring)."""
+    import torch
+    from inferx_amd.config import config_from_dict
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_model
+    from inferx_amd.sampling import SamplingParams
+    from inferx_amd.weights import random_tensors
+
+    layers = args.layers or SHAPE_57B["num_hidden_layers"]
+    raw = dict(SHAPE_57B)
+    raw["num_hidden_layers"] = layers
+    cfg = config_from_dict(raw)
+    rt = Runtime(args.dtype, "cuda:0")
+    elt = 2 if args.dtype == "bfloat16" else 4
+    peak = PEAK_TFLOPS["bf16" if elt == 2 else "fp32"] * 1e12
+    mixed = args.workload == "mixed"
+    context = 8192 if mixed else 32768
+    log(f"drawing random weights on the device ({layers} layers, {args.dtype})")
+    t0 = time.time()
+    model = build_model(cfg.model_spec())
+    weights = {k: rt.place(v) for k, v in random_tensors(model, seed=0, dtype=args.dtype, device="cuda:0").items()}
+    gen = torch.Generator().manual_seed(1234)
+    rnd = lambda n: torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
+    base = {"metric": None, "value": None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+            "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if elt == 2 else "fp32", "data": "synthetic: seeded random weights and token ids"}
+    sizes = {"layers": layers, "layers_of_shape": SHAPE_57B["num_hidden_layers"], "hidden": cfg.hidden_size,
+             "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+             "experts": cfg.num_experts, "top_k": cfg.num_experts_per_tok, "moe_intermediate": cfg.moe_intermediate_size,
+             "shared_intermediate": cfg.shared_expert_intermediate_size, "vocab": cfg.vocab_size, "page_size": PAGE}
+
+    if mixed:
+        n_dec, dec_ctx, n_pre, portion, pre_ctx = 32, 4096, 2, 512, 2048
+        pages = (n_dec * context + n_pre * context) // PAGE
+        runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=n_dec + n_pre,
+                             max_seq_len=context, model=model)
+        log(f"model ready in {time.time() - t0:.1f}s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB on the device")
+        dec = [f"d{i}" for i in range(n_dec)]
+        pre = [f"p{i}" for i in range(n_pre)]
+        for r in dec + pre:  # the contexts the step starts from
+            runner.add_request(r)
+            for s in range(0, dec_ctx if r in dec else pre_ctx, 2048):
+                runner.run_entries([(r, rnd(2048), [])])
+        total = args.warmup + args.steps
+        assert pre_ctx + total * portion <= context and dec_ctx + total <= context, "fewer steps: the context is 8,192"
+        entries = lambda: [(r, rnd(1), [0]) for r in dec] + [(r, rnd(portion), []) for r in pre]
+        for _ in range(args.warmup):
+            runner.run_entries(entries())
+        batches = [entries() for _ in range(args.steps)]
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        for e in batches:
+            runner.run_entries(e)
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t) / args.steps
+        tokens = n_dec + n_pre * portion
+        mid = args.warmup + args.steps // 2
+        cache_tokens = n_dec * (dec_ctx + mid) + n_pre * (pre_ctx + mid * portion)
+        flops = linear_flops(cfg, tokens, n_dec) + n_dec * attention_flops(cfg, 1, dec_ctx + mid) \
+            + n_pre * attention_flops(cfg, portion, pre_ctx + mid * portion)
+        gbs = step_bytes(cfg, tokens, cache_tokens, elt) / dt / 1e9
+        line = dict(base, metric="Qwen2-57B-A14B shape, mixed step (32 decodes at context 4096 beside 2 prompt "
+                                 "portions of 512) through the step function, tokens/s",
+                    value=round(tokens / dt, 1), ms_per_step=round(dt * 1e3, 3),
+                    config=dict(sizes, model="Qwen2-57B-A14B shape", global_batch=n_dec + n_pre, seq_len=context,
+                                tokens_per_step=tokens, parallelism="single GPU"),
+                    prefill=None,
+                    compute={"flops_per_step": flops, "frac": round(flops / dt / peak, 5)},
+                    roofline={"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                              "frac": round(gbs / PEAK_HBM_GBS, 5)}, points={})
+        print(json.dumps(line), flush=True)
+        return 0
+
+    # ---- long context: batch 8, prompts of 16,384 to 32,000 tokens in portions of 2,048, then decoding ----
+    batch, chunk = 8, 2048
+    steps = args.steps
+    lens = torch.randint(16384, 32001, (batch,), generator=gen).tolist()
+    free, _ = torch.cuda.mem_get_info()
+    per_page = cfg.num_hidden_layers * 2 * cfg.kv_dim * PAGE * elt
+    pages = max(batch * context // PAGE, int(free * 0.85) // per_page)  # the pool fills what memory is left
+    runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=batch, max_seq_len=context,
+                         model=model)
+    log(f"model ready in {time.time() - t0:.1f}s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB on the device, "
+        f"{pages} pages ({pages * PAGE} tokens of cache)")
+    engine = LLMEngine("", runner=runner, max_num_seqs=batch, max_model_len=context, max_num_batched_tokens=chunk)
+    # (the first requests decode while the later prompts are still being read, about a hundred steps: room for those)
+    slack = 8 * (32000 // chunk + 1) + 8
+    params = SamplingParams(max_tokens=args.warmup + steps + slack, ignore_eos=True)
+    assert max(lens) + args.warmup + steps + slack <= context, "fewer steps: the context is 32,768"
+    ids = [engine.add_request(rnd(n), params) for n in lens]
+    torch.cuda.synchronize()
+    t = time.perf_counter()
+    n_steps = 0
+    while any(engine.scheduler.sequence(i).generated() == 0 for i in ids):
+        engine.step()
+        n_steps += 1
+    torch.cuda.synchronize()
+    t_pre = time.perf_counter() - t
+    log(f"prompts of {lens}: {t_pre:.2f}s in {n_steps} steps")
+    for _ in range(args.warmup):
+        engine.step()
+    torch.cuda.synchronize()
+    before = engine.stats.tokens_out
+    t = time.perf_counter()
+    for _ in range(steps):
+        engine.step()
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t) / steps
+    assert engine.stats.tokens_out - before == batch * steps, "a timed step was not a decode step of the whole batch"
+    pre_flops = linear_flops(cfg, sum(lens), batch) + sum(attention_flops(cfg, n, 0) for n in lens)
+    cache_tokens = sum(lens) + batch * (args.warmup + steps // 2 + batch)
+    gbs = step_bytes(cfg, batch, cache_tokens, elt) / dt / 1e9
+    line = dict(base, metric="Qwen2-57B-A14B shape, decode tok/s @ batch 8 after prompts of 16384-32000 tokens",
+                value=round(batch / dt, 1), ms_per_step=round(dt * 1e3, 3),
+                config=dict(sizes, model="Qwen2-57B-A14B shape", global_batch=batch, seq_len=context,
+                            prompt_tokens=sum(lens), portion=chunk, cache_pages=pages, parallelism="single GPU"),
+                prefill={"value": round(sum(lens) / t_pre, 1), "tokens": sum(lens), "ms": round(t_pre * 1e3, 1),
+                         "frac": round(pre_flops / t_pre / peak, 5)},
+                roofline={"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                          "frac": round(gbs / PEAK_HBM_GBS, 5)}, points={})
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=32)
-    ap.add_argument("--warmup", type=int, default=4)
-    ap.add_argument("--layers", type=int, default=SHAPE["num_hidden_layers"],
+    ap.add_argument("--steps", type=int, default=None, help="timed steps (32; 8 for mixed, 256 for long)")
+    ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (4; 2 for mixed)")
+    ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the configuration has (sizes of a layer are never reduced)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long"],
+                    help="decode: the Qwen1.5-MoE-A2.7B shape (default); mixed, long: the Qwen2-57B-A14B shape")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
@@ -77,6 +244,14 @@ def main() -> int:
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
         return 2
+    if args.steps is None:
+        args.steps = {"decode": 32, "mixed": 8, "long": 256}[args.workload]
+    if args.warmup is None:
+        args.warmup = {"decode": 4, "mixed": 2, "long": 4}[args.workload]
+    if args.workload != "decode":
+        return run_57b(args)
+    if args.layers is None:
+        args.layers = SHAPE["num_hidden_layers"]
 
     import torch
     from inferx_amd.config import config_from_dict

@@ -86,18 +86,33 @@ class PagedAttention(Mixer):
         return rt.linear(out.view(T, self.q_dim), self.w_out)
 
     def attend(self, ctx, q, cache, out) -> None:
-        """bfloat16 with pages and heads in multiples of 16: a matrix-core kernel (the one that shares keys through
-        LDS when the step is mostly prompt portions, the wavefront-level one otherwise); else the plain one."""
+        """bfloat16 with pages and heads in multiples of 16: the matrix-core kernels (the one that shares keys through
+        LDS for the prompt portions of a step, the wavefront-level one for requests that bring few tokens and for
+        steps without portions); else the plain one."""
         page_size = cache.k.shape[2]
         if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0:
-            T, S = ctx.num_tokens, ctx.num_requests
+            T = ctx.num_tokens
             if (self.head_dim <= 128 and page_size & (page_size - 1) == 0 and T >= PREFILL_MIN_TOKENS
-                    and T >= PREFILL_MIN_ROWS * S):
-                tile = PREFILL_TILE
-                tiles, pairs = paired_tiles(ctx, tile, self.window)
-                ops.attention_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, out,
-                                      self.scale, self.window, tile, pairs)
-                return
+                    and T > ctx.num_requests):
+                plan = mixed_step_plan(ctx, self.window, self.num_heads)
+                if plan is not None:
+                    tiles, pairs, short = plan
+                    ops.attention_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions,
+                                          out, self.scale, self.window, PREFILL_TILE, pairs)
+                    if short is not None:
+                        # requests that bring few tokens (decoding ones beside the prompt portions): their rows,
+                        # put side by side, go to the kernel that cuts a request's keys into slices
+                        rows, s_tiles, s_positions, n_splits = short
+                        qs = q.index_select(0, rows)
+                        outs = torch.empty_like(qs)
+                        work = None
+                        if n_splits > 1:
+                            work = ctx.rt.empty((qs.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),),
+                                                torch.float32)
+                        ops.attention_mfma(qs, cache.k, cache.v, ctx.block_tables[cache.group], s_tiles, s_positions,
+                                           outs, n_splits, work, self.scale, self.window, QUERY_TILE)
+                        out.index_copy_(0, rows, outs)
+                    return
             tiles, tile, n_splits = query_tiles(ctx, self.window, self.num_heads, self.head_dim)
             work = None
             if n_splits > 1:
@@ -115,8 +130,8 @@ LARGE_QUERY_TILE = 32    # ... or 32 when the step brings many tokens (keys and 
 LARGE_TILE_TOKENS = 1 << 30  # measured: no faster than tiles of 16 on MI355X, so off
 WAVES_WANTED = 2048      # two wavefronts per SIMD of 256 compute units: measured best at batch 8 (longer slices per wavefront)
 MIN_KEYS_PER_SPLIT = 128
-PREFILL_MIN_TOKENS = 128  # the LDS-sharing kernel: steps of at least this many tokens ...
-PREFILL_MIN_ROWS = 16     # ... and this many per request on average
+PREFILL_MIN_TOKENS = 128  # the LDS-sharing kernel: steps with at least this many tokens ...
+PREFILL_MIN_ROWS = 16     # ... in requests that bring at least this many each; it takes those requests
 PREFILL_TILE = 64         # queries of one request per workgroup of that kernel
 
 
@@ -141,18 +156,24 @@ def plan_tiles(ctx, tile: int):
     return base
 
 
-def paired_tiles(ctx, tile: int, window: int):
-    """The LDS-sharing kernel's plan: tiles (see plan_tiles) and, int32 [2, n_pairs] on the device, which two
-    tiles each workgroup takes.  A tile's work grows with the keys it reads (all up to its last query, or a
-    window of them), so the tile that reads most is paired with the one that reads least, and so on inwards:
-    workgroups then take about equally long.  Pairs are ordered by falling work."""
-    key = ("attention_pairs", tile, window)
-    hit = ctx.memo.get(key)
-    if hit is not None:
-        return hit
-    tiles_dev, n_tiles, _ = plan_tiles(ctx, tile)
-    t = ctx.memo[("attention_tiles_np", tile)].astype(np.int64)
-    b = ctx.host
+def _tiles_of(n: np.ndarray, first_row: np.ndarray, seqs: np.ndarray, tile: int) -> np.ndarray:
+    """Tiles of up to `tile` consecutive rows for the requests `seqs` (n: their new tokens, first_row: where their
+    rows start): int32 [3, tiles] = request, first row, rows."""
+    counts = -(-n // tile)
+    which = np.repeat(np.arange(len(n)), counts)
+    first = np.cumsum(counts) - counts
+    off = (np.arange(int(counts.sum())) - np.repeat(first, counts)) * tile
+    rows = np.minimum(tile, n[which] - off)
+    return np.stack([seqs[which], first_row[which] + off, rows]).astype(np.int32)
+
+
+def _pairs_by_work(t: np.ndarray, b, window: int) -> np.ndarray:
+    """Which two tiles each workgroup of the LDS-sharing kernel takes, int32 [2, n_pairs].  A tile's work grows
+    with the keys it reads (all up to its last query, or a window of them), so the tile that reads most is paired
+    with the one that reads least, and so on inwards: workgroups then take about equally long.  Pairs are ordered
+    by falling work."""
+    t = t.astype(np.int64)
+    n_tiles = t.shape[1]
     new = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
     first_row = t[1] - b.q_start[:-1].astype(np.int64)[t[0]]           # the tile's first query within its portion
     end = b.seq_lens.astype(np.int64)[t[0]] - new[t[0]] + first_row + t[2]  # one past the last key it reads
@@ -163,8 +184,54 @@ def paired_tiles(ctx, tile: int, window: int):
     pairs = np.full((2, half), -1, dtype=np.int32)
     pairs[0] = order[:half]
     pairs[1, :n_tiles - half] = order[::-1][:n_tiles - half]
-    ctx.memo[key] = (tiles_dev, torch.from_numpy(pairs).to(ctx.rt.device))
-    return ctx.memo[key]
+    return pairs
+
+
+def mixed_step_plan(ctx, window: int, heads: int):
+    """The plan of a step with prompt portions in it, or None if the step has too few rows in portions for the
+    LDS-sharing kernel (then the wavefront-level kernel takes all of it).
+
+    Requests that bring at least PREFILL_MIN_ROWS tokens are cut into tiles of PREFILL_TILE queries for the
+    LDS-sharing kernel: (tiles, pairs) on the device, rows as in the step.  The others -- the decoding requests
+    of a mixed step -- would each walk their whole context alone through that kernel's 64-key tiles, with one
+    query of 64 at work and once per query head (measured at 32 decoding requests with 4,096 keys beside two
+    portions of 512, 28 query heads on 4: 487 us per layer).  They go to the wavefront-level kernel instead, which
+    cuts keys into slices: `short` = (their rows in the step, tiles over those rows put side by side, the rows'
+    positions, the number of slices), or None if there are none."""
+    key = ("attention_mixed", window, heads)
+    if key in ctx.memo:
+        return ctx.memo[key]
+    b = ctx.host
+    dev = ctx.rt.device
+    q_start = b.q_start[:-1].astype(np.int64)
+    n = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
+    long = n >= PREFILL_MIN_ROWS
+    plan = None
+    if int(n[long].sum()) >= PREFILL_MIN_TOKENS:
+        seqs = np.flatnonzero(long)
+        t = _tiles_of(n[seqs], q_start[seqs], seqs, PREFILL_TILE)
+        pairs = _pairs_by_work(t, b, window)
+        short = None
+        seqs = np.flatnonzero(~long & (n > 0))
+        if len(seqs):
+            ns = n[seqs]
+            rows = np.concatenate([np.arange(q_start[i], q_start[i] + n[i]) for i in seqs])
+            st = _tiles_of(ns, np.cumsum(ns) - ns, seqs, QUERY_TILE)
+            longest = int(b.seq_lens[seqs].max())
+            rows_dev = torch.from_numpy(rows).to(dev)
+            short = (rows_dev, torch.from_numpy(np.ascontiguousarray(st)).to(dev),
+                     ctx.positions.index_select(0, rows_dev), _n_splits(st.shape[1] * heads, longest, window, QUERY_TILE))
+        plan = (torch.from_numpy(np.ascontiguousarray(t)).to(dev), torch.from_numpy(pairs).to(dev), short)
+    ctx.memo[key] = plan
+    return plan
+
+
+def _n_splits(units: int, longest: int, window: int, tile: int) -> int:
+    """Into how many slices the wavefront-level kernel cuts each tile's keys: enough for WAVES_WANTED wavefronts,
+    no slice shorter than MIN_KEYS_PER_SPLIT, a power of two (few distinct values, few captured graphs)."""
+    span = min(longest, window + tile + 32) if window > 0 else longest
+    n_splits = 1 if units >= 2048 else max(1, min(WAVES_WANTED // max(1, units), -(-span // MIN_KEYS_PER_SPLIT), 64))
+    return 1 << (n_splits.bit_length() - 1)
 
 
 def query_tiles(ctx, window: int, heads: int, head_dim: int = 128):
@@ -176,11 +243,7 @@ def query_tiles(ctx, window: int, heads: int, head_dim: int = 128):
     if hit is not None:
         return hit
     tiles_dev, n_tiles, longest = plan_tiles(ctx, tile)
-    span = min(longest, window + tile + 32) if window > 0 else longest
-    units = n_tiles * heads
-    n_splits = 1 if units >= 2048 else max(1, min(WAVES_WANTED // max(1, units), -(-span // MIN_KEYS_PER_SPLIT), 64))
-    n_splits = 1 << (n_splits.bit_length() - 1)  # a power of two: few distinct values, few captured graphs
-    ctx.memo[key] = (tiles_dev, tile, n_splits)
+    ctx.memo[key] = (tiles_dev, tile, _n_splits(n_tiles * heads, longest, window, tile))
     return ctx.memo[key]
 
 

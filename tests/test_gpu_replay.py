@@ -124,6 +124,39 @@ def test_mixed_with_few_pages(folders, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_decoding_requests_beside_long_portions(folders, name, dtype):
+    """Steps of more than 128 tokens in prompt portions with requests beside them that bring one to three tokens,
+    before, between and after the portions' rows: in bfloat16 the portions' queries and the others' go to
+    different attention kernels within one step."""
+    cfg = tiny.CONFIGS[name]
+    lengths = {"r0": 200, "r1": 60, "r2": 236}
+    prompts = {rid: tiny.random_tokens(n, cfg["vocab_size"], seed=300 + i) for i, (rid, n) in enumerate(lengths.items())}
+    at = {rid: 0 for rid in prompts}
+    plan = [[("r1", 40), ("r2", 30)],
+            [("r1", 1), ("r0", 150), ("r2", 3)],
+            [("r0", 48), ("r1", 1), ("r2", 100)],
+            [("r2", 1), ("r1", 2), ("r0", 2)],
+            [("r1", 16), ("r2", 102)]]
+    steps = []
+    for entries in plan:
+        step = {"entries": [], "end": []}
+        for rid, n in entries:
+            step["entries"].append((rid, prompts[rid][at[rid]:at[rid] + n], list(range(n))))
+            at[rid] += n
+            if at[rid] == lengths[rid]:
+                step["end"].append(rid)
+        steps.append(step)
+    assert at == lengths
+    raw, weights = tiny.read_folder(folders[(name, dtype)])
+    want = ru.expected_logits(raw, weights, prompts)
+    skip = ru.near_ties(raw, weights, prompts) if dtype == "bfloat16" else set()
+    runner = make_runner(folders, name, dtype, num_pages=40)
+    ru.compare(ru.replay(runner, steps), want, tol_of(dtype), f"beside portions {name} {dtype}", skip)
+    assert all(p.used_pages == 0 for p in runner.cache.pools)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("seed", [1, 2, 3, 5, 8, 13, 19, 34])
 def test_random_configurations(tmp_path, seed, dtype):
     """Configurations drawn at random from what the architecture allows (head sizes up to 256 and some that are no
