@@ -19,6 +19,11 @@
 //
 // With more than one split, each wavefront writes (max, sum, unnormalised O)
 // and `attn_combine_kernel` merges them.
+//
+// GQ (grouped queries, for tiles of ONE token): the sixteen columns of a tile are
+// the query heads that share a key/value head instead of consecutive tokens of
+// one head, and a wavefront serves a (token, key/value head) pair.  Keys and
+// values are then read once per key/value head, not once per query head.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -29,7 +34,7 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 // head_dim = 16 * NB; a tile holds up to 16 * QT queries; PF: request the next iteration's keys and values
 // before this iteration's are multiplied (pays when few wavefronts are resident: decoding)
-template <int NB, int QT, bool PF>
+template <int NB, int QT, bool PF, bool GQ = false>
 __global__ void __launch_bounds__(256)
 attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cache, const __bf16* __restrict__ v_cache,
                  const int32_t* __restrict__ block_table, const int32_t* __restrict__ tile_seq,
@@ -43,18 +48,20 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
   const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (unit >= n_tiles * n_splits) return;
   const int tile = unit / n_splits, split = unit - tile * n_splits;
-  const int head = blockIdx.y;
-  const int kvh = head / (heads / kv_heads);
+  const int group = heads / kv_heads;
+  // GQ: blockIdx.y is the key/value head, column n of the tile is query head kvh * group + n of token tq0
+  const int kvh = GQ ? blockIdx.y : blockIdx.y / group;
   const int n = lane & 15, g = lane >> 4;
+  const int head = GQ ? kvh * group + min(n, group - 1) : blockIdx.y;
 
   const int tq0 = tile_q0[tile];
-  const int rows = tile_rows[tile];
+  const int rows = GQ ? group : tile_rows[tile];  // columns of the tile that hold a query
   const int pos0 = positions[tq0];
   const int32_t* table = block_table + static_cast<int64_t>(tile_seq[tile]) * max_blocks;
 
   // keys this tile reads at all: [lo, hi); this wavefront's slice [ks, ke)
   const int lo = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;
-  const int hi = pos0 + rows;
+  const int hi = pos0 + (GQ ? 1 : rows);
   const int lo_al = lo & ~(ATTN_KEYS_PER_ITER - 1);
   const int per = (((hi - lo_al + n_splits - 1) / n_splits) + ATTN_KEYS_PER_ITER - 1) & ~(ATTN_KEYS_PER_ITER - 1);
   const int ks = lo_al + split * per;
@@ -69,7 +76,7 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
       const int d0 = 32 * c + 8 * g;
       if (16 * t + n < rows && d0 < D)
         qf[t][c] =
-            *reinterpret_cast<const bf16x8*>(q + (static_cast<int64_t>(tq0 + 16 * t + n) * heads + head) * D + d0);
+            *reinterpret_cast<const bf16x8*>(q + (static_cast<int64_t>(tq0 + (GQ ? 0 : 16 * t + n)) * heads + head) * D + d0);
       else
         for (int j = 0; j < 8; ++j) qf[t][c][j] = (__bf16)0.f;
     }
@@ -166,15 +173,17 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
         for (int c = 0; c < NC; ++c) s[b] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[b][c], qf[t][c], s[b], 0, 0, 0);
       }
       // ---- mask, online softmax for this lane's query over its 8 keys ----
-      const int my_pos = pos0 + 16 * t + n;
+      const int my_pos = pos0 + (GQ ? 0 : 16 * t + n);
       const bool my_row = 16 * t + n < rows;
       const int my_lo = (window > 0 && my_pos + 1 > window) ? my_pos + 1 - window : 0;
       // scores stay unscaled: the scale (times log2 e) enters with the reference point in one fused multiply-add
       float sv[8];
       float mx = -INFINITY;
       // keys that every query of these sixteen sees need no mask (uniform over the wavefront)
-      const bool inner = 16 * t + 16 <= rows && kb + ATTN_KEYS_PER_ITER <= ke && kb + ATTN_KEYS_PER_ITER - 1 <= pos0 + 16 * t &&
-                         (window == 0 || kb > pos0 + 16 * t + 15 - window);
+      // (GQ: the columns without a query head hold zeros for q; what they sum is not stored)
+      const bool inner = (GQ || 16 * t + 16 <= rows) && kb + ATTN_KEYS_PER_ITER <= ke &&
+                         kb + ATTN_KEYS_PER_ITER - 1 <= pos0 + (GQ ? 0 : 16 * t) &&
+                         (window == 0 || kb > pos0 + (GQ ? 0 : 16 * t + 15) - window);
       if (inner) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
@@ -228,7 +237,7 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
     l += __shfl_xor(l, 32, 64);
     if (16 * t + n >= rows) continue;
     // lane holds O^T rows d = 16 b + 4 g + i of column n
-    const int64_t token = tq0 + 16 * t + n;
+    const int64_t token = tq0 + (GQ ? 0 : 16 * t + n);
     if (n_splits == 1) {
       const float inv = 1.0f / l;
       __bf16* dst = out + (token * heads + head) * D + 4 * g;
@@ -286,7 +295,7 @@ attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ 
   }
 }
 
-template <int NB, int QT, bool PF>
+template <int NB, int QT, bool PF, bool GQ = false>
 static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void* k, const void* v,
                         const int32_t* table, const int32_t* tile_seq, const int32_t* tile_q0,
                         const int32_t* tile_rows, const int32_t* positions, void* out, float* part_o, float* part_ml,
@@ -295,18 +304,20 @@ static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void
   int page_shift = -1;  // log2 of the page size if it is a power of two
   for (int b = 4; b < 31; ++b)
     if (page_size == (1 << b)) page_shift = b;
-  hipLaunchKernelGGL((attn_mfma_kernel<NB, QT, PF>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
+  hipLaunchKernelGGL((attn_mfma_kernel<NB, QT, PF, GQ>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, positions, (__bf16*)out, part_o, part_ml,
                      n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window, page_shift);
 }
 
 // Workspace (when n_splits > 1): part_o float32 [tokens * heads * n_splits * head_dim],
 // part_ml float32 [tokens * heads * n_splits * 2].
+// grouped: every tile is ONE token (tile_rows is not read), and a wavefront serves the query heads of one key/value
+// head together (at most 16 of them; tile_queries 16).
 extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void* v_cache, const int32_t* block_table,
                                  const int32_t* tile_seq, const int32_t* tile_q0, const int32_t* tile_rows,
                                  const int32_t* positions, void* out, float* part_o, float* part_ml, int64_t tokens,
                                  int n_tiles, int tile_queries, int n_splits, int heads, int kv_heads, int head_dim,
-                                 int page_size, int max_blocks, float scale, int window, int prefetch,
+                                 int page_size, int max_blocks, float scale, int window, int prefetch, int grouped,
                                  hipStream_t stream) {
   IX_REQUIRE(tile_queries == 16 || tile_queries == 32, "a query tile holds up to 16 or 32 queries");
   IX_REQUIRE(tile_queries == 16 || head_dim <= 128, "tiles of 32 queries need head_dim <= 128");
@@ -318,17 +329,22 @@ extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void*
   IX_REQUIRE(n_splits == 1 || (part_o != nullptr && part_ml != nullptr), "workspace needed for split keys");
   IX_REQUIRE(window >= 0, "window must not be negative");
   IX_REQUIRE(heads <= 65535, "too many heads");
+  IX_REQUIRE(!grouped || (tile_queries == 16 && heads / kv_heads <= 16),
+             "grouped queries: tiles of 16, at most 16 query heads per key/value head");
   if (n_tiles == 0 || tokens == 0) return 0;
   const int64_t units = static_cast<int64_t>(n_tiles) * n_splits;
-  dim3 grid(static_cast<unsigned>((units + 3) / 4), heads);
+  dim3 grid(static_cast<unsigned>((units + 3) / 4), grouped ? kv_heads : heads);
   const float scale_log2 = scale * 1.4426950408889634f;
 #define ARGS                                                                                                    \
   grid, stream, q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, positions, out, part_o, part_ml, \
       n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window
-#define CASE(NB)                                   \
-  case NB:                                         \
-    if (prefetch) launch_attn<NB, 1, true>(ARGS);  \
-    else launch_attn<NB, 1, false>(ARGS);          \
+#define CASE(NB)                                                    \
+  case NB:                                                          \
+    if (grouped) {                                                  \
+      if (prefetch) launch_attn<NB, 1, true, true>(ARGS);           \
+      else launch_attn<NB, 1, false, true>(ARGS);                   \
+    } else if (prefetch) launch_attn<NB, 1, true>(ARGS);            \
+    else launch_attn<NB, 1, false>(ARGS);                           \
     break;
 #define CASE4(NB)                        \
   case NB:                               \

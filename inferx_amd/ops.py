@@ -215,10 +215,11 @@ def attention_plain(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
 def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                    tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, n_splits: int,
                    workspace: Optional[torch.Tensor], scale: float, window: int, tile_queries: int = 16,
-                   prefetch: bool = False) -> None:
+                   prefetch: bool = False, grouped: bool = False) -> None:
     """Paged attention on the matrix cores (bfloat16).  `tiles` int32 [3, n_tiles]: request, first token row and
     number of rows (<= tile_queries, which is 16 or 32) of each query tile.  `workspace` float32 with T * heads * n_splits * (d + 2) entries
-    when n_splits > 1."""
+    when n_splits > 1.  `grouped`: every tile is ONE token, and the query heads of a key/value head (at most 16)
+    are served together, so that its keys and values are read once for all of them."""
     T, heads, d = q.shape
     _need(q.dtype == torch.bfloat16, "the matrix-core attention kernel is bfloat16 only")
     _need(out.shape == q.shape and out.dtype == q.dtype, "out mismatch")
@@ -230,6 +231,8 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     _is_i32(tiles)
     _need(tiles.dim() == 2 and tiles.shape[0] == 3 and tiles.is_contiguous(), "tiles must be int32 [3, n_tiles]")
     n_tiles = tiles.shape[1]
+    _need(not grouped or (tile_queries == 16 and heads // kv_heads <= 16 and n_tiles <= T),
+          "grouped queries: one token per tile, tiles of 16, at most 16 query heads per key/value head")
     part_o = part_ml = None
     if n_splits > 1:
         need = T * heads * n_splits * (d + 2)
@@ -240,7 +243,8 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     _call("ix_attention_mfma", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
           _ptr(tiles[1]), _ptr(tiles[2]), _ptr(positions), _ptr(out), _ptr(part_o), _ptr(part_ml), _i64(T),
           _i32(n_tiles), _i32(tile_queries), _i32(n_splits), _i32(heads), _i32(kv_heads), _i32(d), _i32(page_size),
-          _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(1 if prefetch else 0), _stream())
+          _i32(block_table.shape[1]), _f32(scale), _i32(window), _i32(1 if prefetch else 0),
+          _i32(1 if grouped else 0), _stream())
 
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,

@@ -94,7 +94,7 @@ class PagedAttention(Mixer):
             T = ctx.num_tokens
             if (self.head_dim <= 128 and page_size & (page_size - 1) == 0 and T >= PREFILL_MIN_TOKENS
                     and T > ctx.num_requests):
-                plan = mixed_step_plan(ctx, self.window, self.num_heads)
+                plan = mixed_step_plan(ctx, self.window, self.num_heads, self.num_kv_heads)
                 if plan is not None:
                     tiles, pairs, short = plan
                     ops.attention_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions,
@@ -102,7 +102,7 @@ class PagedAttention(Mixer):
                     if short is not None:
                         # requests that bring few tokens (decoding ones beside the prompt portions): their rows,
                         # put side by side, go to the kernel that cuts a request's keys into slices
-                        rows, s_tiles, s_positions, n_splits = short
+                        rows, s_tiles, s_positions, n_splits, grouped = short
                         qs = q.index_select(0, rows)
                         outs = torch.empty_like(qs)
                         work = None
@@ -110,16 +110,17 @@ class PagedAttention(Mixer):
                             work = ctx.rt.empty((qs.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),),
                                                 torch.float32)
                         ops.attention_mfma(qs, cache.k, cache.v, ctx.block_tables[cache.group], s_tiles, s_positions,
-                                           outs, n_splits, work, self.scale, self.window, QUERY_TILE)
+                                           outs, n_splits, work, self.scale, self.window, QUERY_TILE, grouped=grouped)
                         out.index_copy_(0, rows, outs)
                     return
-            tiles, tile, n_splits = query_tiles(ctx, self.window, self.num_heads, self.head_dim)
+            tiles, tile, n_splits, grouped = query_tiles(ctx, self.window, self.num_heads, self.head_dim,
+                                                         self.num_kv_heads)
             work = None
             if n_splits > 1:
                 work = ctx.rt.empty((q.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),), torch.float32)
             ops.attention_mfma(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, out,
                                n_splits, work, self.scale, self.window, tile,
-                               prefetch=ctx.num_tokens == ctx.num_requests)
+                               prefetch=ctx.num_tokens == ctx.num_requests, grouped=grouped)
         else:
             ops.attention_plain(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.seq_of_token, ctx.positions,
                                 out, self.scale, self.window)
@@ -187,7 +188,13 @@ def _pairs_by_work(t: np.ndarray, b, window: int) -> np.ndarray:
     return pairs
 
 
-def mixed_step_plan(ctx, window: int, heads: int):
+def serves_group_together(heads: int, kv_heads: int) -> bool:
+    """Whether a one-token tile of the wavefront-level kernel holds the query heads of a key/value head (2 to 16 of
+    them) side by side, so that its keys and values are read once for all of them."""
+    return 2 <= heads // kv_heads <= 16
+
+
+def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
     """The plan of a step with prompt portions in it, or None if the step has too few rows in portions for the
     LDS-sharing kernel (then the wavefront-level kernel takes all of it).
 
@@ -197,8 +204,9 @@ def mixed_step_plan(ctx, window: int, heads: int):
     query of 64 at work and once per query head (measured at 32 decoding requests with 4,096 keys beside two
     portions of 512, 28 query heads on 4: 487 us per layer).  They go to the wavefront-level kernel instead, which
     cuts keys into slices: `short` = (their rows in the step, tiles over those rows put side by side, the rows'
-    positions, the number of slices), or None if there are none."""
-    key = ("attention_mixed", window, heads)
+    positions, the number of slices, whether a tile is one token with its grouped query heads), or None if there
+    are none."""
+    key = ("attention_mixed", window, heads, kv_heads)
     if key in ctx.memo:
         return ctx.memo[key]
     b = ctx.host
@@ -216,11 +224,13 @@ def mixed_step_plan(ctx, window: int, heads: int):
         if len(seqs):
             ns = n[seqs]
             rows = np.concatenate([np.arange(q_start[i], q_start[i] + n[i]) for i in seqs])
-            st = _tiles_of(ns, np.cumsum(ns) - ns, seqs, QUERY_TILE)
+            grouped = serves_group_together(heads, kv_heads)
+            st = _tiles_of(ns, np.cumsum(ns) - ns, seqs, 1 if grouped else QUERY_TILE)
             longest = int(b.seq_lens[seqs].max())
             rows_dev = torch.from_numpy(rows).to(dev)
+            units = st.shape[1] * (kv_heads if grouped else heads)
             short = (rows_dev, torch.from_numpy(np.ascontiguousarray(st)).to(dev),
-                     ctx.positions.index_select(0, rows_dev), _n_splits(st.shape[1] * heads, longest, window, QUERY_TILE))
+                     ctx.positions.index_select(0, rows_dev), _n_splits(units, longest, window, QUERY_TILE), grouped)
         plan = (torch.from_numpy(np.ascontiguousarray(t)).to(dev), torch.from_numpy(pairs).to(dev), short)
     ctx.memo[key] = plan
     return plan
@@ -234,16 +244,20 @@ def _n_splits(units: int, longest: int, window: int, tile: int) -> int:
     return 1 << (n_splits.bit_length() - 1)
 
 
-def query_tiles(ctx, window: int, heads: int, head_dim: int = 128):
-    """The wavefront-level kernel's plan: tiles (see plan_tiles), the tile size (16 or 32) and into how many
-    slices each tile's keys are cut."""
+def query_tiles(ctx, window: int, heads: int, head_dim: int = 128, kv_heads: Optional[int] = None):
+    """The wavefront-level kernel's plan: tiles (see plan_tiles), the tile size (16 or 32), into how many
+    slices each tile's keys are cut, and whether a tile is one token with its grouped query heads (a step in which
+    every request brings one token, and query heads share key/value heads)."""
     tile = LARGE_QUERY_TILE if (ctx.num_tokens >= LARGE_TILE_TOKENS and head_dim <= 128) else QUERY_TILE
-    key = ("attention_tiles", window, heads, tile)
+    kv_heads = kv_heads or heads
+    key = ("attention_tiles", window, heads, kv_heads, tile)
     hit = ctx.memo.get(key)
     if hit is not None:
         return hit
     tiles_dev, n_tiles, longest = plan_tiles(ctx, tile)
-    ctx.memo[key] = (tiles_dev, tile, _n_splits(n_tiles * heads, longest, window, tile))
+    grouped = tile == QUERY_TILE and ctx.num_tokens == ctx.num_requests and serves_group_together(heads, kv_heads)
+    units = n_tiles * (kv_heads if grouped else heads)
+    ctx.memo[key] = (tiles_dev, tile, _n_splits(units, longest, window, tile), grouped)
     return ctx.memo[key]
 
 

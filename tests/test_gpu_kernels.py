@@ -130,6 +130,33 @@ def test_attention_mfma(case, n_splits, tile):
           f"attention_mfma splits={n_splits} tile={tile}")
 
 
+GROUPED_CASES = [
+    # seq_lens, q_lens, heads, kv_heads, d, page, window
+    ([700, 33, 1], [1, 1, 1], 28, 4, 128, 16, 0),         # seven query heads per key/value head
+    ([1000, 999, 64], [1, 3, 2], 32, 2, 80, 64, 100),     # sixteen; window; requests of two and three tokens
+    ([130, 17], [1, 1], 6, 3, 48, 16, 0),                 # two
+    ([257], [1], 8, 2, 256, 32, 40),
+]
+
+
+@pytest.mark.parametrize("prefetch", [False, True])
+@pytest.mark.parametrize("n_splits", [1, 3, 8, 70])
+@pytest.mark.parametrize("case", GROUPED_CASES)
+def test_attention_mfma_grouped_queries(case, n_splits, prefetch):
+    """One token per tile, the query heads of a key/value head side by side in it."""
+    from inferx_amd import ops
+    seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, torch.bfloat16, seed=6)
+    out = torch.full_like(p["q"], float("nan"))
+    T = p["q"].shape[0]
+    work = torch.empty(T * heads * n_splits * (d + 2), dtype=torch.float32, device=DEV) if n_splits > 1 else None
+    scale = d ** -0.5
+    ops.attention_mfma(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for(q_lens, 1), p["positions"], out,
+                       n_splits, work, scale, window, 16, prefetch, grouped=True)
+    close(out, attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window), TOL[torch.bfloat16],
+          f"attention_mfma grouped splits={n_splits}")
+
+
 PREFILL_CASES = ATTN_CASES + [
     ([1500], [1500], 5, 1, 128, 16, 0),                   # many tiles of one request
     ([777, 300], [130, 300], 4, 2, 112, 16, 0),           # a portion that starts off a tile's edge; odd head blocks
