@@ -168,11 +168,11 @@ def _tiles_of(n: np.ndarray, first_row: np.ndarray, seqs: np.ndarray, tile: int)
     return np.stack([seqs[which], first_row[which] + off, rows]).astype(np.int32)
 
 
-def _pairs_by_work(t: np.ndarray, b, window: int) -> np.ndarray:
+def _pairs_by_work(t: np.ndarray, b, window: int, pair: bool) -> np.ndarray:
     """Which two tiles each workgroup of the LDS-sharing kernel takes, int32 [2, n_pairs].  A tile's work grows
     with the keys it reads (all up to its last query, or a window of them), so the tile that reads most is paired
     with the one that reads least, and so on inwards: workgroups then take about equally long.  Pairs are ordered
-    by falling work."""
+    by falling work.  Without `pair` every tile gets a workgroup of its own, the ones that read most first."""
     t = t.astype(np.int64)
     n_tiles = t.shape[1]
     new = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
@@ -182,6 +182,10 @@ def _pairs_by_work(t: np.ndarray, b, window: int) -> np.ndarray:
     work = -(-(end - (start // 64) * 64) // 64)  # rounds of 64 keys
     order = np.argsort(-work, kind="stable")
     half = (n_tiles + 1) // 2
+    if not pair:
+        pairs = np.full((2, n_tiles), -1, dtype=np.int32)
+        pairs[0] = order
+        return pairs
     pairs = np.full((2, half), -1, dtype=np.int32)
     pairs[0] = order[:half]
     pairs[1, :n_tiles - half] = order[::-1][:n_tiles - half]
@@ -218,7 +222,12 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
     if int(n[long].sum()) >= PREFILL_MIN_TOKENS:
         seqs = np.flatnonzero(long)
         t = _tiles_of(n[seqs], q_start[seqs], seqs, PREFILL_TILE)
-        pairs = _pairs_by_work(t, b, window)
+        # Two workgroups fit a compute unit.  Pairs only when that still leaves two per compute unit: with fewer,
+        # a workgroup per tile keeps two wavefronts on a SIMD instead of one (measured: two portions of 512 on 28
+        # heads, 448 tiles, 15.2 against 15.8 ms for a step of 8 layers; 2,048 tokens on 16 heads, 512 tiles, 15.5
+        # against 15.4 ms for 24 layers).
+        cus = torch.cuda.get_device_properties(dev).multi_processor_count
+        pairs = _pairs_by_work(t, b, window, pair=t.shape[1] * heads >= 2 * cus)
         short = None
         seqs = np.flatnonzero(~long & (n > 0))
         if len(seqs):
