@@ -21,6 +21,10 @@
 // (wi, xi) owns 64 of the weight rows (for gate|up: 32 gate rows and their up
 // rows) and every second sixteen of activation rows, so it reads 4 + 5 operand
 // pieces for 20 products.
+//
+// The wide form has eight wavefronts, 4 x 2, and 256 weight rows per workgroup
+// (template parameter NWW = 4): per product it moves less through LDS and L2,
+// and it fills a compute unit's LDS alone.
 #include "common.h"
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -28,11 +32,15 @@ typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define TL_ROWS 160   // the row-tile map is made for tiles of this many rows
-#define TL_WROWS 128
 #define TL_K 64
 #define TL_STRIDE 64  // elements per LDS row: no padding; the eight 16-byte pieces of a row are stored permuted
-#define TL_WTILE (TL_WROWS * TL_STRIDE)
-#define TL_XTILE (TL_ROWS * TL_STRIDE)
+// NWW: wavefronts along the weight rows (2 or 4; two along the activation rows): 64 NWW weight rows and 128 NWW
+// threads per workgroup.  With four, a row tile's activations are read for half as many column blocks.
+#define TL_WROWS(NWW) (64 * (NWW))
+#define TL_THREADS(NWW) (128 * (NWW))
+#define TL_WTILE(NWW) (TL_WROWS(NWW) * TL_STRIDE)
+#define TL_XROWS(NWW) ((NWW) == 2 ? 160 : 192)  // staged in steps of 16 NWW rows
+#define TL_XTILE(NWW) (TL_XROWS(NWW) * TL_STRIDE)
 // piece p of row r lies at piece p ^ ((r >> 1) & 7): the sixteen rows that a quarter of a wavefront reads at one
 // piece index then fall on sixteen different groups of four banks, as do the pieces that sixteen lanes write
 __device__ __forceinline__ int tl_at(int row, int piece) { return row * TL_STRIDE + ((piece ^ ((row >> 1) & 7)) << 3); }
@@ -42,7 +50,7 @@ __device__ __forceinline__ int tl_at(int row, int piece) { return row * TL_STRID
 // past the row's end for the row's start, and zeros are written over it in LDS), the loop is one straight line,
 // so the compiler can count exactly how many loads may stay in flight at each wait.  With branches in the loop
 // it waited for all of them, also those of three stages ahead.
-template <bool GATE_UP, int NP>
+template <bool GATE_UP, int NP, int NWW>
 __device__ __forceinline__ void
 tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ rows, int n_out, int width,
            int e, int row0, int row_end, int tile, int col_block, __bf16* ws, __bf16* xs) {
@@ -50,8 +58,11 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
   // optimiser, which sinks them to their first use and so undoes the prefetch)
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int m = lane & 15, g = lane >> 4;
-  const int wi = wave & 1, xi = wave >> 1;
-  constexpr int COLS = GATE_UP ? 64 : 128;  // output columns of this workgroup
+  const int wi = wave % NWW, xi = wave / NWW;
+  constexpr int THREADS = TL_THREADS(NWW), WROWS = TL_WROWS(NWW), HALF = WROWS / 2;
+  constexpr int STEP = THREADS / 8;                     // rows that the workgroup's threads stage at once
+  constexpr int NPX = (32 * NP + STEP - 1) / STEP;      // pieces of activations per thread and stage
+  constexpr int COLS = GATE_UP ? HALF : WROWS;          // output columns of this workgroup
   const int n0 = col_block * COLS;
 
   // what this thread copies per stage: 4 pieces of 8 weights, NP pieces of 8 activations
@@ -62,27 +73,27 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
   int wsrc[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int c = tid + 256 * i, r = c >> 3;
+    const int c = tid + THREADS * i, r = c >> 3;
     int src_row;
     if (GATE_UP)
-      src_row = (r < 64 ? 0 : n_out) + min(n0 + (r & 63), n_out - 1);
+      src_row = (r < HALF ? 0 : n_out) + min(n0 + (r % HALF), n_out - 1);
     else
       src_row = min(n0 + r, n_out - 1);
     wsrc[i] = src_row * width;
   }
-  int xsrc[NP];
+  int xsrc[NPX];
 #pragma unroll
-  for (int i = 0; i < NP; ++i) {
-    const int r = (tid >> 3) + 32 * i;
+  for (int i = 0; i < NPX; ++i) {
+    const int r = (tid >> 3) + STEP * i;
     const int gr = min(row0 + r, row_end - 1);  // rows past the end repeat the last one; their results are dropped
     xsrc[i] = (rows ? rows[gr] : gr) * width;
   }
-  const int xdst = tl_at(tid >> 3, tid & 7);  // rows 32 further on have the same permutation
+  const int xdst = tl_at(tid >> 3, tid & 7);  // rows STEP further on have the same permutation
 
   // The weights come from memory and are what the kernel waits for: three register sets keep the loads of three
   // stages on their way while one stage is multiplied and the next one lies in the other LDS buffer.  The
   // activations, which mostly come from L2, are in two sets.
-  bf16x8 wreg[3][4], xreg[2][NP];
+  bf16x8 wreg[3][4], xreg[2][NPX];
   // Row tiles walk the reduction in the same order but start at different stages (and wrap round): were all
   // workgroups at the same offset of their weight rows at the same time, a row length that is a power of two
   // would send their loads to the same few memory channels (measured with few rows per expert: 4.0 instead of
@@ -109,17 +120,19 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
 #pragma unroll
     for (int i = 0; i < 4; ++i) wr[i] = *reinterpret_cast<const bf16x8*>(w_expert + wsrc[i] + k);
   };
-  auto fetch_x = [&](int k0, bf16x8 (&xr)[NP]) {
+  auto fetch_x = [&](int k0, bf16x8 (&xr)[NPX]) {
     bool ok;
     const int k = place(k0, ok);
 #pragma unroll
-    for (int i = 0; i < NP; ++i) xr[i] = *reinterpret_cast<const bf16x8*>(a + xsrc[i] + k);
+    for (int i = 0; i < NPX; ++i) xr[i] = *reinterpret_cast<const bf16x8*>(a + xsrc[i] + k);
   };
-  auto stage = [&](int k0, int buf, const bf16x8 (&wr)[4], const bf16x8 (&xr)[NP]) {
+  auto stage = [&](int k0, int buf, const bf16x8 (&wr)[4], const bf16x8 (&xr)[NPX]) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + buf * TL_WTILE + xdst + 32 * i * TL_STRIDE) = wr[i];
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<bf16x8*>(ws + buf * TL_WTILE(NWW) + xdst + STEP * i * TL_STRIDE) = wr[i];
 #pragma unroll
-    for (int i = 0; i < NP; ++i) *reinterpret_cast<bf16x8*>(xs + buf * TL_XTILE + xdst + 32 * i * TL_STRIDE) = xr[i];
+    for (int i = 0; i < NPX; ++i)
+      *reinterpret_cast<bf16x8*>(xs + buf * TL_XTILE(NWW) + xdst + STEP * i * TL_STRIDE) = xr[i];
     if (ragged) {
       bool ok;
       place(k0, ok);
@@ -127,10 +140,11 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
         const bf16x8 zero = {(__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f,
                              (__bf16)0.f, (__bf16)0.f, (__bf16)0.f, (__bf16)0.f};
 #pragma unroll
-        for (int i = 0; i < 4; ++i) *reinterpret_cast<bf16x8*>(ws + buf * TL_WTILE + xdst + 32 * i * TL_STRIDE) = zero;
+        for (int i = 0; i < 4; ++i)
+          *reinterpret_cast<bf16x8*>(ws + buf * TL_WTILE(NWW) + xdst + STEP * i * TL_STRIDE) = zero;
 #pragma unroll
-        for (int i = 0; i < NP; ++i)
-          *reinterpret_cast<bf16x8*>(xs + buf * TL_XTILE + xdst + 32 * i * TL_STRIDE) = zero;
+        for (int i = 0; i < NPX; ++i)
+          *reinterpret_cast<bf16x8*>(xs + buf * TL_XTILE(NWW) + xdst + STEP * i * TL_STRIDE) = zero;
       }
     }
   };
@@ -150,14 +164,14 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
     xat[kk] = tl_at(16 * xi + m, 4 * kk + g);
   }
   auto multiply = [&](int buf) {
-    const __bf16* wt = ws + buf * TL_WTILE;
-    const __bf16* xt = xs + buf * TL_XTILE;
+    const __bf16* wt = ws + buf * TL_WTILE(NWW);
+    const __bf16* xt = xs + buf * TL_XTILE(NWW);
 #pragma unroll
     for (int kk = 0; kk < 2; ++kk) {
       bf16x8 wa[4];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {  // gate|up: blocks 32 wi + {0, 16} and the same + 64; down: 64 wi + 16 j
-        const int block = GATE_UP ? 16 * (j & 1) + 64 * (j >> 1) : 16 * j;
+        const int block = GATE_UP ? 16 * (j & 1) + HALF * (j >> 1) : 16 * j;
         wa[j] = *reinterpret_cast<const bf16x8*>(wt + wat[kk] + block * TL_STRIDE);
       }
 #pragma unroll
@@ -259,14 +273,14 @@ tiled_body(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restr
   }
 }
 
-template <bool GATE_UP>
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2)))
+template <bool GATE_UP, int NWW>
+__global__ void __launch_bounds__(TL_THREADS(NWW)) __attribute__((amdgpu_waves_per_eu(2, 2)))
 moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const int32_t* __restrict__ offsets,
                          const int32_t* __restrict__ rows,
                          const int32_t* __restrict__ tile_expert, const int32_t* __restrict__ tile_row0,
                          const int32_t* __restrict__ tile_info, int n_out, int width, int n_col_blocks) {
-  __shared__ __attribute__((aligned(16))) __bf16 ws[2 * TL_WTILE];
-  __shared__ __attribute__((aligned(16))) __bf16 xs[2 * TL_XTILE];
+  __shared__ __attribute__((aligned(16))) __bf16 ws[2 * TL_WTILE(NWW)];
+  __shared__ __attribute__((aligned(16))) __bf16 xs[2 * TL_XTILE(NWW)];
   // Workgroups go to the chip's eight dies in turn, by their number.  All column blocks of a row tile read the
   // same activations: they are numbered so that they land on one die and share its L2 (tile t on die t % 8).
   const int slot = blockIdx.x >> 3;
@@ -278,19 +292,19 @@ moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const in
   const int held = min(TL_ROWS, row_end - row0);
   if (held <= 0) return;
   switch ((held + 31) >> 5) {  // pairs of sixteens of rows this tile holds
-    case 1: tiled_body<GATE_UP, 1>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    case 2: tiled_body<GATE_UP, 2>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    case 3: tiled_body<GATE_UP, 3>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    case 4: tiled_body<GATE_UP, 4>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    default: tiled_body<GATE_UP, 5>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 1: tiled_body<GATE_UP, 1, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 2: tiled_body<GATE_UP, 2, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 3: tiled_body<GATE_UP, 3, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 4: tiled_body<GATE_UP, 4, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    default: tiled_body<GATE_UP, 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
   }
 }
 
-// The row-tile map must have been made for tiles of TL_ROWS (160) rows.
+// The row-tile map must have been made for tiles of TL_ROWS (160) rows.  `wide`: see below.
 extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, const int32_t* offsets,
                                     const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
                                     const int32_t* tile_info, int max_tiles, int64_t a_rows, int64_t n_out,
-                                    int64_t width, int gate_up, hipStream_t stream) {
+                                    int64_t width, int gate_up, int wide, hipStream_t stream) {
   IX_REQUIRE(n_out > 0 && width > 0 && max_tiles >= 0, "sizes must be positive");
   IX_REQUIRE(width % 8 == 0, "the reduction width must be a multiple of 8 for the matrix-core kernel");
   IX_REQUIRE(n_out < (1 << 30) && width < (1 << 30), "sizes too large");
@@ -298,18 +312,26 @@ extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, con
              "the activations, and one expert's weights, must hold fewer than 2^31 numbers");
   IX_REQUIRE(max_tiles <= 65535, "too many row tiles for one launch");
   if (max_tiles == 0) return 0;
-  const int cols = gate_up ? 64 : 128;
+  // wide: four wavefronts along the weight rows instead of two (256 weight rows per workgroup, 112 KB of LDS, one
+  // workgroup per compute unit): the activations are staged for half as many column blocks.  Same sums in the
+  // same order either way.
+  const int nww = wide ? 4 : 2;
+  const int cols = gate_up ? 32 * nww : 64 * nww;
   const int n_col_blocks = static_cast<int>((n_out + cols - 1) / cols);
   const int64_t groups = 8 * static_cast<int64_t>(n_col_blocks) * ((max_tiles + 7) / 8);
   IX_REQUIRE(groups < (int64_t(1) << 31), "too many workgroups for one launch");
-  dim3 grid(static_cast<unsigned>(groups)), block(256);
-  if (gate_up)
-    hipLaunchKernelGGL(moe_grouped_tiled_kernel<true>, grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w,
-                       (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width,
-                       n_col_blocks);
-  else
-    hipLaunchKernelGGL(moe_grouped_tiled_kernel<false>, grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w,
-                       (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width,
-                       n_col_blocks);
+  dim3 grid(static_cast<unsigned>(groups)), block(TL_THREADS(nww));
+#define LAUNCH(GU, NWW)                                                                                             \
+  hipLaunchKernelGGL((moe_grouped_tiled_kernel<GU, NWW>), grid, block, 0, stream, (const __bf16*)a, (const __bf16*)w, \
+                     (__bf16*)out, offsets, rows, tile_expert, tile_row0, tile_info, (int)n_out, (int)width,         \
+                     n_col_blocks)
+  if (nww == 4) {
+    if (gate_up) LAUNCH(true, 4);
+    else LAUNCH(false, 4);
+  } else {
+    if (gate_up) LAUNCH(true, 2);
+    else LAUNCH(false, 2);
+  }
+#undef LAUNCH
   return ix_check_launch("ix_moe_grouped_tiled");
 }

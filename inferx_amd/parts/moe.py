@@ -20,6 +20,13 @@ from .dense_mlp import stack_rows
 
 
 SHARED_BESIDE_TOKENS = 256  # from here on the shared expert runs on a second stream beside the routed ones
+# From this width on the LDS-staged expert products run in their wide form (256 weight rows per workgroup) and the
+# shared expert stays on the main stream (a wide workgroup fills a compute unit's LDS, the library's kernels find
+# no place beside it).  Measured, prompt portions at a width of 3,584 (64 experts of 2,560, 8 per token): 14.9 against
+# 15.5 ms for a mixed step of 1,056 tokens and 8 layers, 2.86 against 3.03 s for 193,000 tokens of long prompts; at a
+# width of 2,048 (60 experts of 1,408, 4 per token) the narrow form beside the shared expert is ahead, 15.2 against
+# 16.0 ms for 2,048 tokens and 24 layers.
+WIDE_TILES_WIDTH = 3072
 
 
 class MoeFeedForward(FeedForward):
@@ -36,6 +43,7 @@ class MoeFeedForward(FeedForward):
         self.expert_width, self.shared_width = int(expert_width), int(shared_width)
         self.shared_gated, self.renormalize = bool(shared_gated), bool(renormalize)
         self.routed_scale, self.init_std = float(routed_scale), float(init_std)
+        self.wide_tiles = self.hidden_size >= WIDE_TILES_WIDTH
         self.w_router = self.w13 = self.w2 = None
         self.w_shared_gate_up = self.w_shared_down = self.w_shared_gate = None
 
@@ -107,8 +115,8 @@ class MoeFeedForward(FeedForward):
         act = rt.empty((A, self.expert_width))
         y = rt.empty((A, self.hidden_size))
         if tile_rows == ops.MOE_TILED_ROWS:  # many rows per expert: operands staged through LDS
-            ops.moe_grouped_tiled(x, self.w13, act, offsets, rows, tile_map, True)
-            ops.moe_grouped_tiled(act, self.w2, y, offsets, None, tile_map, False)
+            ops.moe_grouped_tiled(x, self.w13, act, offsets, rows, tile_map, True, self.wide_tiles)
+            ops.moe_grouped_tiled(act, self.w2, y, offsets, None, tile_map, False, self.wide_tiles)
         elif tile_rows:
             # few rows: the weights are the traffic, the reduction is split over a workgroup's four wavefronts
             ops.moe_grouped_mfma(x, self.w13, act, offsets, rows, tile_map, tile_rows, True, 4)
@@ -170,7 +178,7 @@ class MoeFeedForward(FeedForward):
         tile_rows = self._tile_rows(ctx, x)
         one_launch = self._one_launch(ctx, x, tile_rows)
         shared = join = None
-        if (not one_launch and self.shared_width > 0 and tile_rows == ops.MOE_TILED_ROWS
+        if (not one_launch and self.shared_width > 0 and tile_rows == ops.MOE_TILED_ROWS and not self.wide_tiles
                 and x.shape[0] >= SHARED_BESIDE_TOKENS and ctx.rt.can_run_beside()):
             # a prompt portion: the shared expert's library products are bound by the matrix cores, the routed
             # experts' kernels by memory, so the two run beside each other on two streams

@@ -229,9 +229,11 @@ def test_grouped_mfma(T, H, E, k, mi, tile_rows, k_split):
     assert torch.equal(y.view(torch.int16), y2.view(torch.int16))
 
 
+@pytest.mark.parametrize("wide", [False, True])
 @pytest.mark.parametrize("T,H,E,k,mi", GROUPED + [(900, 136, 6, 2, 88), (2048, 512, 12, 4, 352)])
-def test_grouped_tiled(T, H, E, k, mi):
-    """Experts with a handful of rows, with about one tile of them, and with several tiles (the last one partial)."""
+def test_grouped_tiled(T, H, E, k, mi, wide):
+    """Experts with a handful of rows, with about one tile of them, and with several tiles (the last one partial);
+    128 and 256 weight rows per workgroup, which give the same bits."""
     from inferx_amd import ops
     g = torch.Generator().manual_seed(1)
     topk_e = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
@@ -240,9 +242,15 @@ def test_grouped_tiled(T, H, E, k, mi):
     w13 = rnd(E, 2 * mi, H, seed=2, dtype=torch.bfloat16, scale=H ** -0.5)
     w2 = rnd(E, H, mi, seed=3, dtype=torch.bfloat16, scale=mi ** -0.5)
     act = torch.full((T * k, mi), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ops.moe_grouped_tiled(x, w13, act, offsets, rows, tile_map, True)
+    ops.moe_grouped_tiled(x, w13, act, offsets, rows, tile_map, True, wide)
     y = torch.full((T * k, H), float("nan"), dtype=torch.bfloat16, device=DEV)
-    ops.moe_grouped_tiled(act, w2, y, offsets, None, tile_map, False)
+    ops.moe_grouped_tiled(act, w2, y, offsets, None, tile_map, False, wide)
+    if wide:
+        act_n, y_n = torch.empty_like(act), torch.empty_like(y)
+        ops.moe_grouped_tiled(x, w13, act_n, offsets, rows, tile_map, True, False)
+        ops.moe_grouped_tiled(act, w2, y_n, offsets, None, tile_map, False, False)
+        assert torch.equal(act.view(torch.int16), act_n.view(torch.int16))
+        assert torch.equal(y.view(torch.int16), y_n.view(torch.int16))
     if T <= 900:
         assert rel_err(act, grouped_reference(x, w13, offsets.cpu(), rows.cpu(), True)) < 1.5e-2
         assert rel_err(y, grouped_reference(act, w2, offsets.cpu(), None, False)) < 1.5e-2

@@ -168,6 +168,32 @@ def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated, T):
                        again.view(torch.int16 if dtype == "bfloat16" else torch.int32))
 
 
+def test_moe_part_with_wide_expert_tiles():
+    """The expert products' wide form (chosen by the part from a width of 3,072 on; forced here at a small one)
+    gives the bits of the narrow form, with the shared expert on the main stream."""
+    from inferx_amd.config import PartSpec
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_part, resolve_delta
+    from inferx_amd.parts import moe as moe_part
+    rt = Runtime("bfloat16")
+    H, E, k, mi, si, T = 64, 4, 2, 32, 64, 300
+    assert build_part("feed_forward", PartSpec("moe", {"hidden_size": moe_part.WIDE_TILES_WIDTH, "num_experts": 2,
+                                                       "top_k": 1, "expert_width": 8})).wide_tiles
+    part = build_part("feed_forward", PartSpec("moe", {
+        "hidden_size": H, "num_experts": E, "top_k": k, "expert_width": mi, "shared_width": si, "init_std": 0.15}))
+    assert not part.wide_tiles
+    w = tensors_for(part, rt, seed=8)
+    part.bind({n: v.to(DEV) for n, v in w.items()}, rt)
+    ctx, _ = make_ctx(rt, [T], [T], 16, 32)
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(9)).to(rt.dtype)
+    narrow = resolve_delta(ctx, part.forward(ctx, x.to(DEV)))
+    part.wide_tiles = True
+    wide = resolve_delta(ctx, part.forward(ctx, x.to(DEV)))
+    assert torch.equal(narrow.view(torch.int16), wide.view(torch.int16))
+    wd = {"m." + n: v.double() for n, v in w.items()}
+    assert err(wide, pm.moe_block(x.double(), wd, "m.", E, k, False, si)) < 2e-2
+
+
 def test_shared_expert_beside_the_routed_ones():
     """A prompt portion: the shared expert runs on a second stream beside the routed experts.  The sum is bit for
     bit that of one stream, also when the calls follow one another without a wait (memory of one call is given
