@@ -134,6 +134,7 @@ MIN_KEYS_PER_SPLIT = 128
 PREFILL_MIN_TOKENS = 128  # the LDS-sharing kernel: steps with at least this many tokens ...
 PREFILL_MIN_ROWS = 16     # ... in requests that bring at least this many each; it takes those requests
 PREFILL_TILE = 64         # queries of one request per workgroup of that kernel
+PREFILL_MIN_WORKGROUPS = 120  # ... and at least this many (tile, head) pairs
 
 
 def plan_tiles(ctx, tile: int):
@@ -219,9 +220,12 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
     n = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
     long = n >= PREFILL_MIN_ROWS
     plan = None
-    if int(n[long].sum()) >= PREFILL_MIN_TOKENS:
-        seqs = np.flatnonzero(long)
-        t = _tiles_of(n[seqs], q_start[seqs], seqs, PREFILL_TILE)
+    seqs = np.flatnonzero(long)
+    t = _tiles_of(n[seqs], q_start[seqs], seqs, PREFILL_TILE) if len(seqs) else None
+    # The LDS-sharing kernel walks a tile's keys in one workgroup, so with few tiles it leaves compute units idle
+    # however long the context is (128 queries of 16 heads, 32 workgroups, on 30,000 keys: 624 us; the wavefront-
+    # level kernel, which cuts the keys into slices, 153 us; from about 120 workgroups on it is level or ahead).
+    if t is not None and int(n[long].sum()) >= PREFILL_MIN_TOKENS and t.shape[1] * heads >= PREFILL_MIN_WORKGROUPS:
         # Two workgroups fit a compute unit.  Pairs only when that still leaves two per compute unit: with fewer,
         # a workgroup per tile keeps two wavefronts on a SIMD instead of one (measured: two portions of 512 on 28
         # heads, 448 tiles, 15.2 against 15.8 ms for a step of 8 layers; 2,048 tokens on 16 heads, 512 tiles, 15.5

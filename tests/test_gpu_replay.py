@@ -125,10 +125,15 @@ def test_mixed_with_few_pages(folders, name, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B", "C"])
-def test_decoding_requests_beside_long_portions(folders, name, dtype):
+@pytest.mark.parametrize("min_workgroups", [0, None])
+def test_decoding_requests_beside_long_portions(folders, name, dtype, min_workgroups, monkeypatch):
     """Steps of more than 128 tokens in prompt portions with requests beside them that bring one to three tokens,
     before, between and after the portions' rows: in bfloat16 the portions' queries and the others' go to
-    different attention kernels within one step."""
+    different attention kernels within one step (min_workgroups 0: also with as few query tiles as a tiny model
+    has; None: the rule as it is, which sends such steps to one kernel)."""
+    if min_workgroups is not None:
+        from inferx_amd.parts import attention
+        monkeypatch.setattr(attention, "PREFILL_MIN_WORKGROUPS", min_workgroups)
     cfg = tiny.CONFIGS[name]
     lengths = {"r0": 200, "r1": 60, "r2": 236}
     prompts = {rid: tiny.random_tokens(n, cfg["vocab_size"], seed=300 + i) for i, (rid, n) in enumerate(lengths.items())}
@@ -158,11 +163,15 @@ def test_decoding_requests_beside_long_portions(folders, name, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("seed", [1, 2, 3, 5, 8, 13, 19, 34])
-def test_random_configurations(tmp_path, seed, dtype):
+def test_random_configurations(tmp_path, seed, dtype, monkeypatch):
     """Configurations drawn at random from what the architecture allows (head sizes up to 256 and some that are no
     multiple of 16, odd widths, up to 130 experts, pages of 16 to 64, windows): portions of changing size and
-    mixed steps against the plain implementation."""
+    mixed steps against the plain implementation.  (Odd seeds: prompt portions go to the attention kernel for
+    many query tiles also with the few tiles that a tiny model has.)"""
     from inferx_amd.engine.runner import ModelRunner
+    if seed % 2:
+        from inferx_amd.parts import attention
+        monkeypatch.setattr(attention, "PREFILL_MIN_WORKGROUPS", 0)
     cfg = tiny.random_config(seed)
     page = cfg.pop("_page_size")
     tiny.make_folder(cfg, seed=seed, out_dir=str(tmp_path), dtype=dtype)
