@@ -295,6 +295,13 @@ attn_combine_kernel(const float* __restrict__ part_o, const float* __restrict__ 
   }
 }
 
+int ix_attention_combine(const float* part_o, const float* part_ml, void* out, int64_t tokens, int heads,
+                         int n_splits, int head_dim, hipStream_t stream) {
+  hipLaunchKernelGGL(attn_combine_kernel, dim3(static_cast<unsigned>(tokens * heads)), dim3(128), 0, stream, part_o,
+                     part_ml, (__bf16*)out, n_splits, head_dim);
+  return ix_check_launch("ix_attention_combine");
+}
+
 template <int NB, int QT, bool PF, bool GQ = false>
 static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void* k, const void* v,
                         const int32_t* table, const int32_t* tile_seq, const int32_t* tile_q0,
@@ -364,10 +371,6 @@ extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void*
 #undef CASE4
 #undef ARGS
   if (ix_check_launch("ix_attention_mfma")) return 1;
-  if (n_splits > 1) {
-    hipLaunchKernelGGL(attn_combine_kernel, dim3(static_cast<unsigned>(tokens * heads)), dim3(128), 0, stream, part_o,
-                       part_ml, (__bf16*)out, n_splits, head_dim);
-    return ix_check_launch("ix_attention_combine");
-  }
+  if (n_splits > 1) return ix_attention_combine(part_o, part_ml, out, tokens, heads, n_splits, head_dim, stream);
   return 0;
 }

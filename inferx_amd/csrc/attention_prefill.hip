@@ -31,7 +31,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
                     const int32_t* __restrict__ tile_seq, const int32_t* __restrict__ tile_q0,
                     const int32_t* __restrict__ tile_rows, const int32_t* __restrict__ pair_a,
                     const int32_t* __restrict__ pair_b, const int32_t* __restrict__ positions,
-                    __bf16* __restrict__ out, int heads, int kv_heads, int page_size, int max_blocks, float scale_log2,
+                    __bf16* __restrict__ out, float* __restrict__ part_o, float* __restrict__ part_ml, int n_splits,
+                    int heads, int kv_heads, int page_size, int max_blocks, float scale_log2,
                     int window, int page_shift) {
   constexpr int D = 16 * NB;
   constexpr int NC = (NB + 1) / 2;          // 32-wide chunks of the head dimension
@@ -51,16 +52,27 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
   // reads few, so that workgroups take about equally long whichever compute unit they land on.
 #pragma unroll 1
   for (int which = 0; which < 2; ++which) {
-  const int tile = which ? pair_b[blockIdx.x] : pair_a[blockIdx.x], head = blockIdx.y;
-  if (tile < 0) break;
+  // a unit of work is a tile, or (n_splits > 1) one slice of a tile's keys: unit = tile * n_splits + slice
+  const int unit = which ? pair_b[blockIdx.x] : pair_a[blockIdx.x], head = blockIdx.y;
+  if (unit < 0) break;
+  const int tile = unit / n_splits, split = unit - tile * n_splits;
   const int kvh = head / (heads / kv_heads);
   const int tq0 = tile_q0[tile];
   const int rows = tile_rows[tile];
   const int pos0 = positions[tq0];
   const int32_t* table = block_table + static_cast<int64_t>(tile_seq[tile]) * max_blocks;
   const int lo = (window > 0 && pos0 + 1 > window) ? pos0 + 1 - window : 0;
-  const int hi = pos0 + rows;
-  const int kb0 = lo & ~(PF_KEYS - 1);
+  // this workgroup's keys [kb0, hi): all that the tile reads, or one slice of them.  Slices are whole rounds of 64
+  // keys from the tile's first round on, so a slice ends at a round's edge or where the tile's keys end, and the
+  // masks below need not know of it.  A slice may be empty: then nothing is summed, and (-inf, 0, 0) is written.
+  const int hi_tile = pos0 + rows;
+  int kb0 = lo & ~(PF_KEYS - 1);
+  int hi = hi_tile;
+  if (n_splits > 1) {
+    const int per = (((hi_tile - kb0 + n_splits - 1) / n_splits) + PF_KEYS - 1) & ~(PF_KEYS - 1);
+    kb0 += split * per;
+    hi = min(hi_tile, kb0 + per);
+  }
   const int wq0 = 16 * QT * wave;  // this wavefront's first query within the tile
 
   bf16x8 qf[QT][NC];
@@ -118,7 +130,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
   const int64_t page_elems = static_cast<int64_t>(kv_heads) * page_size * D;
   const __bf16* k_head = k_cache + static_cast<int64_t>(kvh) * page_size * D;
   const __bf16* v_head = v_cache + static_cast<int64_t>(kvh) * page_size * D;
-  const int last_page = (hi - 1) >> page_shift;
+  const int last_page = (hi_tile - 1) >> page_shift;
   // The table entries of a tile's groups are asked for one round before they are used, with vector loads (every
   // lane the same address): a scalar load would share its counter with the LDS reads of the round and be waited
   // for at the first of them.
@@ -164,7 +176,8 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
       if (tid + 256 * i < V_CHUNKS) *reinterpret_cast<bf16x8*>(vs + v_dst[i]) = vreg[i];
   };
 
-  // a tile has at least one query, so kb0 < hi: the first key tile is staged without a condition (the wait for
+  // a tile has at least one query, so kb0 < hi (but for an empty slice, whose staged keys are then not used): the
+  // first key tile is staged without a condition (the wait for
   // it also covers the loads of the queries above, which the loop then need not wait for again)
   ask_pages(kb0);
   locate(kb0);
@@ -287,6 +300,17 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
     l += __shfl_xor(l, 32, 64);
     const int r = wq0 + 16 * t + n;
     if (r >= rows) continue;
+    if (n_splits > 1) {  // this slice's part: reference point, sum and unnormalised output, for attn_combine_kernel
+      const int64_t p = (static_cast<int64_t>(tq0 + r) * heads + head) * n_splits + split;
+      float* dst = part_o + p * D + 4 * g;
+#pragma unroll
+      for (int b = 0; b < NB; ++b) *reinterpret_cast<f32x4*>(dst + 16 * b) = o[t][b];
+      if (g == 0) {
+        part_ml[2 * p] = m[t];
+        part_ml[2 * p + 1] = l;
+      }
+      continue;
+    }
     const float inv = 1.0f / l;
     __bf16* dst = out + (static_cast<int64_t>(tq0 + r) * heads + head) * D + 4 * g;  // rows d = 16 b + 4 g + i
 #pragma unroll
@@ -304,24 +328,28 @@ template <int NB>
 static void launch_prefill(int tile_queries, dim3 grid, hipStream_t stream, const void* q, const void* k,
                            const void* v, const int32_t* table, const int32_t* tile_seq, const int32_t* tile_q0,
                            const int32_t* tile_rows, const int32_t* pair_a, const int32_t* pair_b,
-                           const int32_t* positions, void* out, int heads, int kv_heads,
-                           int page_size, int max_blocks, float scale_log2, int window) {
+                           const int32_t* positions, void* out, float* part_o, float* part_ml, int n_splits,
+                           int heads, int kv_heads, int page_size, int max_blocks, float scale_log2, int window) {
   int page_shift = 4;  // log2 of the page size, a power of two (the entry point has checked)
   while ((1 << page_shift) < page_size) ++page_shift;
   (void)tile_queries;  // 64: the entry point has checked
   hipLaunchKernelGGL((attn_prefill_kernel<NB, 1>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
-                     (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, pair_a, pair_b, positions, (__bf16*)out, heads, kv_heads,
-                     page_size, max_blocks, scale_log2, window, page_shift);
+                     (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, pair_a, pair_b, positions, (__bf16*)out, part_o,
+                     part_ml, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window, page_shift);
 }
 
 // Tiles of up to `tile_queries` (64) consecutive queries of one request; head_dim a multiple of 16 up to 128; pages
 // of a power of two (from 16) of keys.
-// Workgroup p (per head) takes tiles pair_a[p] and then pair_b[p] (or none if that is -1); the caller names every
-// tile exactly once (a tile left out stays unwritten).
+// Workgroup p (per head) takes units pair_a[p] and then pair_b[p] (or none if that is -1); the caller names every
+// unit exactly once (a tile left out stays unwritten).  A unit is a tile, or with n_splits > 1 the slice
+// unit % n_splits of the keys of tile unit / n_splits: then the slices' parts go to part_o float32
+// [tokens * heads * n_splits * head_dim] and part_ml float32 [tokens * heads * n_splits * 2], and a second kernel
+// puts them together for ALL `tokens` rows of `out` (rows of no tile get what their unwritten parts give).
 extern "C" int ix_attention_prefill(const void* q, const void* k_cache, const void* v_cache,
                                     const int32_t* block_table, const int32_t* tile_seq, const int32_t* tile_q0,
                                     const int32_t* tile_rows, const int32_t* pair_a, const int32_t* pair_b,
-                                    int n_pairs, const int32_t* positions, void* out, int n_tiles,
+                                    int n_pairs, const int32_t* positions, void* out, float* part_o,
+                                    float* part_ml, int n_splits, int64_t tokens, int n_tiles,
                                     int tile_queries, int heads, int kv_heads, int head_dim, int page_size,
                                     int max_blocks, float scale, int window, hipStream_t stream) {
   IX_REQUIRE(n_tiles >= 0 && heads > 0 && kv_heads > 0 && max_blocks > 0, "sizes must be positive");
@@ -331,16 +359,21 @@ extern "C" int ix_attention_prefill(const void* q, const void* k_cache, const vo
   IX_REQUIRE(tile_queries == 64, "a query tile holds up to 64 queries");
   IX_REQUIRE(window >= 0, "window must not be negative");
   IX_REQUIRE(heads <= 65535, "too many heads");
-  IX_REQUIRE(n_pairs >= 0 && n_pairs <= n_tiles, "there are at most as many pairs as tiles");
+  IX_REQUIRE(n_splits >= 1 && n_splits <= 256, "n_splits must be between 1 and 256");
+  IX_REQUIRE(n_splits == 1 || (part_o != nullptr && part_ml != nullptr && tokens > 0), "workspace needed for split keys");
+  IX_REQUIRE(n_pairs >= 0 && n_pairs <= static_cast<int64_t>(n_tiles) * n_splits, "there are at most as many pairs as units");
   if (n_tiles == 0 || n_pairs == 0) return 0;
   dim3 grid(n_pairs, heads);
   const float scale_log2 = scale * 1.4426950408889634f;
 #define CASE(NB)                                                                                                   \
   case NB:                                                                                                         \
     launch_prefill<NB>(tile_queries, grid, stream, q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, \
-                       pair_a, pair_b, positions, out, heads, kv_heads, page_size, max_blocks, scale_log2, window);                \
+                       pair_a, pair_b, positions, out, part_o, part_ml, n_splits, heads, kv_heads, page_size, max_blocks,  \
+                       scale_log2, window);                                                                        \
     break;
   switch (head_dim / 16) { CASE(1) CASE(2) CASE(3) CASE(4) CASE(5) CASE(6) CASE(7) CASE(8) }
 #undef CASE
-  return ix_check_launch("ix_attention_prefill");
+  if (ix_check_launch("ix_attention_prefill")) return 1;
+  if (n_splits > 1) return ix_attention_combine(part_o, part_ml, out, tokens, heads, n_splits, head_dim, stream);
+  return 0;
 }

@@ -124,6 +124,9 @@ __device__ __forceinline__ float ix_block_max(float v, float* red) {
 #include <algorithm>
 #include <string>
 void ix_set_error(const std::string& msg);
+// out[t, h, :] from the parts that kernels which cut keys into slices leave (attention_mfma.hip)
+int ix_attention_combine(const float* part_o, const float* part_ml, void* out, int64_t tokens, int heads,
+                         int n_splits, int head_dim, hipStream_t stream);
 int ix_check_launch(const char* what);
 #define IX_REQUIRE(cond, msg)                          \
   do {                                                 \

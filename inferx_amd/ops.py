@@ -249,11 +249,16 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
 
 def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                       tiles: torch.Tensor, positions: torch.Tensor, out: torch.Tensor, scale: float, window: int,
-                      tile_queries: int = 64, pairs: Optional[torch.Tensor] = None) -> None:
+                      tile_queries: int = 64, pairs: Optional[torch.Tensor] = None, n_splits: int = 1,
+                      workspace: Optional[torch.Tensor] = None) -> None:
     """Paged attention for prompt portions (bfloat16, head_dim <= 128): tiles of up to 64 queries of one
     request, keys and values shared through LDS.  `tiles` as for attention_mfma.  `pairs` int32 [2, n]: the two
-    tiles that workgroup i takes one after the other (second -1: none); every tile is to be named exactly once
-    (one left out stays unwritten).  Without `pairs` every tile gets a workgroup of its own."""
+    units that workgroup i takes one after the other (second -1: none); every unit is to be named exactly once
+    (a tile left out stays unwritten).  Without `pairs` every unit gets a workgroup of its own.
+
+    A unit is a tile, or with n_splits > 1 slice `unit % n_splits` of the keys of tile `unit // n_splits`; then
+    `workspace` (float32, T * heads * n_splits * (d + 2) entries) takes the slices' parts, and ALL T rows of `out`
+    are written from it: rows that no tile covers get no meaningful values and are for the caller to fill."""
     T, heads, d = q.shape
     _need(q.dtype == torch.bfloat16, "the matrix-core attention kernel is bfloat16 only")
     _need(out.shape == q.shape and out.dtype == q.dtype, "out mismatch")
@@ -264,17 +269,24 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _is_i32(positions, T)
     _is_i32(tiles)
     _need(tiles.dim() == 2 and tiles.shape[0] == 3 and tiles.is_contiguous(), "tiles must be int32 [3, n_tiles]")
-    n_tiles = tiles.shape[1]
+    n_units = tiles.shape[1] * n_splits
     if pairs is None:
-        pairs = torch.stack([torch.arange(n_tiles, dtype=torch.int32), torch.full((n_tiles,), -1, dtype=torch.int32)])
+        pairs = torch.stack([torch.arange(n_units, dtype=torch.int32), torch.full((n_units,), -1, dtype=torch.int32)])
         pairs = pairs.to(q.device)
     _is_i32(pairs)
     _need(pairs.dim() == 2 and pairs.shape[0] == 2 and pairs.is_contiguous(), "pairs must be int32 [2, n_pairs]")
-    _need(pairs.shape[1] <= n_tiles <= 2 * pairs.shape[1], "pairs must name every tile once")
+    _need(pairs.shape[1] <= n_units <= 2 * pairs.shape[1], "pairs must name every unit once")
     _need(page_size & (page_size - 1) == 0, "this kernel takes pages of a power of two of keys")
+    part_o = part_ml = None
+    if n_splits > 1:
+        need = T * heads * n_splits * (d + 2)
+        _need(workspace is not None and workspace.dtype == torch.float32 and workspace.numel() >= need,
+              f"workspace of {need} float32 needed")
+        part_o = workspace
+        part_ml = workspace[T * heads * n_splits * d:]
     _call("ix_attention_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
           _ptr(tiles[1]), _ptr(tiles[2]), _ptr(pairs[0]), _ptr(pairs[1]), _i32(pairs.shape[1]), _ptr(positions),
-          _ptr(out), _i32(n_tiles), _i32(tile_queries),
+          _ptr(out), _ptr(part_o), _ptr(part_ml), _i32(n_splits), _i64(T), _i32(tiles.shape[1]), _i32(tile_queries),
           _i32(heads), _i32(kv_heads), _i32(d), _i32(page_size), _i32(block_table.shape[1]), _f32(scale),
           _i32(window), _stream())
 

@@ -96,9 +96,12 @@ class PagedAttention(Mixer):
                     and T > ctx.num_requests):
                 plan = mixed_step_plan(ctx, self.window, self.num_heads, self.num_kv_heads)
                 if plan is not None:
-                    tiles, pairs, short = plan
+                    tiles, pairs, short, slices = plan
+                    work = None
+                    if slices > 1:
+                        work = ctx.rt.empty((T * self.num_heads * slices * (self.head_dim + 2),), torch.float32)
                     ops.attention_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions,
-                                          out, self.scale, self.window, PREFILL_TILE, pairs)
+                                          out, self.scale, self.window, PREFILL_TILE, pairs, slices, work)
                     if short is not None:
                         # requests that bring few tokens (decoding ones beside the prompt portions): their rows,
                         # put side by side, go to the kernel that cuts a request's keys into slices
@@ -134,7 +137,9 @@ MIN_KEYS_PER_SPLIT = 128
 PREFILL_MIN_TOKENS = 128  # the LDS-sharing kernel: steps with at least this many tokens ...
 PREFILL_MIN_ROWS = 16     # ... in requests that bring at least this many each; it takes those requests
 PREFILL_TILE = 64         # queries of one request per workgroup of that kernel
-PREFILL_MIN_WORKGROUPS = 120  # ... and at least this many (tile, head) pairs
+PREFILL_MIN_WORKGROUPS = 120  # ... and at least this many (tile, head) pairs,
+PREFILL_SLICED_MIN_ROUNDS = 96  # or a context of this many rounds of 64 keys (then with the keys in slices
+PREFILL_SLICE_ROUNDS = 8        # of at least this many rounds)
 
 
 def plan_tiles(ctx, tile: int):
@@ -169,11 +174,12 @@ def _tiles_of(n: np.ndarray, first_row: np.ndarray, seqs: np.ndarray, tile: int)
     return np.stack([seqs[which], first_row[which] + off, rows]).astype(np.int32)
 
 
-def _pairs_by_work(t: np.ndarray, b, window: int, pair: bool) -> np.ndarray:
+def _pairs_by_work(t: np.ndarray, b, window: int, pair: bool, slices: int = 1) -> np.ndarray:
     """Which two tiles each workgroup of the LDS-sharing kernel takes, int32 [2, n_pairs].  A tile's work grows
     with the keys it reads (all up to its last query, or a window of them), so the tile that reads most is paired
     with the one that reads least, and so on inwards: workgroups then take about equally long.  Pairs are ordered
-    by falling work.  Without `pair` every tile gets a workgroup of its own, the ones that read most first."""
+    by falling work.  Without `pair` every tile gets a workgroup of its own, the ones that read most first; with
+    `slices` > 1 every slice of every tile does (unit = tile * slices + slice)."""
     t = t.astype(np.int64)
     n_tiles = t.shape[1]
     new = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
@@ -183,6 +189,10 @@ def _pairs_by_work(t: np.ndarray, b, window: int, pair: bool) -> np.ndarray:
     work = -(-(end - (start // 64) * 64) // 64)  # rounds of 64 keys
     order = np.argsort(-work, kind="stable")
     half = (n_tiles + 1) // 2
+    if slices > 1:
+        pairs = np.full((2, n_tiles * slices), -1, dtype=np.int32)
+        pairs[0] = (order[:, None] * slices + np.arange(slices)[None, :]).ravel()
+        return pairs
     if not pair:
         pairs = np.full((2, n_tiles), -1, dtype=np.int32)
         pairs[0] = order
@@ -204,7 +214,8 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
     LDS-sharing kernel (then the wavefront-level kernel takes all of it).
 
     Requests that bring at least PREFILL_MIN_ROWS tokens are cut into tiles of PREFILL_TILE queries for the
-    LDS-sharing kernel: (tiles, pairs) on the device, rows as in the step.  The others -- the decoding requests
+    LDS-sharing kernel: (tiles, pairs, ..., slices) on the device, rows as in the step; slices: into how many
+    workgroups each tile's keys are cut.  The others -- the decoding requests
     of a mixed step -- would each walk their whole context alone through that kernel's 64-key tiles, with one
     query of 64 at work and once per query head (measured at 32 decoding requests with 4,096 keys beside two
     portions of 512, 28 query heads on 4: 487 us per layer).  They go to the wavefront-level kernel instead, which
@@ -222,16 +233,28 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
     plan = None
     seqs = np.flatnonzero(long)
     t = _tiles_of(n[seqs], q_start[seqs], seqs, PREFILL_TILE) if len(seqs) else None
-    # The LDS-sharing kernel walks a tile's keys in one workgroup, so with few tiles it leaves compute units idle
-    # however long the context is (128 queries of 16 heads, 32 workgroups, on 30,000 keys: 624 us; the wavefront-
-    # level kernel, which cuts the keys into slices, 153 us; from about 120 workgroups on it is level or ahead).
-    if t is not None and int(n[long].sum()) >= PREFILL_MIN_TOKENS and t.shape[1] * heads >= PREFILL_MIN_WORKGROUPS:
+    # The LDS-sharing kernel walks a tile's keys in one workgroup.  With few tiles that leaves compute units idle
+    # however long the context is (128 queries of 16 heads on 30,000 keys: 638 us in 32 workgroups).  Then, from
+    # about 6,000 keys on, every tile's keys are cut into slices with a workgroup each, about a thousand in all and
+    # none under eight rounds of 64 keys (97 us in the example; the wavefront-level kernel, which also cuts keys
+    # into slices, 152 us).  On shorter contexts the slices' parts cost more than they gain (a floor of about
+    # 45 us), and the wavefront-level kernel takes steps of fewer than PREFILL_MIN_WORKGROUPS (tile, head) pairs
+    # (2,048 keys + 128 queries: 24 against 52 us); from there on the LDS-sharing kernel is level or ahead.
+    cus = torch.cuda.get_device_properties(dev).multi_processor_count
+    slices = 1
+    if t is not None and t.shape[1] * heads < 2 * cus:
+        keys = int(b.seq_lens[seqs].max())
+        rounds = -(-(min(keys, window + PREFILL_TILE) if window > 0 else keys) // 64)
+        if rounds >= PREFILL_SLICED_MIN_ROUNDS:
+            slices = max(1, min(4 * cus // (t.shape[1] * heads), rounds // PREFILL_SLICE_ROUNDS, 64))
+            slices = 1 << (slices.bit_length() - 1)
+    if t is not None and int(n[long].sum()) >= PREFILL_MIN_TOKENS and \
+            (slices > 1 or t.shape[1] * heads >= PREFILL_MIN_WORKGROUPS):
         # Two workgroups fit a compute unit.  Pairs only when that still leaves two per compute unit: with fewer,
         # a workgroup per tile keeps two wavefronts on a SIMD instead of one (measured: two portions of 512 on 28
         # heads, 448 tiles, 15.2 against 15.8 ms for a step of 8 layers; 2,048 tokens on 16 heads, 512 tiles, 15.5
         # against 15.4 ms for 24 layers).
-        cus = torch.cuda.get_device_properties(dev).multi_processor_count
-        pairs = _pairs_by_work(t, b, window, pair=t.shape[1] * heads >= 2 * cus)
+        pairs = _pairs_by_work(t, b, window, pair=t.shape[1] * heads >= 2 * cus, slices=slices)
         short = None
         seqs = np.flatnonzero(~long & (n > 0))
         if len(seqs):
@@ -244,7 +267,8 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
             units = st.shape[1] * (kv_heads if grouped else heads)
             short = (rows_dev, torch.from_numpy(np.ascontiguousarray(st)).to(dev),
                      ctx.positions.index_select(0, rows_dev), _n_splits(units, longest, window, QUERY_TILE), grouped)
-        plan = (torch.from_numpy(np.ascontiguousarray(t)).to(dev), torch.from_numpy(pairs).to(dev), short)
+        plan = (torch.from_numpy(np.ascontiguousarray(t)).to(dev), torch.from_numpy(np.ascontiguousarray(pairs)).to(dev),
+                short, slices)
     ctx.memo[key] = plan
     return plan
 

@@ -187,6 +187,26 @@ def test_attention_prefill(case, paired, tile=64):
           f"attention_prefill tile={tile}")
 
 
+@pytest.mark.parametrize("paired", [False, True])
+@pytest.mark.parametrize("n_splits", [2, 3, 16])
+@pytest.mark.parametrize("case", PREFILL_CASES)
+def test_attention_prefill_with_key_slices(case, n_splits, paired, tile=64):
+    """Every tile's keys cut into slices, a workgroup per slice (or two slices), parts put together afterwards:
+    with more slices than a tile has rounds of keys some are empty."""
+    from inferx_amd import ops
+    seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, torch.bfloat16, seed=7)
+    out = torch.full_like(p["q"], float("nan"))
+    T = p["q"].shape[0]
+    scale = d ** -0.5
+    tiles = tiles_for(q_lens, tile)
+    work = torch.full((T * heads * n_splits * (d + 2),), float("nan"), dtype=torch.float32, device=DEV)
+    ops.attention_prefill(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles, p["positions"], out, scale, window,
+                          tile, outside_in_pairs(tiles.shape[1] * n_splits) if paired else None, n_splits, work)
+    close(out, attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window), TOL[torch.bfloat16],
+          f"attention_prefill slices={n_splits}")
+
+
 def test_attention_prefill_finds_far_keys(tile=64):
     """Each of a few queries of a long portion matches one key far before it: its output must be that key's value
     (a tile staged from the wrong page, a wrong causal bound of a wavefront or a stale LDS buffer would miss)."""

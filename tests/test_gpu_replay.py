@@ -125,14 +125,18 @@ def test_mixed_with_few_pages(folders, name, dtype):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["B", "C"])
-@pytest.mark.parametrize("min_workgroups", [0, None])
+@pytest.mark.parametrize("min_workgroups", [0, None, "slices"])
 def test_decoding_requests_beside_long_portions(folders, name, dtype, min_workgroups, monkeypatch):
     """Steps of more than 128 tokens in prompt portions with requests beside them that bring one to three tokens,
     before, between and after the portions' rows: in bfloat16 the portions' queries and the others' go to
     different attention kernels within one step (min_workgroups 0: also with as few query tiles as a tiny model
-    has; None: the rule as it is, which sends such steps to one kernel)."""
-    if min_workgroups is not None:
-        from inferx_amd.parts import attention
+    has; None: the rule as it is, which sends such steps to one kernel; "slices": the portions' keys are cut into
+    slices of one round, as those of long contexts are)."""
+    from inferx_amd.parts import attention
+    if min_workgroups == "slices":
+        monkeypatch.setattr(attention, "PREFILL_SLICED_MIN_ROUNDS", 2)
+        monkeypatch.setattr(attention, "PREFILL_SLICE_ROUNDS", 1)
+    elif min_workgroups is not None:
         monkeypatch.setattr(attention, "PREFILL_MIN_WORKGROUPS", min_workgroups)
     cfg = tiny.CONFIGS[name]
     lengths = {"r0": 200, "r1": 60, "r2": 236}
