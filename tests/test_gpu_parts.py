@@ -112,6 +112,72 @@ def test_attention_part_whole_and_in_two_steps(dtype, tol, heads, kv, d, window,
     assert err(run([20, 2, 14, 1]), want) < tol
 
 
+@pytest.mark.parametrize("heads,kv,d,window,q_lens,seq_lens,expect", [
+    (16, 16, 128, 0, [128], [7000], "slices"),                  # few tiles on a long context: keys in slices
+    (28, 4, 128, 0, [1, 300, 1, 2], [5000, 6500, 900, 40], "slices, grouped beside"),  # ... beside requests of one
+                                                                # and two tokens, served per key/value head
+    (16, 16, 64, 0, [130, 1], [400, 77], "one kernel"),         # few tiles, short context
+    (16, 16, 64, 0, [2100], [2100], "pairs"),                   # many tiles, in pairs
+    (8, 2, 64, 512, [200, 1, 1], [3000, 2000, 10], "one kernel"),  # a window
+    (28, 4, 128, 0, [1, 1, 1], [3000, 17, 600], "grouped"),     # one token each
+])
+def test_attention_kernels_chosen_by_the_step(heads, kv, d, window, q_lens, seq_lens, expect):
+    """`PagedAttention.attend` on steps of realistic head counts and contexts: whichever kernels the step's plan
+    chooses (portions in tiles, in pairs or with their keys in slices; few-token requests beside them), the result
+    is float64 attention per request."""
+    from inferx_amd.config import PartSpec
+    from inferx_amd.engine.runtime import CacheBinding, Runtime
+    from inferx_amd.parts import build_part
+    rt = Runtime("bfloat16")
+    part = build_part("mixer", PartSpec("attention", {"hidden_size": 64, "num_heads": heads, "num_kv_heads": kv,
+                                                      "head_dim": d, "window": window}))
+    page = 16
+    pages = sum(-(-L // page) for L in seq_lens) + 2
+    ctx, batch = make_ctx(rt, q_lens, seq_lens, page, pages)
+    table = batch.block_tables[0].reshape(len(q_lens), -1)
+    k_cache = torch.zeros(pages, kv, page, d, dtype=torch.bfloat16)
+    v_cache = torch.zeros(pages, kv, d, page, dtype=torch.bfloat16)
+    g = torch.Generator().manual_seed(12)
+    qs, wants = [], []
+    for s, (n, L) in enumerate(zip(q_lens, seq_lens)):
+        k = torch.randn(L, kv, d, generator=g).bfloat16()
+        v = torch.randn(L, kv, d, generator=g).bfloat16()
+        q = torch.randn(n, heads, d, generator=g).bfloat16()
+        for j in range(-(-L // page)):
+            rows = slice(j * page, min(L, (j + 1) * page))
+            m = rows.stop - rows.start
+            k_cache[int(table[s, j]), :, :m, :] = k[rows].transpose(0, 1)
+            v_cache[int(table[s, j]), :, :, :m] = v[rows].permute(1, 2, 0)
+        qs.append(q)
+        wants.append(None)
+        # float64 attention of this request's new rows over all its keys
+        kk, vv = k.double().repeat_interleave(heads // kv, 1), v.double().repeat_interleave(heads // kv, 1)
+        sc = torch.einsum("qhd,khd->hqk", q.double(), kk) * d ** -0.5
+        qpos, kpos = torch.arange(L - n, L)[:, None], torch.arange(L)[None, :]
+        ok = kpos <= qpos
+        if window > 0:
+            ok &= kpos >= qpos + 1 - window
+        wants[-1] = torch.einsum("hqk,khd->qhd", torch.softmax(sc.masked_fill(~ok[None], -float("inf")), -1), vv)
+    q = torch.cat(qs).to(DEV)
+    out = torch.full_like(q, float("nan"))
+    part.attend(ctx, q, CacheBinding(group=0, k=k_cache.to(DEV), v=v_cache.to(DEV)), out)
+    assert err(out, torch.cat(wants)) < 1.5e-2
+    # the plan that attend() followed (memoised in the step's context)
+    from inferx_amd.parts import attention
+    if expect == "grouped":
+        assert attention.query_tiles(ctx, window, heads, d, kv)[3]
+    else:
+        plan = attention.mixed_step_plan(ctx, window, heads, kv)
+        if expect == "one kernel":
+            assert plan is None
+        elif expect == "pairs":
+            assert plan[3] == 1 and plan[2] is None and int(plan[1][1].max()) >= 0
+        elif expect == "slices":
+            assert plan[3] > 1 and plan[2] is None
+        else:
+            assert plan[3] > 1 and plan[2] is not None and plan[2][4]
+
+
 @pytest.mark.parametrize("dtype,tol", PARAMS)
 def test_dense_mlp_part(dtype, tol):
     from inferx_amd.config import PartSpec
