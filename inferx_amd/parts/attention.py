@@ -242,11 +242,14 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
     # (2,048 keys + 128 queries: 24 against 52 us); from there on the LDS-sharing kernel is level or ahead.
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     slices = 1
-    if t is not None and t.shape[1] * heads < 2 * cus:
+    if t is not None and t.shape[1] * heads < 8 * cus:
         keys = int(b.seq_lens[seqs].max())
         rounds = -(-(min(keys, window + PREFILL_TILE) if window > 0 else keys) // 64)
         if rounds >= PREFILL_SLICED_MIN_ROUNDS:
-            slices = max(1, min(4 * cus // (t.shape[1] * heads), rounds // PREFILL_SLICE_ROUNDS, 64))
+            # (with two to eight workgroups per compute unit a few slices still even out what the compute units
+            # get: 2,048 queries of 28 heads on 30,000 keys, 896 workgroups, 1.53 against 1.73 ms in four slices)
+            want = (4 if t.shape[1] * heads < 2 * cus else 16) * cus
+            slices = max(1, min(want // (t.shape[1] * heads), rounds // PREFILL_SLICE_ROUNDS, 64))
             slices = 1 << (slices.bit_length() - 1)
     if t is not None and int(n[long].sum()) >= PREFILL_MIN_TOKENS and \
             (slices > 1 or t.shape[1] * heads >= PREFILL_MIN_WORKGROUPS):
@@ -254,7 +257,7 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
         # a workgroup per tile keeps two wavefronts on a SIMD instead of one (measured: two portions of 512 on 28
         # heads, 448 tiles, 15.2 against 15.8 ms for a step of 8 layers; 2,048 tokens on 16 heads, 512 tiles, 15.5
         # against 15.4 ms for 24 layers).
-        pairs = _pairs_by_work(t, b, window, pair=t.shape[1] * heads >= 2 * cus, slices=slices)
+        pairs = _pairs_by_work(t, b, window, pair=slices == 1 and t.shape[1] * heads >= 2 * cus, slices=slices)
         short = None
         seqs = np.flatnonzero(~long & (n > 0))
         if len(seqs):
