@@ -129,17 +129,22 @@ class PagedAttention(Mixer):
                                 out, self.scale, self.window)
 
 
+# ---- the wavefront-level kernel (ops.attention_mfma)
 QUERY_TILE = 16          # queries of one request per wavefront ...
 LARGE_QUERY_TILE = 32    # ... or 32 when the step brings many tokens (keys and values are then read once per 32)
 LARGE_TILE_TOKENS = 1 << 30  # measured: no faster than tiles of 16 on MI355X, so off
 WAVES_WANTED = 2048      # two wavefronts per SIMD of 256 compute units: measured best at batch 8 (longer slices per wavefront)
 MIN_KEYS_PER_SPLIT = 128
-PREFILL_MIN_TOKENS = 128  # the LDS-sharing kernel: steps with at least this many tokens ...
-PREFILL_MIN_ROWS = 16     # ... in requests that bring at least this many each; it takes those requests
-PREFILL_TILE = 64         # queries of one request per workgroup of that kernel
-PREFILL_MIN_WORKGROUPS = 120  # ... and at least this many (tile, head) pairs,
-PREFILL_SLICED_MIN_ROUNDS = 96  # or a context of this many rounds of 64 keys (then with the keys in slices
-PREFILL_SLICE_ROUNDS = 8        # of at least this many rounds)
+# ---- the LDS-sharing kernel (ops.attention_prefill) takes the requests of a step that bring at least
+# PREFILL_MIN_ROWS tokens each, if they bring PREFILL_MIN_TOKENS together and make enough workgroups: at least
+# PREFILL_MIN_WORKGROUPS (tile, head) pairs, or a context of PREFILL_SLICED_MIN_ROUNDS rounds of 64 keys, which
+# is then cut into slices of at least PREFILL_SLICE_ROUNDS rounds (see mixed_step_plan)
+PREFILL_TILE = 64        # queries of one request per workgroup
+PREFILL_MIN_ROWS = 16
+PREFILL_MIN_TOKENS = 128
+PREFILL_MIN_WORKGROUPS = 120
+PREFILL_SLICED_MIN_ROUNDS = 96
+PREFILL_SLICE_ROUNDS = 8
 
 
 def plan_tiles(ctx, tile: int):
@@ -150,16 +155,10 @@ def plan_tiles(ctx, tile: int):
     if base is None:
         b = ctx.host
         n = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
-        counts = -(-n // tile)
-        seq = np.repeat(np.arange(len(n)), counts)
-        first = np.cumsum(counts) - counts
-        off = (np.arange(int(counts.sum())) - np.repeat(first, counts)) * tile
-        rows = np.minimum(tile, n[seq] - off)
-        tiles_host = np.stack([seq, b.q_start[:-1][seq] + off, rows]).astype(np.int32)
+        tiles_host = _tiles_of(n, b.q_start[:-1].astype(np.int64), np.arange(len(n)), tile)
         tiles_dev = torch.from_numpy(np.ascontiguousarray(tiles_host)).to(ctx.rt.device)
         longest = int(b.seq_lens.max()) if len(b.seq_lens) else 0
         base = ctx.memo[("attention_tiles_host", tile)] = (tiles_dev, tiles_host.shape[1], longest)
-        ctx.memo[("attention_tiles_np", tile)] = tiles_host
     return base
 
 
