@@ -88,42 +88,41 @@ class PagedAttention(Mixer):
     def attend(self, ctx, q, cache, out) -> None:
         """bfloat16 with pages and heads in multiples of 16: the matrix-core kernels (the one that shares keys through
         LDS for the prompt portions of a step, the wavefront-level one for requests that bring few tokens and for
-        steps without portions); else the plain one."""
+        steps of one token per request); else the plain one."""
         page_size = cache.k.shape[2]
         if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0:
             T = ctx.num_tokens
-            if (self.head_dim <= 128 and page_size & (page_size - 1) == 0 and T >= PREFILL_MIN_TOKENS
-                    and T > ctx.num_requests):
-                plan = mixed_step_plan(ctx, self.window, self.num_heads, self.num_kv_heads)
-                if plan is not None:
-                    tiles, pairs, short, slices = plan
+            if T > ctx.num_requests:  # some request brings more than one token: the step's plan says who goes where
+                lds_fits = self.head_dim <= 128 and page_size & (page_size - 1) == 0
+                lds, waves = mixed_step_plan(ctx, self.window, self.num_heads, self.num_kv_heads, lds_fits)
+                table = ctx.block_tables[cache.group]
+                if lds is not None:
+                    tiles, pairs, slices = lds
                     work = None
                     if slices > 1:
                         work = ctx.rt.empty((T * self.num_heads * slices * (self.head_dim + 2),), torch.float32)
-                    ops.attention_prefill(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions,
-                                          out, self.scale, self.window, PREFILL_TILE, pairs, slices, work)
-                    if short is not None:
-                        # requests that bring few tokens (decoding ones beside the prompt portions): their rows,
-                        # put side by side, go to the kernel that cuts a request's keys into slices
-                        rows, s_tiles, s_positions, n_splits, grouped = short
-                        qs = q.index_select(0, rows)
-                        outs = torch.empty_like(qs)
-                        work = None
-                        if n_splits > 1:
-                            work = ctx.rt.empty((qs.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),),
-                                                torch.float32)
-                        ops.attention_mfma(qs, cache.k, cache.v, ctx.block_tables[cache.group], s_tiles, s_positions,
-                                           outs, n_splits, work, self.scale, self.window, QUERY_TILE, grouped=grouped)
+                    ops.attention_prefill(q, cache.k, cache.v, table, tiles, ctx.positions, out, self.scale,
+                                          self.window, PREFILL_TILE, pairs, slices, work)
+                for rows, tiles, positions, n_splits, grouped in waves:
+                    # a launch that serves some of the step's requests gets their rows put side by side
+                    qs = q if rows is None else q.index_select(0, rows)
+                    outs = out if rows is None else torch.empty_like(qs)
+                    work = None
+                    if n_splits > 1:
+                        work = ctx.rt.empty((qs.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),),
+                                            torch.float32)
+                    ops.attention_mfma(qs, cache.k, cache.v, table, tiles, positions, outs, n_splits, work,
+                                       self.scale, self.window, QUERY_TILE, grouped=grouped)
+                    if rows is not None:
                         out.index_copy_(0, rows, outs)
-                    return
+                return
             tiles, tile, n_splits, grouped = query_tiles(ctx, self.window, self.num_heads, self.head_dim,
                                                          self.num_kv_heads)
             work = None
             if n_splits > 1:
                 work = ctx.rt.empty((q.shape[0] * self.num_heads * n_splits * (self.head_dim + 2),), torch.float32)
             ops.attention_mfma(q, cache.k, cache.v, ctx.block_tables[cache.group], tiles, ctx.positions, out,
-                               n_splits, work, self.scale, self.window, tile,
-                               prefetch=ctx.num_tokens == ctx.num_requests, grouped=grouped)
+                               n_splits, work, self.scale, self.window, tile, prefetch=True, grouped=grouped)
         else:
             ops.attention_plain(q, cache.k, cache.v, ctx.block_tables[cache.group], ctx.seq_of_token, ctx.positions,
                                 out, self.scale, self.window)
@@ -208,30 +207,34 @@ def serves_group_together(heads: int, kv_heads: int) -> bool:
     return 2 <= heads // kv_heads <= 16
 
 
-def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
-    """The plan of a step with prompt portions in it, or None if the step has too few rows in portions for the
-    LDS-sharing kernel (then the wavefront-level kernel takes all of it).
+def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int, lds_fits: bool = True):
+    """Who serves which requests of a step in which some request brings more than one token: (lds, waves).
 
-    Requests that bring at least PREFILL_MIN_ROWS tokens are cut into tiles of PREFILL_TILE queries for the
-    LDS-sharing kernel: (tiles, pairs, ..., slices) on the device, rows as in the step; slices: into how many
-    workgroups each tile's keys are cut.  The others -- the decoding requests
-    of a mixed step -- would each walk their whole context alone through that kernel's 64-key tiles, with one
-    query of 64 at work and once per query head (measured at 32 decoding requests with 4,096 keys beside two
-    portions of 512, 28 query heads on 4: 487 us per layer).  They go to the wavefront-level kernel instead, which
-    cuts keys into slices: `short` = (their rows in the step, tiles over those rows put side by side, the rows'
-    positions, the number of slices, whether a tile is one token with its grouped query heads), or None if there
-    are none."""
-    key = ("attention_mixed", window, heads, kv_heads)
+    lds = (tiles, pairs, slices) for the LDS-sharing kernel, rows as in the step, or None.  It takes the requests
+    that bring at least PREFILL_MIN_ROWS tokens, in tiles of PREFILL_TILE queries, if they bring
+    PREFILL_MIN_TOKENS together and make enough workgroups (below); slices: into how many workgroups each tile's
+    keys are cut.
+
+    waves = launches of the wavefront-level kernel for the other requests, each (rows, tiles, positions, slices of
+    the keys, grouped): where query heads share key/value heads, requests that bring fewer tokens than a key/value
+    head has query heads -- the decoding requests of a mixed step -- are served a token per tile with those heads
+    side by side (`grouped`), the rest in tiles of QUERY_TILE queries of one head.  `rows` are the launch's rows in
+    the step, to be put side by side for it, or None if it is the step's only launch and takes all rows as they lie.
+
+    Sent through the LDS-sharing kernel, a decoding request would walk its whole context alone, with one query of
+    a tile's 64 at work and once per query head (measured at 32 decoding requests with 4,096 keys beside two
+    portions of 512, 28 query heads on 4: 487 us per layer; 162 + 57 us in two launches)."""
+    key = ("attention_mixed", window, heads, kv_heads, lds_fits)
     if key in ctx.memo:
         return ctx.memo[key]
     b = ctx.host
     dev = ctx.rt.device
     q_start = b.q_start[:-1].astype(np.int64)
     n = (b.q_start[1:] - b.q_start[:-1]).astype(np.int64)
+    to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     long = n >= PREFILL_MIN_ROWS
-    plan = None
     seqs = np.flatnonzero(long)
-    t = _tiles_of(n[seqs], q_start[seqs], seqs, PREFILL_TILE) if len(seqs) else None
+    t = _tiles_of(n[seqs], q_start[seqs], seqs, PREFILL_TILE) if (lds_fits and len(seqs)) else None
     # The LDS-sharing kernel walks a tile's keys in one workgroup.  With few tiles that leaves compute units idle
     # however long the context is (128 queries of 16 heads on 30,000 keys: 638 us in 32 workgroups).  Then, from
     # about 6,000 keys on, every tile's keys are cut into slices with a workgroup each, about a thousand in all and
@@ -250,6 +253,8 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
             want = (4 if t.shape[1] * heads < 2 * cus else 16) * cus
             slices = max(1, min(want // (t.shape[1] * heads), rounds // PREFILL_SLICE_ROUNDS, 64))
             slices = 1 << (slices.bit_length() - 1)
+    lds = None
+    served = np.zeros(len(n), dtype=bool)
     if t is not None and int(n[long].sum()) >= PREFILL_MIN_TOKENS and \
             (slices > 1 or t.shape[1] * heads >= PREFILL_MIN_WORKGROUPS):
         # Two workgroups fit a compute unit.  Pairs only when that still leaves two per compute unit: with fewer,
@@ -257,22 +262,30 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int):
         # heads, 448 tiles, 15.2 against 15.8 ms for a step of 8 layers; 2,048 tokens on 16 heads, 512 tiles, 15.5
         # against 15.4 ms for 24 layers).
         pairs = _pairs_by_work(t, b, window, pair=slices == 1 and t.shape[1] * heads >= 2 * cus, slices=slices)
-        short = None
-        seqs = np.flatnonzero(~long & (n > 0))
-        if len(seqs):
-            ns = n[seqs]
-            rows = np.concatenate([np.arange(q_start[i], q_start[i] + n[i]) for i in seqs])
-            grouped = serves_group_together(heads, kv_heads)
-            st = _tiles_of(ns, np.cumsum(ns) - ns, seqs, 1 if grouped else QUERY_TILE)
-            longest = int(b.seq_lens[seqs].max())
-            rows_dev = torch.from_numpy(rows).to(dev)
-            units = st.shape[1] * (kv_heads if grouped else heads)
-            short = (rows_dev, torch.from_numpy(np.ascontiguousarray(st)).to(dev),
-                     ctx.positions.index_select(0, rows_dev), _n_splits(units, longest, window, QUERY_TILE), grouped)
-        plan = (torch.from_numpy(np.ascontiguousarray(t)).to(dev), torch.from_numpy(np.ascontiguousarray(pairs)).to(dev),
-                short, slices)
-    ctx.memo[key] = plan
-    return plan
+        lds = (to_dev(t), to_dev(pairs), slices)
+        served = long.copy()
+    group = heads // kv_heads
+    together = serves_group_together(heads, kv_heads)
+    sets = [(~served & (n > 0) & (n < group), True), (~served & (n >= group), False)] if together \
+        else [(~served & (n > 0), False)]
+    sets = [(np.flatnonzero(mask), grouped) for mask, grouped in sets if mask.any()]
+    waves = []
+    for seqs, grouped in sets:
+        ns = n[seqs]
+        alone = lds is None and len(sets) == 1
+        first = q_start[seqs] if alone else np.cumsum(ns) - ns
+        st = _tiles_of(ns, first, seqs, 1 if grouped else QUERY_TILE)
+        rows = positions = None
+        if alone:
+            positions = ctx.positions
+        else:
+            rows = to_dev(np.concatenate([np.arange(q_start[i], q_start[i] + n[i]) for i in seqs]))
+            positions = ctx.positions.index_select(0, rows)
+        units = st.shape[1] * (kv_heads if grouped else heads)
+        waves.append((rows, to_dev(st), positions, _n_splits(units, int(b.seq_lens[seqs].max()), window, QUERY_TILE),
+                      grouped))
+    ctx.memo[key] = (lds, waves)
+    return ctx.memo[key]
 
 
 def _n_splits(units: int, longest: int, window: int, tile: int) -> int:

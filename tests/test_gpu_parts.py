@@ -118,7 +118,8 @@ def test_attention_part_whole_and_in_two_steps(dtype, tol, heads, kv, d, window,
                                                                 # and two tokens, served per key/value head
     (16, 16, 64, 0, [130, 1], [400, 77], "one kernel"),         # few tiles, short context
     (16, 16, 64, 0, [2100], [2100], "pairs"),                   # many tiles, in pairs
-    (8, 2, 64, 512, [200, 1, 1], [3000, 2000, 10], "one kernel"),  # a window
+    (8, 2, 64, 512, [200, 1, 1], [3000, 2000, 10], "two launches"),  # a window; the one-token requests grouped
+    (28, 4, 128, 0, [64, 1, 1, 1], [500, 3000, 200, 10], "two launches"),  # a small step: no LDS-sharing kernel
     (28, 4, 128, 0, [1, 1, 1], [3000, 17, 600], "grouped"),     # one token each
 ])
 def test_attention_kernels_chosen_by_the_step(heads, kv, d, window, q_lens, seq_lens, expect):
@@ -167,15 +168,17 @@ def test_attention_kernels_chosen_by_the_step(heads, kv, d, window, q_lens, seq_
     if expect == "grouped":
         assert attention.query_tiles(ctx, window, heads, d, kv)[3]
     else:
-        plan = attention.mixed_step_plan(ctx, window, heads, kv)
+        lds, waves = attention.mixed_step_plan(ctx, window, heads, kv)
         if expect == "one kernel":
-            assert plan is None
+            assert lds is None and len(waves) == 1 and waves[0][0] is None and not waves[0][4]
+        elif expect == "two launches":
+            assert lds is None and [w[4] for w in waves] == [True, False] and all(w[0] is not None for w in waves)
         elif expect == "pairs":
-            assert plan[3] == 1 and plan[2] is None and int(plan[1][1].max()) >= 0
+            assert lds[2] == 1 and not waves and int(lds[1][1].max()) >= 0
         elif expect == "slices":
-            assert plan[3] > 1 and plan[2] is None
+            assert lds[2] > 1 and not waves
         else:
-            assert plan[3] > 1 and plan[2] is not None and plan[2][4]
+            assert lds[2] > 1 and len(waves) == 1 and waves[0][4]
 
 
 @pytest.mark.parametrize("dtype,tol", PARAMS)
