@@ -161,7 +161,7 @@ def qkv_rope_skinny(x: torch.Tensor, w_qkv: torch.Tensor, bias: Optional[torch.T
                     cos_sin: Optional[torch.Tensor], slots: Optional[torch.Tensor], q_out: torch.Tensor,
                     k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor], heads: int, kv_heads: int,
                     head_dim: int) -> None:
-    """For at most 16 tokens (bfloat16): the q/k/v product, bias, rotation and cache append in one launch."""
+    """For at most 32 tokens (bfloat16): the q/k/v product, bias, rotation and cache append in one launch."""
     T, K = x.shape
     width = (heads + 2 * kv_heads) * head_dim
     _need(x.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and q_out.dtype == torch.bfloat16,

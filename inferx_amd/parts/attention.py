@@ -76,7 +76,7 @@ class PagedAttention(Mixer):
         writes = cache.writes
         epilogue = (self.b_qkv, table, ctx.slots[cache.group] if writes else None, q, cache.k if writes else None,
                     cache.v if writes else None, self.num_heads, self.num_kv_heads, self.head_dim)
-        if (T <= 16 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16 and self.head_dim % 32 == 0
+        if (T <= 32 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16 and self.head_dim % 32 == 0
                 and self.hidden_size % 8 == 0):
             ops.qkv_rope_skinny(x, self.w_qkv, *epilogue)  # few tokens: product and epilogue in one launch
         else:

@@ -175,7 +175,9 @@ def test_qkv_rope_append_many_tokens(dtype, heads, kv, d, page, bias):
 
 @pytest.mark.parametrize("T,H,heads,kv,d,page,bias", [(1, 64, 4, 2, 32, 16, True), (8, 2048, 16, 16, 128, 16, True),
                                                        (16, 96, 3, 1, 32, 32, False), (5, 72, 6, 3, 64, 16, True),
-                                                       (3, 1160, 5, 5, 96, 16, True), (9, 904, 2, 1, 128, 64, False)])
+                                                       (3, 1160, 5, 5, 96, 16, True), (9, 904, 2, 1, 128, 64, False),
+                                                       (17, 96, 3, 1, 32, 16, True), (32, 2048, 16, 16, 128, 16, True),
+                                                       (29, 904, 7, 1, 64, 32, False)])
 def test_qkv_rope_skinny_equals_product_then_epilogue(T, H, heads, kv, d, page, bias):
     """The one-launch q/k/v path for few tokens writes what the product followed by qkv_rope_append writes."""
     from inferx_amd import ops
