@@ -79,6 +79,7 @@ def host_lib():
             "ixh_sched_launched": (ci, [vp]),
             "ixh_sched_resolve": (ci, [vp, i32p, ci]),
             "ixh_sched_is_planned": (ci, [vp]),
+            "ixh_sched_abandon": (None, [vp]),
             "ixh_sched_plan_token_values": (None, [vp, i32p]),
             "ixh_sched_num_completed": (ci, [vp]),
             "ixh_sched_completed": (None, [vp, ci, i64p, i32p, i32p]),

@@ -120,9 +120,17 @@ struct Sched {
       }
       if (!ixh_cache_can_add(cache)) return;
       ixh_cache_add(cache, s.rid);
-      if (ixh_cache_reserve(cache, s.rid, static_cast<int64_t>(s.tokens.size())) != kOk) {
-        ixh_cache_free(cache, s.rid);  // not a preemption site: it waits at the head of the queue
-        return;
+      const int status = ixh_cache_reserve(cache, s.rid, static_cast<int64_t>(s.tokens.size()));
+      if (status != kOk) {
+        ixh_cache_free(cache, s.rid);
+        // Not a preemption site: it waits at the head of the queue for a running sequence to end.  With nothing
+        // running nobody will ever give a page back (and a context that is too long never gets shorter), so it
+        // ends here instead of being planned for ever (reference: tests/unit/scheduler_test.cc:963-984).
+        if (status != kContextFull && !running.empty()) return;
+        std::unique_ptr<Seq> gone = std::move(waiting.front());
+        waiting.pop_front();
+        retire(std::move(gone), status == kContextFull ? kContext : kOutOfMemory);
+        continue;
       }
       running.push_back(std::move(waiting.front()));
       waiting.pop_front();
@@ -387,6 +395,12 @@ int ixh_sched_commit(void* h, const int32_t* sampled, int n) { return S(h)->comm
 int ixh_sched_launched(void* h) { return S(h)->launched(); }
 int ixh_sched_resolve(void* h, const int32_t* sampled, int n) { return S(h)->resolve(sampled, n); }
 int ixh_sched_is_planned(void* h) { return S(h)->planned ? 1 : 0; }
+// The planned step will not run after all (its launch failed): the plan is dropped, the pages it reserved stay
+// with their sequences, and the next prepare plans afresh.
+void ixh_sched_abandon(void* h) {
+  S(h)->planned = false;
+  S(h)->plan.clear();
+}
 // the tokens of the planned step again (flat, as ixh_sched_plan gives them): after resolve they are all known
 void ixh_sched_plan_token_values(void* h, int32_t* tokens) {
   size_t at = 0;

@@ -33,29 +33,35 @@ KV_HEADROOM_BYTES = 1 << 30
 
 def resolve_kv_blocks(block_bytes: int, *, explicit_blocks: Optional[int] = None,
                       kv_cache_memory_bytes: Optional[int] = None, gpu_memory_utilization: float = 0.92,
-                      total_bytes: int = 0, used_bytes: int = 0, min_blocks: int = 1) -> int:
-    """How many pages the pool gets.  An explicit count wins; else explicit bytes;
-    else utilization * total - used - 1 GiB of headroom (reference: ResolveKvBlocks,
-    src/engine/kv_autosize.cc:10-47; vector tests/unit/kv_autosize_test.cc:33-42)."""
-    if block_bytes <= 0:
-        raise ValueError("block_bytes must be positive")
+                      total_bytes: int = 0, used_bytes: int = 0, min_blocks: int = 1,
+                      headroom_bytes: int = KV_HEADROOM_BYTES) -> int:
+    """How many pages the pool gets.  An explicit count wins, unchecked; else explicit bytes; else
+    utilization * total - used - headroom.  Fewer than `min_blocks` (one sequence of the longest length) is an
+    error that says which option to change (reference: ResolveKvBlocks, src/engine/kv_autosize.cc:10-47;
+    vectors tests/unit/kv_autosize_test.cc:14-78)."""
     if explicit_blocks is not None:
         if explicit_blocks <= 0:
             raise ValueError("--num-gpu-blocks-override must be positive")
         return explicit_blocks
+    if block_bytes <= 0:
+        raise ValueError(f"sizing the cache needs a positive page size in bytes, got {block_bytes}")
     if kv_cache_memory_bytes is not None:
         blocks = kv_cache_memory_bytes // block_bytes
-        what = f"--kv-cache-memory-bytes {kv_cache_memory_bytes}"
-    else:
-        if not 0.0 < gpu_memory_utilization <= 1.0:
-            raise ValueError("--gpu-memory-utilization must be within (0, 1]")
-        budget = int(gpu_memory_utilization * total_bytes) - used_bytes - KV_HEADROOM_BYTES
-        blocks = max(0, budget) // block_bytes
-        what = (f"--gpu-memory-utilization {gpu_memory_utilization} of {total_bytes} bytes with {used_bytes} in use "
-                f"and {KV_HEADROOM_BYTES} of headroom")
+        if blocks < min_blocks:
+            raise ValueError(f"--kv-cache-memory-bytes {kv_cache_memory_bytes} holds only {blocks} pages of "
+                             f"{block_bytes} bytes but one sequence of --max-model-len needs {min_blocks}; raise "
+                             "the budget or lower --max-model-len")
+        return blocks
+    if not 0.0 < gpu_memory_utilization <= 1.0:
+        raise ValueError("--gpu-memory-utilization must be within (0, 1]")
+    budget = int(gpu_memory_utilization * total_bytes) - used_bytes - headroom_bytes
+    blocks = max(0, budget) // block_bytes
     if blocks < min_blocks:
-        raise ValueError(f"{what} gives {blocks} cache pages of {block_bytes} bytes; {min_blocks} are needed for one "
-                         "sequence of --max-model-len: lower --max-model-len or give the cache more memory")
+        raise ValueError(f"the cache does not fit: --gpu-memory-utilization {gpu_memory_utilization} of "
+                         f"{total_bytes} bytes leaves {max(budget, 0)} bytes after the {used_bytes} already in use "
+                         f"(weights, activations) and {headroom_bytes} of headroom, which holds {blocks} pages of "
+                         f"{block_bytes} bytes but one sequence of --max-model-len needs {min_blocks}; raise "
+                         "--gpu-memory-utilization or lower --max-model-len")
     return blocks
 
 
@@ -101,6 +107,7 @@ class LLMEngine:
         self._next_id = 0
         self.plan_ahead = True  # plan and lay out the next step while the device runs this one
         self._ahead = None      # (plan, batch) made that way
+        self._failed: Optional[str] = None  # set when a launched step could not be finished
 
     # ---- requests -----------------------------------------------------------
     def add_request(self, prompt_token_ids: Sequence[int], params: Optional[SamplingParams] = None,
@@ -135,19 +142,34 @@ class LLMEngine:
         step in two halves: `launched` and `resolve`); when the sampled tokens arrive they are written into that
         layout, which is then ready to go.  If one of its sequences has just ended the plan is dropped and made
         again at the next call."""
-        if self._ahead is not None:
-            plan, batch = self._ahead
-            self._ahead = None
-        else:
-            plan = self.scheduler.prepare_step()
-            if plan is None:
-                return self.scheduler.take_completed()
-            batch = build_step_batch(self.runner.cache, plan.entries())
-        t0 = time.perf_counter()
-        logits = self.runner.step(batch)
-        rows = [self.scheduler.sequence(c.rid).sampling_row() for c in plan.contributions if c.samples]
-        pending = self.sampler.launch(logits, rows)
+        if self._failed is not None:
+            raise RuntimeError(f"the engine stopped after an error inside a running step: {self._failed}")
+        ahead, self._ahead = self._ahead, None
+        try:
+            if ahead is not None:
+                plan, batch = ahead
+            else:
+                plan = self.scheduler.prepare_step()
+                if plan is None:
+                    return self.scheduler.take_completed()
+                batch = build_step_batch(self.runner.cache, plan.entries())
+            t0 = time.perf_counter()
+            logits = self.runner.step(batch)
+            rows = [self.scheduler.sequence(c.rid).sampling_row() for c in plan.contributions if c.samples]
+            pending = self.sampler.launch(logits, rows)
+        except BaseException:
+            # nothing of this step counts: the plan is dropped (its pages stay reserved for the sequences) and the
+            # next call plans afresh, so a bad request can be cancelled and the others go on
+            self.scheduler.abandon_step()
+            raise
         self.scheduler.launched()
+        try:
+            return self._finish_step(plan, pending, t0)
+        except BaseException as e:
+            self._failed = f"{type(e).__name__}: {e}"
+            raise
+
+    def _finish_step(self, plan, pending, t0) -> List[Completion]:
         nxt = nbatch = None
         if self.plan_ahead:
             nxt = self.scheduler.prepare_step()
@@ -176,10 +198,14 @@ class LLMEngine:
         ids = [self.add_request(p, sp) for p, sp in zip(prompts, params)]
         done: Dict[Hashable, Completion] = {}
         while len(done) < len(ids):
+            before = self.stats.steps
             finished = self.step()
             for c in finished:
                 done[c.rid] = c
-            if not finished and not self.scheduler.has_work():
+            if not finished and self.stats.steps == before:
+                # no step ran and nobody finished: nothing would change by asking again
+                if self.scheduler.has_work():
+                    raise RuntimeError("the scheduler has requests but can neither run nor end any of them")
                 break
         missing = [i for i in ids if i not in done]
         if missing:

@@ -244,6 +244,11 @@ class Scheduler:
         self._plan = plan
         return plan
 
+    def abandon_step(self) -> None:
+        """The planned step will not run (its launch failed): drop the plan; the next `prepare_step` plans afresh."""
+        self._lib.ixh_sched_abandon(self._h)
+        self._plan = None
+
     def commit_step(self, sampled: List[int], logprobs: Optional[List] = None) -> None:
         """`sampled`: one token per contribution that samples, in order; `logprobs`: what the sampler reported
         for those rows (or None).  `launched` and `resolve` in one."""

@@ -153,6 +153,51 @@ def test_lone_sequence_runs_out_of_pages():
     assert cache.pools[0].used_pages == 0
 
 
+def test_prompt_larger_than_the_pool_ends_instead_of_waiting_for_ever():
+    # 2 pages of 4 and a prompt of 20: nothing runs, so nobody will ever give a page back.  The request ends
+    # out_of_memory at once, nothing is held, and the request behind it runs (the reference's "retires rather
+    # than spinning", scheduler_test.cc:963-984, at admission)
+    sched, cache = make(pages=2, page_size=4, max_seq_len=64)
+    sched.add_request("a", list(range(20)), P(4))
+    sched.add_request("b", [1, 2, 3], P(2))
+    plan = sched.prepare_step()
+    early = sched.take_completed()
+    assert [(c.rid, c.reason, c.output_tokens) for c in early] == [("a", FINISH_OOM, [])]
+    assert plan is not None and [e[0] for e in plan.entries()] == ["b"]
+    batch = build_step_batch(cache, plan.entries())
+    sched.commit_step([fake_token(int(batch.positions[r])) for r in batch.logits_rows])
+    done = drain(sched, cache)
+    assert [(c.rid, c.reason, len(c.output_tokens)) for c in done] == [("b", FINISH_LENGTH, 2)]
+    assert cache.pools[0].used_pages == 0 and not sched.has_work()
+    cache.check()
+
+
+def test_large_prompt_behind_a_running_one_waits_then_ends():
+    # while something runs, a prompt that does not fit waits at the head (pages may come back); once the pool is
+    # all free and it still does not fit, it ends
+    sched, cache = make(pages=3, page_size=4, max_seq_len=64)
+    sched.add_request("small", [1, 2], P(3))
+    sched.add_request("big", list(range(16)), P(1))
+    done = drain(sched, cache, max_steps=50)
+    assert [(c.rid, c.reason) for c in done] == [("small", FINISH_LENGTH), ("big", FINISH_OOM)]
+    assert not sched.has_work() and cache.pools[0].used_pages == 0
+
+
+def test_abandoned_step_is_planned_again():
+    # a step whose launch failed is dropped and the same work is planned afresh, nothing lost or counted twice
+    sched, cache = make(budget=4)
+    sched.add_request(1, [1, 2, 3, 4, 5, 6], P(2))
+    first = sched.prepare_step().entries()
+    with pytest.raises(RuntimeError, match="twice"):
+        sched.prepare_step()
+    sched.abandon_step()
+    assert sched.prepare_step().entries() == first
+    sched.abandon_step()
+    done = drain(sched, cache)
+    assert done[0].reason == FINISH_LENGTH and len(done[0].output_tokens) == 2
+    assert cache.pools[0].used_pages == 0
+
+
 def test_prompt_longer_than_the_context_is_refused():
     sched, cache = make(max_seq_len=8)
     sched.add_request(1, list(range(9)), P(1))
