@@ -25,6 +25,9 @@
 // one head, and a wavefront serves a (token, key/value head) pair.  Keys and
 // values are then read once per key/value head, not once per query head.
 #include "common.h"
+#include "inferx_hip.h"
+
+#include <mutex>
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
@@ -373,4 +376,71 @@ extern "C" int ix_attention_mfma(const void* q, const void* k_cache, const void*
   if (ix_check_launch("ix_attention_mfma")) return 1;
   if (n_splits > 1) return ix_attention_combine(part_o, part_ml, out, tokens, heads, n_splits, head_dim, stream);
   return 0;
+}
+
+// ---- the same operation without a workspace argument -----------------------------------------------------------
+// The slices' parts go to an array that is part of the library's image on every device.  In host code the
+// array's name stands for the symbol, not for device memory: its address on the current device is looked up
+// once per device and only that pointer is handed to kernels.
+static __device__ __align__(256) float scratch[IX_ATTENTION_SCRATCH_BYTES / sizeof(float)];
+
+#define IX_MAX_DEVICES 64
+static float* g_scratch_of_device[IX_MAX_DEVICES];  // null until the device's first call
+static std::mutex g_scratch_mutex;
+
+// the current device's copy of `scratch`; 0 on success
+static int scratch_of_current_device(float** ptr) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  if (e != hipSuccess) {
+    ix_set_error(std::string("ix_attention_mfma_noalloc: hipGetDevice: ") + hipGetErrorString(e));
+    return 1;
+  }
+  if (device < 0 || device >= IX_MAX_DEVICES) {
+    ix_set_error("ix_attention_mfma_noalloc: device index " + std::to_string(device) + " is beyond " +
+                 std::to_string(IX_MAX_DEVICES));
+    return 1;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_of_device[device] == nullptr) {
+    float* found = nullptr;
+    e = hipGetSymbolAddress(reinterpret_cast<void**>(&found), HIP_SYMBOL(scratch));
+    if (e != hipSuccess || found == nullptr) {
+      ix_set_error(std::string("ix_attention_mfma_noalloc: hipGetSymbolAddress: ") + hipGetErrorString(e));
+      return 1;
+    }
+    g_scratch_of_device[device] = found;
+  }
+  *ptr = g_scratch_of_device[device];
+  return 0;
+}
+
+extern "C" int ix_attention_mfma_noalloc(const void* q, const void* k_cache, const void* v_cache,
+                                         const int32_t* block_table, const int32_t* tile_seq, const int32_t* tile_q0,
+                                         const int32_t* tile_rows, const int32_t* positions, void* out, int64_t tokens,
+                                         int n_tiles, int tile_queries, int n_splits, int heads, int kv_heads,
+                                         int head_dim, int page_size, int max_blocks, float scale, int window,
+                                         int prefetch, int grouped, hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && heads > 0 && head_dim > 0 && n_splits >= 1 && n_splits <= 256, "sizes must be positive");
+  float* part_o = nullptr;
+  float* part_ml = nullptr;
+  if (n_splits > 1) {
+    const int64_t capacity = IX_ATTENTION_SCRATCH_BYTES / sizeof(float);
+    IX_REQUIRE(tokens <= capacity && heads <= capacity, "sizes beyond the library's buffer");
+    const int64_t parts = tokens * heads * n_splits;  // at most 2^22 * 2^22 * 2^8: no overflow
+    if (parts > capacity || parts * (head_dim + 2) > capacity) {
+      ix_set_error("ix_attention_mfma_noalloc: tokens * heads * n_splits * (head_dim + 2) = " +
+                   std::to_string(parts) + " * " + std::to_string(head_dim + 2) + " floats do not fit the library's " +
+                   std::to_string(IX_ATTENTION_SCRATCH_BYTES) + " bytes: fewer slices or tokens per call, or " +
+                   "ix_attention_mfma with a workspace of the caller's");
+      return 1;
+    }
+    float* base = nullptr;
+    if (scratch_of_current_device(&base)) return 1;
+    part_o = base;
+    part_ml = base + parts * head_dim;
+  }
+  return ix_attention_mfma(q, k_cache, v_cache, block_table, tile_seq, tile_q0, tile_rows, positions, out, part_o,
+                           part_ml, tokens, n_tiles, tile_queries, n_splits, heads, kv_heads, head_dim, page_size,
+                           max_blocks, scale, window, prefetch, grouped, stream);
 }
