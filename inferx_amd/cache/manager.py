@@ -138,9 +138,18 @@ class PagePool:
 
 @dataclass(frozen=True)
 class GroupLayout:
-    """One page group: `window` 0 keeps every token, W > 0 only the last W."""
+    """One page group: `window` 0 keeps every token, W > 0 only the last W.  `release_passed` False keeps the
+    pages that the window has passed until the request ends (what the reference does for its windowed layers,
+    src/model/gpt_oss.cc:259-262); the attention kernels mask by the window either way, so the two settings must
+    give the same logits, which is what the switch is for."""
 
     window: int = 0
+    release_passed: bool = True
+
+    @property
+    def release_window(self) -> int:
+        """The window as the bookkeeping sees it: 0 if no page is ever given back early."""
+        return self.window if self.release_passed else 0
 
 
 class _PoolView:
@@ -188,7 +197,7 @@ class CacheManager:
         self.max_blocks = -(-max_seq_len // page_size)
         self._lib = host_lib()
         G = len(self.groups)
-        windows = (ctypes.c_int32 * max(G, 1))(*[g.window for g in self.groups])
+        windows = (ctypes.c_int32 * max(G, 1))(*[g.release_window for g in self.groups])
         pages = (ctypes.c_int32 * max(G, 1))(*pages_per_group)
         self._h = self._lib.ixh_cache_create(G, windows, pages, page_size, max_requests, max_seq_len)
         if not self._h:

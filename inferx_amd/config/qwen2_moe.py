@@ -4,7 +4,9 @@ Keys, defaults and checks follow the reference's parser and validator
 (`src/model/config.cc:272-520` parse, `:82-240` validate; fixture
 `tests/unit/config_test.cc:152-201`).  Four keys that the reference never
 reads decide which layer is which here: `decoder_sparse_step`,
-`mlp_only_layers`, `use_sliding_window`, `max_window_layers`.
+`mlp_only_layers`, `use_sliding_window`, `max_window_layers`; a fifth,
+`layer_types` (one of "full_attention" / "sliding_attention" per layer), names
+the windowed layers outright where a config.json carries it.
 
 Differences from the reference, on purpose:
   * q/k/v carry a bias unless config.json says otherwise (the reference's default
@@ -19,7 +21,7 @@ from dataclasses import dataclass, field, asdict
 from typing import Any, Dict, List
 
 from .registry import ConfigError, register_architecture
-from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry
+from .spec import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, linear_head, token_embedding
 
 ARCHITECTURE = "Qwen2MoeForCausalLM"
 
@@ -63,6 +65,8 @@ class Qwen2MoeConfig:
     use_sliding_window: bool = False
     sliding_window: int = 0
     max_window_layers: int = 0
+    # per layer "full_attention" or "sliding_attention"; empty: the rule of use_sliding_window / max_window_layers
+    layer_types: List[str] = field(default_factory=list)
     initializer_range: float = 0.02
     torch_dtype: str = "bfloat16"
     hidden_act: str = "silu"
@@ -98,6 +102,9 @@ class Qwen2MoeConfig:
         eos = [] if eos is None else (eos if isinstance(eos, list) else [eos])
         if any(isinstance(x, bool) or not isinstance(x, int) for x in eos):
             raise ConfigError("config.json: eos_token_id must be an integer or a list of integers")
+        layer_types = raw.get("layer_types") or []
+        if not isinstance(layer_types, list) or any(not isinstance(x, str) for x in layer_types):
+            raise ConfigError("config.json: layer_types must be a list of strings")
         bias = raw.get("qkv_bias", raw.get("attention_bias"))
         if bias is None:
             bias = True
@@ -126,6 +133,7 @@ class Qwen2MoeConfig:
             use_sliding_window=_get(raw, "use_sliding_window", bool, False),
             sliding_window=_get(raw, "sliding_window", int, 0),
             max_window_layers=_get(raw, "max_window_layers", int, layers),
+            layer_types=list(layer_types),
             initializer_range=_get(raw, "initializer_range", float, 0.02),
             torch_dtype=_get(raw, "torch_dtype", str, "bfloat16"),
             hidden_act=_get(raw, "hidden_act", str, "silu"),
@@ -137,6 +145,8 @@ class Qwen2MoeConfig:
         eos = d.pop("eos_token_ids")
         if eos:
             d["eos_token_id"] = eos[0] if len(eos) == 1 else eos
+        if not d["layer_types"]:
+            del d["layer_types"]
         d["architectures"] = [ARCHITECTURE]
         d["model_type"] = "qwen2_moe"
         return d
@@ -178,6 +188,14 @@ class Qwen2MoeConfig:
         if self.use_sliding_window:
             need(self.sliding_window > 0, "use_sliding_window is set but sliding_window is not positive")
             need(0 <= self.max_window_layers, "max_window_layers must not be negative")
+        if self.layer_types:
+            need(len(self.layer_types) == self.num_hidden_layers,
+                 f"layer_types names {len(self.layer_types)} layers, the model has {self.num_hidden_layers}")
+            for t in self.layer_types:
+                need(t in ("full_attention", "sliding_attention"),
+                     f"layer_types holds {t!r}: only full_attention and sliding_attention are known")
+            need("sliding_attention" not in self.layer_types or self.sliding_window > 0,
+                 "layer_types names a sliding_attention layer but sliding_window is not positive")
         need(any(self.is_moe_layer(l) for l in range(self.num_hidden_layers)),
              "experts are declared but no layer is sparse (decoder_sparse_step / mlp_only_layers)")
 
@@ -188,7 +206,10 @@ class Qwen2MoeConfig:
         return (layer + 1) % self.decoder_sparse_step == 0
 
     def window_of_layer(self, layer: int) -> int:
-        """0 = every earlier key; W = the last W keys including the query's own."""
+        """0 = every earlier key; W = the last W keys including the query's own.  An explicit `layer_types`
+        decides alone; else layers from `max_window_layers` on are windowed if `use_sliding_window` is set."""
+        if self.layer_types:
+            return self.sliding_window if self.layer_types[layer] == "sliding_attention" else 0
         if self.use_sliding_window and self.sliding_window > 0 and layer >= self.max_window_layers:
             return self.sliding_window
         return 0
@@ -247,8 +268,10 @@ class Qwen2MoeConfig:
                     {"hidden_size": self.hidden_size, "width": self.intermediate_size, "init_std": std},
                     prefix=p + "mlp.",
                 )
-            layers.append(LayerSpec("prenorm", mixer, ffn, norm("input_layernorm"),
-                                    norm("post_attention_layernorm")))
+            layers.append(LayerSpec("prenorm", {"mixer": mixer, "feed_forward": ffn,
+                                                "mixer_norm": norm("input_layernorm"),
+                                                "feed_forward_norm": norm("post_attention_layernorm")}))
+        embed = "model.embed_tokens.weight"
         spec = ModelSpec(
             architecture=ARCHITECTURE,
             hidden_size=self.hidden_size,
@@ -256,11 +279,14 @@ class Qwen2MoeConfig:
             max_positions=self.max_position_embeddings,
             layers=layers,
             schedule=[ScheduleEntry(l) for l in range(self.num_hidden_layers)],
-            embedding_name="model.embed_tokens.weight",
+            embedding=token_embedding(embed, self.vocab_size, self.hidden_size, std),
             final_norm=PartSpec("rmsnorm", {"width": self.hidden_size, "eps": self.rms_norm_eps},
                                 prefix="model.norm."),
-            head_name=None if self.tie_word_embeddings else "lm_head.weight",
+            # a tied head reads the embedding's table (reference: src/model/qwen2.cc:1335-1336)
+            head=linear_head(embed if self.tie_word_embeddings else "lm_head.weight", self.vocab_size,
+                             self.hidden_size, std),
             init_std=std,
+            ignored_tensor_suffixes=("rotary_emb.inv_freq",) + (("lm_head.weight",) if self.tie_word_embeddings else ()),
         )
         spec.validate()
         return spec

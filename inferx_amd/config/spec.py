@@ -14,7 +14,7 @@ config is turned into a list of `LayerSpec`.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional
+from typing import Any, Dict, List, Optional, Tuple
 
 
 @dataclass(frozen=True)
@@ -37,13 +37,13 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """One decoder layer: how its parts are arranged (`block`) and the parts."""
+    """One decoder layer: how its parts are arranged (`block`, a registered arrangement) and the parts themselves
+    under the names that arrangement gives them.  The arrangement says which names it needs and of which kind
+    each is ("prenorm": mixer, feed_forward, mixer_norm, feed_forward_norm); another arrangement may want more
+    norms, fewer, or two mixers, without a change here."""
 
     block: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    mixer_norm: PartSpec
-    feed_forward_norm: PartSpec
+    parts: Dict[str, PartSpec]
 
 
 @dataclass(frozen=True)
@@ -59,16 +59,23 @@ class ScheduleEntry:
 
 @dataclass(frozen=True)
 class ModelSpec:
+    """`embedding` (kind "embedding") turns the step's token ids into the residual stream, `final_norm` (kind
+    "norm") and `head` (kind "head") turn the wanted rows of the stream into logits.  A head that shares the
+    embedding's table names the same checkpoint tensor through its `rename`."""
+
     architecture: str
     hidden_size: int
     vocab_size: int
     max_positions: int
     layers: List[LayerSpec]
     schedule: List[ScheduleEntry]
-    embedding_name: str
+    embedding: PartSpec
     final_norm: PartSpec
-    head_name: Optional[str]  # None: the head is the embedding table (tied)
+    head: PartSpec
     init_std: float = 0.02
+    # endings of tensor names that a checkpoint may hold although no part reads them (tables some writers add, the
+    # head's copy of a tied embedding)
+    ignored_tensor_suffixes: Tuple[str, ...] = ()
 
     def validate(self) -> None:
         if self.hidden_size <= 0 or self.vocab_size <= 0:
@@ -83,3 +90,16 @@ class ModelSpec:
                     raise ValueError(f"schedule[{i}].cache_from={e.cache_from} must name an earlier entry")
                 if self.schedule[e.cache_from].cache_from is not None:
                     raise ValueError(f"schedule[{i}].cache_from names an entry that owns no cache")
+
+
+def token_embedding(name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02,
+                    scale: float = 1.0) -> PartSpec:
+    """The usual embedding: one table `name` of [vocab, hidden]."""
+    return PartSpec("token_embedding", {"vocab_size": vocab_size, "hidden_size": hidden_size, "scale": scale,
+                                        "init_std": init_std}, rename={"weight": name})
+
+
+def linear_head(name: str, vocab_size: int, hidden_size: int, init_std: float = 0.02) -> PartSpec:
+    """The usual head: logits = x . W^T with W = `name` of [vocab, hidden]; a tied head names the embedding's table."""
+    return PartSpec("linear_head", {"vocab_size": vocab_size, "hidden_size": hidden_size, "init_std": init_std},
+                    rename={"weight": name})

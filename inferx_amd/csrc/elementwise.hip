@@ -7,29 +7,30 @@
 #include "common.h"
 
 // ---------------------------------------------------------------------------
-// h[t, :] = table[ids[t], :]        (reference: EmbeddingKernel, layers.cu:465-481;
+// h[t, :] = table[ids[t], :] * scale   (reference: EmbeddingKernel, layers.cu:465-481, which has no scale;
 // an id outside the table gives a zero row here instead of row 0 -- the host
 // rejects such ids before any launch)
 template <typename TW>
 __global__ void embed_kernel(float* __restrict__ h, const TW* __restrict__ table,
-                             const int32_t* __restrict__ ids, int64_t width, int64_t vocab) {
+                             const int32_t* __restrict__ ids, int64_t width, int64_t vocab, float scale) {
   const int64_t t = blockIdx.x;
   const int64_t id = ids[t];
   const bool ok = id >= 0 && id < vocab;
   const TW* row = table + (ok ? id : 0) * width;
-  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) h[t * width + i] = ok ? ix_load(row + i) : 0.f;
+  for (int64_t i = threadIdx.x; i < width; i += blockDim.x) h[t * width + i] = ok ? ix_load(row + i) * scale : 0.f;
 }
 
 extern "C" int ix_embed(void* h, const void* table, int table_dtype, const int32_t* ids, int64_t tokens,
-                        int64_t width, int64_t vocab, hipStream_t stream) {
+                        int64_t width, int64_t vocab, float scale, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && width > 0 && vocab > 0, "sizes must be positive");
   if (tokens == 0) return 0;
   dim3 grid(tokens), block(256);
   if (table_dtype == IX_F32)
-    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (float*)h, (const float*)table, ids, width, vocab);
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (float*)h, (const float*)table, ids, width, vocab,
+                       scale);
   else if (table_dtype == IX_BF16)
     hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (float*)h, (const bf16_t*)table, ids, width,
-                       vocab);
+                       vocab, scale);
   else
     IX_REQUIRE(false, "table dtype must be float32 or bfloat16");
   return ix_check_launch("ix_embed");

@@ -52,6 +52,12 @@ class StepBatch:
     def num_requests(self) -> int:
         return int(self.seq_lens.shape[0])
 
+    @property
+    def one_token_each(self) -> bool:
+        """Every request of the step brings exactly one token (a request may also bring none, so equal counts of
+        tokens and requests do not say so)."""
+        return self.num_tokens == self.num_requests and bool(np.all(self.q_start[1:] - self.q_start[:-1] == 1))
+
     def validate(self, vocab_size: int, pages_per_group: Sequence[int], page_size: int) -> None:
         T, S = self.num_tokens, self.num_requests
         if T and (self.token_ids.min() < 0 or self.token_ids.max() >= vocab_size):

@@ -47,7 +47,7 @@ def _pack(batch: StepBatch, out: Optional[np.ndarray] = None) -> Tuple[List[int]
 class ModelRunner:
     def __init__(self, config, weights: Dict[str, torch.Tensor], rt: Runtime, *, page_size: int = 16,
                  num_pages: int = 256, max_requests: int = 8, max_seq_len: Optional[int] = None, model=None,
-                 use_graphs: bool = True):
+                 use_graphs: bool = True, release_window_pages: bool = True):
         self.config = config
         self.rt = rt
         self.spec = config.model_spec()
@@ -59,6 +59,8 @@ class ModelRunner:
         self.max_seq_len = int(max_seq_len)
         self.max_requests = int(max_requests)
         self.use_graphs = bool(use_graphs) and self.model.graph_safe()
+        # False: windowed groups keep every page until the request ends (for differential tests of the release)
+        self.release_window_pages = bool(release_window_pages)
         self._lay_out_cache(int(num_pages))
 
     @classmethod
@@ -71,46 +73,63 @@ class ModelRunner:
 
     # ---- cache memory ------------------------------------------------------
     def _lay_out_cache(self, num_pages: int) -> None:
+        """Memory for what the parts keep between steps, from their own descriptions: per page group (the owners
+        of equal `CacheNeed`s) and array one tensor [owners, pages, heads, page_size, width] (the last two swapped
+        for a transposed array), per state one tensor [requests, *shape]."""
         plan = self.model.cache_plan()
-        needs: List = []           # distinct CacheNeed, one page group each
-        owners: List[List[int]] = []
-        for i, (need, _state, cache_from) in enumerate(plan):
-            if need is None or cache_from is not None:
-                continue
-            if need not in needs:
-                needs.append(need)
-                owners.append([])
-            owners[needs.index(need)].append(i)
-        self.group_needs = needs
         rt = self.rt
-        self.kv: List[torch.Tensor] = [
-            torch.zeros((len(owners[g]), 2, num_pages, n.kv_heads, self.page_size, n.head_dim), dtype=rt.dtype,
-                        device=rt.device) for g, n in enumerate(needs)]
-        self.bindings: List[CacheBinding] = []
-        for i, (need, state, cache_from) in enumerate(plan):
-            b = CacheBinding()
-            if need is not None:
-                src = i if cache_from is None else cache_from
-                src_need = plan[src][0]
-                if src_need != need:
-                    raise ValueError(f"schedule entry {i} reads the cache of entry {src}, whose layout differs")
-                g = needs.index(need)
-                j = owners[g].index(src)
-                b.group, b.k, b.writes = g, self.kv[g][j, 0], cache_from is None
-                # values are kept transposed within a page: [pages, kv_heads, head_dim, page_size]
-                b.v = self.kv[g][j, 1].view(-1, need.kv_heads, need.head_dim, self.page_size)
-            if state is not None:
-                b.state = torch.zeros((self.max_requests,) + tuple(state.shape), dtype=torch.float32,
-                                      device=rt.device)
-            self.bindings.append(b)
-        self.cache = CacheManager([GroupLayout(n.window) for n in needs], [num_pages] * len(needs), self.page_size,
-                                  self.max_requests, self.max_seq_len)
+        needs: List = []                        # distinct CacheNeed, one page group each
+        owners: List[List[Tuple[int, str]]] = []  # per group the (schedule entry, part name) that own pages in it
+        for i, (keeps, cache_from) in enumerate(plan):
+            if cache_from is not None:
+                continue
+            for name, (need, _state) in keeps.items():
+                if need is None:
+                    continue
+                if need not in needs:
+                    needs.append(need)
+                    owners.append([])
+                owners[needs.index(need)].append((i, name))
+        self.group_needs, self.group_owners = needs, owners
+        dtype_of = lambda name: rt.dtype if name is None else {"float32": torch.float32, "bfloat16": torch.bfloat16}[name]
+        self.pages: List[Dict[str, torch.Tensor]] = []
+        for g, need in enumerate(needs):
+            arrays = {}
+            for a in need.arrays:
+                shape = (a.heads, a.width, self.page_size) if a.transposed else (a.heads, self.page_size, a.width)
+                arrays[a.name] = torch.zeros((len(owners[g]), num_pages) + shape, dtype=dtype_of(a.dtype),
+                                             device=rt.device)
+            self.pages.append(arrays)
+        self.bindings: List[Dict[str, CacheBinding]] = []
+        for i, (keeps, cache_from) in enumerate(plan):
+            bound: Dict[str, CacheBinding] = {}
+            for name, (need, state) in keeps.items():
+                b = CacheBinding()
+                if need is not None:
+                    src = i if cache_from is None else cache_from
+                    src_need = plan[src][0].get(name, (None, None))[0]
+                    if src_need != need:
+                        raise ValueError(f"schedule entry {i} reads the cache that entry {src} keeps for its part "
+                                         f"{name!r}, whose layout differs")
+                    g = needs.index(need)
+                    j = owners[g].index((src, name))
+                    b.group, b.writes = g, cache_from is None
+                    b.arrays = {a.name: self.pages[g][a.name][j] for a in need.arrays}
+                if state is not None:
+                    b.state = torch.zeros((self.max_requests,) + tuple(state.shape), device=rt.device,
+                                          dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[state.dtype])
+                bound[name] = b
+            self.bindings.append(bound)
+        self._states = [b.state for bound in self.bindings for b in bound.values() if b.state is not None]
+        self.cache = CacheManager([GroupLayout(n.window, self.release_window_pages) for n in needs],
+                                  [num_pages] * len(needs), self.page_size, self.max_requests, self.max_seq_len)
         self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
         self._graph_pool = None
 
     def kv_bytes_per_token(self) -> int:
-        size = torch.empty((), dtype=self.rt.dtype).element_size()
-        return sum(t.shape[0] * 2 * n.kv_heads * n.head_dim * size for t, n in zip(self.kv, self.group_needs))
+        """Bytes that one token takes in the pages of all groups."""
+        return sum(t.shape[0] * t.shape[2] * t.shape[3] * t.shape[4] // self.page_size * t.element_size()
+                   for arrays in self.pages for t in arrays.values())
 
     # ---- the step ------------------------------------------------------------
     def step(self, batch: StepBatch) -> torch.Tensor:
@@ -119,20 +138,23 @@ class ModelRunner:
         if batch.num_tokens == 0:
             return self.rt.empty((0, self.spec.vocab_size), torch.float32)
         self._zero_fresh_state(batch)
-        if self.use_graphs and batch.num_tokens == batch.num_requests:
+        if self.use_graphs and batch.one_token_each:
             return self._graph_step(batch)
         return self.model.forward(self._upload(batch), self.bindings)
 
     def _zero_fresh_state(self, batch: StepBatch) -> None:
-        """State slots of requests that start at position 0 in this step are cleared."""
-        if not any(b.state is not None for b in self.bindings):
+        """State slots of requests that start at position 0 in this step are cleared (before the step is
+        launched, so also before a captured step is replayed)."""
+        if not self._states:
             return
-        fresh = [int(batch.state_slots[s]) for s in range(batch.num_requests)
-                 if batch.q_start[s + 1] > batch.q_start[s] and batch.positions[batch.q_start[s]] == 0]
-        if fresh:
-            for b in self.bindings:
-                if b.state is not None:
-                    b.state[fresh] = 0
+        first = batch.q_start[:-1]
+        brings = batch.q_start[1:] > first
+        starts = np.zeros(batch.num_requests, dtype=bool)
+        starts[brings] = batch.positions[first[brings]] == 0
+        if starts.any():
+            slots = torch.from_numpy(batch.state_slots[starts].astype(np.int64)).to(self.rt.device)
+            for state in self._states:
+                state.index_fill_(0, slots, 0)
 
     def _context(self, dev: torch.Tensor, sizes: List[int], batch: StepBatch) -> StepContext:
         views, at = [], 0
@@ -144,7 +166,8 @@ class ModelRunner:
         tables = [views[N_FIXED + G + g].view(S, -1) for g in range(G)]
         return StepContext(rt=self.rt, num_tokens=T, num_requests=S, token_ids=views[0], positions=views[1],
                            seq_of_token=views[2], q_start=views[3], seq_lens=views[4], state_slots=views[5],
-                           logits_rows=views[6], slots=views[N_FIXED:N_FIXED + G], block_tables=tables, host=batch)
+                           logits_rows=views[6], slots=views[N_FIXED:N_FIXED + G], block_tables=tables, host=batch,
+                           one_token_each=batch.one_token_each)
 
     def _upload(self, batch: StepBatch) -> StepContext:
         sizes, flat = _pack(batch)
@@ -197,11 +220,16 @@ class _DecodeGraph:
         ctx.memo[("attention_tiles_host", 16)] = (tiles, S, bucket)
         ctx.host = None  # nothing may plan from host data inside the capture
         self.ctx = ctx
+        # The warm-up run really executes the step.  What it appends to the pages the replay writes again, the same
+        # values to the same places; per-request state, though, would be advanced twice, so it is put back.
+        kept = [state.clone() for state in runner._states]
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             runner.model.forward(ctx, runner.bindings)  # warm-up: library plans, allocator
             ctx.memo = {("attention_tiles_host", 16): (tiles, S, bucket)}
+            for state, before in zip(runner._states, kept):
+                state.copy_(before)
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()

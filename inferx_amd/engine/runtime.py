@@ -154,13 +154,22 @@ class Runtime:
 
 @dataclass
 class CacheBinding:
-    """What one layer execution sees of the cache manager's memory."""
+    """What one part of one layer execution sees of the cache manager's memory."""
 
     group: int = -1
-    k: Optional[torch.Tensor] = None       # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None       # [pages, kv_heads, head_dim, page_size] (transposed within a page)
+    arrays: Dict[str, torch.Tensor] = field(default_factory=dict)  # by the names of the part's `CacheNeed`
     writes: bool = True                    # False: reads another execution's cache
-    state: Optional[torch.Tensor] = None   # [slots, *shape] float32
+    state: Optional[torch.Tensor] = None   # [slots, *shape]
+
+    @property
+    def k(self) -> Optional[torch.Tensor]:
+        """Attention's keys: [pages, kv_heads, page_size, head_dim]."""
+        return self.arrays.get("k")
+
+    @property
+    def v(self) -> Optional[torch.Tensor]:
+        """Attention's values, transposed within a page: [pages, kv_heads, head_dim, page_size]."""
+        return self.arrays.get("v")
 
 
 @dataclass
@@ -178,4 +187,5 @@ class StepContext:
     slots: List[torch.Tensor]
     block_tables: List[torch.Tensor]
     host: Any = None                       # the StepBatch (host arrays), for parts that plan on the host
+    one_token_each: bool = False           # every request brings exactly one token (a decoding step)
     memo: Dict[Any, Any] = field(default_factory=dict)  # per-step results shared between layers

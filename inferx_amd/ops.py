@@ -85,14 +85,14 @@ def _is_i32(t, n=None):
 
 
 # ---------------------------------------------------------------------------
-def embed(h: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
-    """h[t] = table[ids[t]]; h float32 [T, H]."""
+def embed(h: torch.Tensor, table: torch.Tensor, ids: torch.Tensor, scale: float = 1.0) -> None:
+    """h[t] = table[ids[t]] * scale; h float32 [T, H]."""
     T, H = h.shape
     _need(h.dtype == torch.float32, "the residual stream is float32")
     _need(table.dim() == 2 and table.shape[1] == H, "table width differs from h")
     _is_i32(ids, T)
     _call("ix_embed", _ptr(h), _ptr(table), _i32(_dt(table)), _ptr(ids), _i64(T), _i64(H), _i64(table.shape[0]),
-          _stream())
+          _f32(scale), _stream())
 
 
 def add_rmsnorm(h: torch.Tensor, delta: Optional[torch.Tensor], weight: torch.Tensor, out: torch.Tensor, eps: float,

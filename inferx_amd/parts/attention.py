@@ -50,7 +50,10 @@ class PagedAttention(Mixer):
         return self.num_kv_heads * self.head_dim
 
     def cache_need(self) -> CacheNeed:
-        return CacheNeed(self.num_kv_heads, self.head_dim, self.window)
+        return CacheNeed.keys_and_values(self.num_kv_heads, self.head_dim, self.window)
+
+    def subparts(self):
+        return [self.position]
 
     def param_specs(self) -> List[ParamSpec]:
         H, s = self.hidden_size, self.init_std
@@ -92,7 +95,7 @@ class PagedAttention(Mixer):
         page_size = cache.k.shape[2]
         if q.dtype == torch.bfloat16 and page_size % 16 == 0 and self.head_dim % 16 == 0:
             T = ctx.num_tokens
-            if T > ctx.num_requests:  # some request brings more than one token: the step's plan says who goes where
+            if not ctx.one_token_each:  # some request brings more than one token: the step's plan says who goes where
                 lds_fits = self.head_dim <= 128 and page_size & (page_size - 1) == 0
                 lds, waves = mixed_step_plan(ctx, self.window, self.num_heads, self.num_kv_heads, lds_fits)
                 table = ctx.block_tables[cache.group]
@@ -307,7 +310,7 @@ def query_tiles(ctx, window: int, heads: int, head_dim: int = 128, kv_heads: Opt
     if hit is not None:
         return hit
     tiles_dev, n_tiles, longest = plan_tiles(ctx, tile)
-    grouped = tile == QUERY_TILE and ctx.num_tokens == ctx.num_requests and serves_group_together(heads, kv_heads)
+    grouped = tile == QUERY_TILE and ctx.one_token_each and serves_group_together(heads, kv_heads)
     units = n_tiles * (kv_heads if grouped else heads)
     ctx.memo[key] = (tiles_dev, tile, _n_splits(units, longest, window, tile), grouped)
     return ctx.memo[key]

@@ -1,22 +1,24 @@
 """Interfaces of the parts a layer is put together from, and their registries.
 
 A part is built from the parameters in its `PartSpec`, never from a config
-object, and does not know which model it is in.  Five kinds:
+object, and does not know which model it is in.  Seven kinds:
 
+  Embedding         forward(ctx) -> the residual stream h, float32 [T, hidden]
   Norm              forward(ctx, h, delta=None, rows=None) -> normed activations
   PositionEncoding  prepare(ctx) -> whatever its mixer's kernels need this step
   Mixer             forward(ctx, x, cache) -> delta   (attention here)
   FeedForward       forward(ctx, x) -> delta          (dense or experts)
-  Block             forward(ctx, h, pending, layer, cache) -> pending delta
+  Block             forward(ctx, h, pending, caches) -> pending delta; names the parts it arranges
+  Head              forward(ctx, x) -> float32 logits [rows, vocab]
 
 Every part lists the tensors it needs (`param_specs`) under local names; the
 `PartSpec` maps those to checkpoint names.  `bind` receives the loaded tensors
 (on the device, in their stored floating type or the run's type) and may fuse
 them (q/k/v rows stacked, experts stacked).
 
-A mixer also says what it keeps between steps: `cache_need()` (pages of keys
-and values, all of them or a window) and `state_need()` (a block of fixed size
-per request).
+Any part may keep something between steps and says so: `cache_need()` (arrays
+in pages, one entry per token: all tokens or a window of them) and
+`state_need()` (a block of fixed size per request).
 """
 from __future__ import annotations
 
@@ -37,21 +39,42 @@ class ParamSpec:
 
 
 @dataclass(frozen=True)
-class CacheNeed:
-    """Keys and values in pages.  `window` 0: all earlier tokens are read; W > 0:
-    only the last W (the query's own included), so older pages may be given back.
-    Entries with equal needs share a group of pages."""
+class CacheArray:
+    """One array that a part keeps per token, in pages: `heads` x `width` numbers per token.  Laid out
+    [pages, heads, page_size, width], or with `transposed` [pages, heads, width, page_size] (a page's tokens
+    contiguous per column).  `dtype` None: the run's type; else "float32" or "bfloat16".
+    (The reference's `KvLayout{entries_per_token, kv_heads, head_dim, dtype}`, include/inferx/core/kv_cache.h:14-38.)"""
 
-    kv_heads: int
-    head_dim: int
+    name: str
+    heads: int
+    width: int
+    transposed: bool = False
+    dtype: Optional[str] = None
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """What a part keeps per token, in pages: the arrays it names, for all earlier tokens (`window` 0) or only
+    the last W (the query's own included), so that older pages may be given back.  Parts with equal needs share a
+    group of pages (one pool, one block table per request); the runner allocates each array from this description
+    and knows nothing else about it."""
+
+    arrays: Tuple[CacheArray, ...]
     window: int = 0
+
+    @staticmethod
+    def keys_and_values(kv_heads: int, head_dim: int, window: int = 0) -> "CacheNeed":
+        """Attention's cache: keys [pages, kv_heads, page_size, head_dim] and values transposed within a page."""
+        return CacheNeed((CacheArray("k", kv_heads, head_dim), CacheArray("v", kv_heads, head_dim, transposed=True)),
+                         window)
 
 
 @dataclass(frozen=True)
 class StateNeed:
-    """A block of `shape` float32 numbers per request, zero when a request starts."""
+    """A block of `shape` numbers per request (float32 unless `dtype` says "bfloat16"), zero when a request starts."""
 
     shape: Tuple[int, ...]
+    dtype: str = "float32"
 
 
 class LazyDelta:
@@ -107,6 +130,17 @@ class Part:
     def bind(self, tensors: Dict[str, Any], rt) -> None:
         """Take ownership of the loaded tensors (keys: local names)."""
 
+    def subparts(self) -> List["Part"]:
+        """Parts this part built for itself (a mixer's position encoding)."""
+        return []
+
+    # ---- what the part keeps between steps (nothing unless it says so) ----
+    def cache_need(self) -> Optional[CacheNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
 
 class Norm(Part):
     def rms_operands(self):
@@ -123,13 +157,21 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    def cache_need(self) -> Optional[CacheNeed]:
-        return None
-
-    def state_need(self) -> Optional[StateNeed]:
-        return None
-
     def forward(self, ctx, x, cache):
+        """`cache`: the `CacheBinding` of this execution (its arrays of pages, its state), or None if the mixer
+        keeps nothing."""
+        raise NotImplementedError
+
+
+class Embedding(Part):
+    def forward(self, ctx):
+        """The residual stream for this step's tokens: float32 [T, hidden]."""
+        raise NotImplementedError
+
+
+class Head(Part):
+    def forward(self, ctx, x):
+        """x: the normalised wanted rows in the run's type; returns float32 logits [rows, vocab]."""
         raise NotImplementedError
 
 
@@ -141,23 +183,32 @@ class FeedForward(Part):
 
 
 class Block:
+    """An arrangement of parts around the residual stream.  `part_kinds` names the parts the arrangement needs
+    and the kind of each (a key of the registries); names in `optional_parts` may be left out of a `LayerSpec`.
+    The parts arrive built, by name, and are also set as attributes.  `caches` in `forward` holds, by part name,
+    the `CacheBinding` of every part of this execution that keeps pages or state."""
+
     graph_safe = False
+    part_kinds: Dict[str, str] = {}
+    optional_parts: Tuple[str, ...] = ()
 
-    def __init__(self, mixer: Mixer, feed_forward: FeedForward, mixer_norm: Norm, feed_forward_norm: Norm):
-        self.mixer, self.feed_forward = mixer, feed_forward
-        self.mixer_norm, self.feed_forward_norm = mixer_norm, feed_forward_norm
+    def __init__(self, parts: Dict[str, Part]):
+        self.parts = dict(parts)
+        for name in self.part_kinds:
+            setattr(self, name, self.parts.get(name))
 
-    def forward(self, ctx, h, pending, cache):
+    def forward(self, ctx, h, pending, caches):
         raise NotImplementedError
 
 
 _REGISTRIES: Dict[str, Dict[str, Callable[..., Any]]] = {
-    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {},
+    "norm": {}, "position": {}, "mixer": {}, "feed_forward": {}, "block": {}, "embedding": {}, "head": {},
 }
 
 
 def register_part(kind: str, name: str, factory: Callable[..., Any]) -> None:
-    """kind: 'norm' | 'position' | 'mixer' | 'feed_forward' | 'block'."""
+    """kind: 'norm' | 'position' | 'mixer' | 'feed_forward' | 'block' | 'embedding' | 'head'.  A block is
+    registered by its class (see `Block`), every other kind by a callable that takes the `PartSpec`'s parameters."""
     if kind not in _REGISTRIES:
         raise KeyError(f"no such kind of part: {kind!r} (known: {', '.join(_REGISTRIES)})")
     _REGISTRIES[kind][name] = factory
@@ -170,8 +221,18 @@ def build_part(kind: str, spec: PartSpec):
     return reg[spec.kind](**spec.params)
 
 
-def build_block(name: str, mixer, feed_forward, mixer_norm, feed_forward_norm) -> Block:
+def build_block(name: str, part_specs: Dict[str, PartSpec]) -> Block:
+    """The arrangement `name` with its parts built from their specs; a part the arrangement does not know, or one
+    it needs and does not get, is an error that names it."""
     reg = _REGISTRIES["block"]
     if name not in reg:
         raise KeyError(f"no block registered as {name!r} (known: {', '.join(sorted(reg)) or '(none)'})")
-    return reg[name](mixer, feed_forward, mixer_norm, feed_forward_norm)
+    cls = reg[name]
+    kinds = cls.part_kinds
+    unknown = sorted(set(part_specs) - set(kinds))
+    missing = sorted(set(kinds) - set(part_specs) - set(cls.optional_parts))
+    if unknown or missing:
+        raise KeyError(f"block {name!r} arranges the parts {sorted(kinds)}: " +
+                       "; ".join(([f"not known to it: {unknown}"] if unknown else []) +
+                                 ([f"missing: {missing}"] if missing else [])))
+    return cls({n: build_part(kinds[n], spec) for n, spec in part_specs.items()})

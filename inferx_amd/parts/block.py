@@ -14,10 +14,11 @@ from .base import Block, LazyNorm, register_part
 
 class PreNormBlock(Block):
     graph_safe = True
+    part_kinds = {"mixer": "mixer", "feed_forward": "feed_forward", "mixer_norm": "norm", "feed_forward_norm": "norm"}
 
-    def forward(self, ctx, h, pending, cache):
+    def forward(self, ctx, h, pending, caches):
         x = self.mixer_norm.forward(ctx, h, pending)
-        a = self.mixer.forward(ctx, x, cache)
+        a = self.mixer.forward(ctx, x, caches.get("mixer"))
         if self.feed_forward.takes_lazy_norm:
             return self.feed_forward.forward(ctx, LazyNorm(self.feed_forward_norm, h, a))
         return self.feed_forward.forward(ctx, self.feed_forward_norm.forward(ctx, h, a))

@@ -1,10 +1,13 @@
 """A decoder model put together from a `ModelSpec`: embedding, layers in the
 order of the schedule, final norm, head.  Nothing here names an architecture.
 
-    logits = head( final_norm( run of blocks( embed(ids) ) )[wanted rows] )
+    logits = head( final_norm( run of blocks( embedding(ids) ) )[wanted rows] )
 
 Only the wanted rows go through the final norm and the head (the reference
-computes all rows and picks afterwards, src/model/qwen2.cc:1059-1066).
+computes all rows and picks afterwards, src/model/qwen2.cc:1059-1066).  Both
+ends are parts like the others: an architecture that scales its embeddings,
+adds learned positions or caps its logits registers an embedding or a head of
+its own.
 """
 from __future__ import annotations
 
@@ -12,9 +15,8 @@ from typing import Dict, List, Optional, Tuple
 
 import torch
 
-from .. import ops
 from ..config.spec import ModelSpec, PartSpec
-from .base import CacheNeed, ParamSpec, StateNeed, build_block, build_part
+from .base import CacheNeed, ParamSpec, Part, StateNeed, build_block, build_part
 
 
 class DecoderModel:
@@ -22,69 +24,70 @@ class DecoderModel:
         spec.validate()
         self.spec = spec
         self.blocks = []
-        self._part_specs: List[Tuple[PartSpec, object]] = []  # (spec, part) for every part that has tensors
+        self._part_specs: List[Tuple[PartSpec, Part]] = []  # (spec, part) for every part built from a spec
+        self.embedding = build_part("embedding", spec.embedding)
+        self._part_specs.append((spec.embedding, self.embedding))
         for layer in spec.layers:
-            mixer = build_part("mixer", layer.mixer)
-            ffn = build_part("feed_forward", layer.feed_forward)
-            n1 = build_part("norm", layer.mixer_norm)
-            n2 = build_part("norm", layer.feed_forward_norm)
-            self.blocks.append(build_block(layer.block, mixer, ffn, n1, n2))
-            self._part_specs += [(layer.mixer, mixer), (layer.feed_forward, ffn), (layer.mixer_norm, n1),
-                                 (layer.feed_forward_norm, n2)]
+            block = build_block(layer.block, layer.parts)
+            self.blocks.append(block)
+            self._part_specs += [(layer.parts[name], block.parts[name]) for name in layer.parts]
         self.final_norm = build_part("norm", spec.final_norm)
-        self._part_specs.append((spec.final_norm, self.final_norm))
-        self.embedding: Optional[torch.Tensor] = None
-        self.head: Optional[torch.Tensor] = None
+        self.head = build_part("head", spec.head)
+        self._part_specs += [(spec.final_norm, self.final_norm), (spec.head, self.head)]
 
     # ---- tensors ---------------------------------------------------------
     def expected_tensors(self) -> Dict[str, ParamSpec]:
-        """Checkpoint name -> what must be there (shape, and how to draw it at random)."""
-        s = self.spec
-        out: Dict[str, ParamSpec] = {
-            s.embedding_name: ParamSpec(s.embedding_name, (s.vocab_size, s.hidden_size), std=s.init_std)}
-        if s.head_name is not None:
-            out[s.head_name] = ParamSpec(s.head_name, (s.vocab_size, s.hidden_size), std=s.init_std)
+        """Checkpoint name -> what must be there (shape, and how to draw it at random).  Two parts may name the
+        same tensor (a head tied to the embedding) if they agree on its shape."""
+        out: Dict[str, ParamSpec] = {}
         for pspec, part in self._part_specs:
             for p in part.param_specs():
                 name = pspec.tensor_name(p.name)
-                if name in out and out[name].shape != tuple(p.shape):
+                if name in out and tuple(out[name].shape) != tuple(p.shape):
                     raise ValueError(f"tensor {name!r} is claimed twice with different shapes")
-                out[name] = p
+                out.setdefault(name, p)
         return out
 
     def bind(self, weights: Dict[str, torch.Tensor], rt) -> None:
         """Hand every part its tensors (already on the device).  `weights` is emptied."""
-        s = self.spec
-        self.embedding = weights[s.embedding_name].contiguous()
-        self.head = weights[s.head_name].contiguous() if s.head_name is not None else self.embedding
         for pspec, part in self._part_specs:
             local = {p.name: weights[pspec.tensor_name(p.name)] for p in part.param_specs()}
             part.bind(local, rt)
         weights.clear()
 
+    def all_parts(self) -> List[Part]:
+        """Every part of the model, the blocks and the parts' own sub-parts included."""
+        out: List = [self.embedding, self.final_norm, self.head]
+        for b in self.blocks:
+            out.append(b)
+            out += list(b.parts.values())
+        for p in list(out):
+            out += [s for s in getattr(p, "subparts", lambda: [])() if s is not None]
+        return out
+
     def graph_safe(self) -> bool:
         """True if every part may run inside a captured HIP graph."""
-        parts = [self.final_norm]
-        for b in self.blocks:
-            parts += [b, b.mixer, b.feed_forward, b.mixer_norm, b.feed_forward_norm]
-            parts.append(getattr(b.mixer, "position", None))
-        return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
+        return all(getattr(p, "graph_safe", False) for p in self.all_parts())
 
     # ---- what the cache manager must provide -------------------------------
     def cache_plan(self):
-        """Per schedule entry: (CacheNeed or None, StateNeed or None, cache_from)."""
+        """Per schedule entry: ({part name: (CacheNeed or None, StateNeed or None)} for the parts of the layer that
+        keep something between steps, cache_from)."""
         plan = []
         for entry in self.spec.schedule:
-            mixer = self.blocks[entry.layer].mixer
-            plan.append((mixer.cache_need(), mixer.state_need(), entry.cache_from))
+            keeps: Dict[str, Tuple[Optional[CacheNeed], Optional[StateNeed]]] = {}
+            for name, part in self.blocks[entry.layer].parts.items():
+                need, state = part.cache_need(), part.state_need()
+                if need is not None or state is not None:
+                    keeps[name] = (need, state)
+            plan.append((keeps, entry.cache_from))
         return plan
 
     # ---- one step ----------------------------------------------------------
     def forward(self, ctx, caches) -> torch.Tensor:
-        """caches: one CacheBinding per schedule entry.  Returns float32 [R, vocab]."""
+        """caches: per schedule entry, the `CacheBinding`s of its parts by name.  Returns float32 [R, vocab]."""
         s = self.spec
-        h = ctx.rt.empty((ctx.num_tokens, s.hidden_size), torch.float32)
-        ops.embed(h, self.embedding, ctx.token_ids)
+        h = self.embedding.forward(ctx)
         pending = None
         for i, entry in enumerate(s.schedule):
             pending = self.blocks[entry.layer].forward(ctx, h, pending, caches[i])
@@ -92,7 +95,7 @@ class DecoderModel:
         if rows.numel() == 0:
             return ctx.rt.empty((0, s.vocab_size), torch.float32)
         x = self.final_norm.forward(ctx, h, pending, rows=rows)
-        return ctx.rt.linear_f32(x, self.head)
+        return self.head.forward(ctx, x)
 
 
 def build_model(spec: ModelSpec) -> DecoderModel:

@@ -10,22 +10,19 @@ run; integer tables become int32.
 """
 from __future__ import annotations
 
-from typing import Dict, List
+from typing import Dict, List, Sequence
 
 import torch
 
 from .safetensors_io import Checkpoint, CheckpointError
 
-# tensors some writers add that no part asks for
-_IGNORED_SUFFIXES = ("rotary_emb.inv_freq",)
 
-
-def check_names_and_shapes(expected: Dict[str, tuple], ckpt: Checkpoint, tied_head_name: str = "lm_head.weight",
-                           head_is_tied: bool = False) -> None:
+def check_names_and_shapes(expected: Dict[str, tuple], ckpt: Checkpoint, ignored_suffixes: Sequence[str] = ()) -> None:
+    """`ignored_suffixes`: endings of tensor names that a checkpoint of this architecture may hold although no part
+    asks for them (the model's spec lists them)."""
     missing: List[str] = sorted(n for n in expected if n not in ckpt)
-    unexpected = sorted(
-        n for n in ckpt.names()
-        if n not in expected and not n.endswith(_IGNORED_SUFFIXES) and not (head_is_tied and n == tied_head_name))
+    ignored = tuple(ignored_suffixes)
+    unexpected = sorted(n for n in ckpt.names() if n not in expected and not (ignored and n.endswith(ignored)))
     wrong = sorted(
         f"{n}: expected {list(expected[n])}, file has {list(ckpt.shape(n))}"
         for n in expected if n in ckpt and tuple(ckpt.shape(n)) != tuple(expected[n]))
@@ -51,5 +48,5 @@ def load_weights(model, model_dir: str, rt) -> Dict[str, torch.Tensor]:
     """All tensors the model needs, on the device, keyed by checkpoint name."""
     ckpt = Checkpoint.open(model_dir)
     expected = {name: tuple(p.shape) for name, p in model.expected_tensors().items()}
-    check_names_and_shapes(expected, ckpt, head_is_tied=model.spec.head_name is None)
+    check_names_and_shapes(expected, ckpt, model.spec.ignored_tensor_suffixes)
     return {name: rt.place(ckpt.get(name)) for name in expected}

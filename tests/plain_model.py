@@ -3,7 +3,7 @@ float64, whole sequences, no cache, no batching, one function per part.
 
 It shares no code with `inferx_amd`: it reads config.json keys and checkpoint
 tensor names itself.  Every function cites the place in the reference
-(/root/reference, paths relative to it) whose formula it follows.  The
+(divedb/InferX, paths relative to its root) whose formula it follows.  The
 reference was read, not run.
 """
 from __future__ import annotations
@@ -151,7 +151,10 @@ def is_moe_layer(cfg: dict, layer: int) -> bool:
 
 
 def window_of_layer(cfg: dict, layer: int) -> int:
-    """Windowed iff use_sliding_window and layer >= max_window_layers (window semantics layers.cu:346-354)."""
+    """Windowed iff use_sliding_window and layer >= max_window_layers (window semantics layers.cu:346-354); a
+    config that lists `layer_types` names its windowed layers itself ("sliding_attention")."""
+    if cfg.get("layer_types"):
+        return int(cfg["sliding_window"]) if cfg["layer_types"][layer] == "sliding_attention" else 0
     if cfg.get("use_sliding_window", False) and cfg.get("sliding_window", 0) and \
             layer >= cfg.get("max_window_layers", cfg["num_hidden_layers"]):
         return int(cfg["sliding_window"])

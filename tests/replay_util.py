@@ -79,8 +79,9 @@ def mixed(prompts: Dict[str, List[int]], seed: int, max_live: int = 4, max_token
     return steps
 
 
-def replay(runner, steps: List[Step]) -> Dict[Tuple[str, int], torch.Tensor]:
-    """Run the steps; logits by (request, position) on the CPU."""
+def replay(runner, steps: List[Step], page_owners: dict = None) -> Dict[Tuple[str, int], torch.Tensor]:
+    """Run the steps; logits by (request, position) on the CPU.  `page_owners`, if given, collects for every
+    physical page (group, page) the requests that held it during some step."""
     got: Dict[Tuple[str, int], torch.Tensor] = {}
     for step in steps:
         for rid, _, _ in step["entries"]:
@@ -96,6 +97,12 @@ def replay(runner, steps: List[Step]) -> Dict[Tuple[str, int], torch.Tensor]:
                 got[key] = logits[row]
                 row += 1
         assert row == logits.shape[0]
+        if page_owners is not None:
+            for rid, _, _ in step["entries"]:
+                for g in range(len(runner.cache.groups)):
+                    for page in runner.cache.block_row(rid, g):
+                        if page >= 0:
+                            page_owners.setdefault((g, int(page)), set()).add(rid)
         for rid in step["end"]:
             runner.end_request(rid)
         runner.cache.check()

@@ -44,11 +44,34 @@ def test_which_layer_is_which():
     a = config_from_dict(tiny.CONFIG_A)
     assert [a.is_moe_layer(l) for l in range(2)] == [True, True]
     spec = b.model_spec()
-    assert [l.feed_forward.kind for l in spec.layers] == ["dense_mlp", "moe", "dense_mlp", "moe"]
-    assert [l.mixer.params["window"] for l in spec.layers] == [0, 0, 16, 16]
-    assert spec.head_name is None and a.model_spec().head_name == "lm_head.weight"
-    assert spec.layers[1].feed_forward.params["renormalize"] is True
-    assert spec.layers[0].mixer_norm.params["eps"] == 1e-5
+    assert [l.parts["feed_forward"].kind for l in spec.layers] == ["dense_mlp", "moe", "dense_mlp", "moe"]
+    assert [l.parts["mixer"].params["window"] for l in spec.layers] == [0, 0, 16, 16]
+    # B ties its head to the embedding: both parts name the same checkpoint tensor
+    assert spec.head.tensor_name("weight") == spec.embedding.tensor_name("weight") == "model.embed_tokens.weight"
+    assert a.model_spec().head.tensor_name("weight") == "lm_head.weight"
+    assert spec.layers[1].parts["feed_forward"].params["renormalize"] is True
+    assert spec.layers[0].parts["mixer_norm"].params["eps"] == 1e-5
+    assert all(l.block == "prenorm" and sorted(l.parts) == ["feed_forward", "feed_forward_norm", "mixer",
+                                                            "mixer_norm"] for l in spec.layers)
+
+
+def test_layer_types_name_the_windowed_layers_outright():
+    raw = dict(tiny.CONFIG_B, layer_types=["sliding_attention", "full_attention", "sliding_attention",
+                                           "full_attention"])
+    c = config_from_dict(raw)
+    assert [c.window_of_layer(l) for l in range(4)] == [16, 0, 16, 0]
+    assert [l.parts["mixer"].params["window"] for l in c.model_spec().layers] == [16, 0, 16, 0]
+    assert config_from_dict(c.to_dict()).layer_types == raw["layer_types"]
+    assert "layer_types" not in config_from_dict(tiny.CONFIG_B).to_dict()
+    # the list decides alone, whatever use_sliding_window says
+    off = config_from_dict(dict(raw, use_sliding_window=False))
+    assert [off.window_of_layer(l) for l in range(4)] == [16, 0, 16, 0]
+    for bad, needle in [(["full_attention"] * 3, "names 3 layers"), (["chunked"] * 4, "only full_attention"),
+                        ("full_attention", "list of strings")]:
+        with pytest.raises(ConfigError, match=needle):
+            config_from_dict(dict(raw, layer_types=bad))
+    with pytest.raises(ConfigError, match="sliding_window is not positive"):
+        config_from_dict(dict(raw, sliding_window=0, use_sliding_window=False))
 
 
 @pytest.mark.parametrize("change, needle", [

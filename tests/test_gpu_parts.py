@@ -36,7 +36,8 @@ def make_ctx(rt, q_lens, seq_lens, page_size, pages, groups=1):
     return StepContext(rt=rt, num_tokens=batch.num_tokens, num_requests=S, token_ids=views[0], positions=views[1],
                        seq_of_token=views[2], q_start=views[3], seq_lens=views[4], state_slots=views[5],
                        logits_rows=views[6], slots=views[7:7 + G],
-                       block_tables=[views[7 + G + g].view(S, -1) for g in range(G)], host=batch), batch
+                       block_tables=[views[7 + G + g].view(S, -1) for g in range(G)], host=batch,
+                       one_token_each=batch.one_token_each), batch
 
 
 def tensors_for(part, rt, seed=0, std=None):
@@ -99,8 +100,8 @@ def test_attention_part_whole_and_in_two_steps(dtype, tol, heads, kv, d, window,
 
     def run(splits):
         pages, page = 4, 16
-        cache = CacheBinding(group=0, k=torch.zeros(pages, kv, page, d, dtype=rt.dtype, device=DEV),
-                             v=torch.zeros(pages, kv, d, page, dtype=rt.dtype, device=DEV))
+        cache = CacheBinding(group=0, arrays=dict(k=torch.zeros(pages, kv, page, d, dtype=rt.dtype, device=DEV),
+                                                v=torch.zeros(pages, kv, d, page, dtype=rt.dtype, device=DEV)))
         outs, done = [], 0
         for n in splits:
             ctx, _ = make_ctx(rt, [n], [done + n], page, pages)
@@ -161,7 +162,7 @@ def test_attention_kernels_chosen_by_the_step(heads, kv, d, window, q_lens, seq_
         wants[-1] = torch.einsum("hqk,khd->qhd", torch.softmax(sc.masked_fill(~ok[None], -float("inf")), -1), vv)
     q = torch.cat(qs).to(DEV)
     out = torch.full_like(q, float("nan"))
-    part.attend(ctx, q, CacheBinding(group=0, k=k_cache.to(DEV), v=v_cache.to(DEV)), out)
+    part.attend(ctx, q, CacheBinding(group=0, arrays=dict(k=k_cache.to(DEV), v=v_cache.to(DEV))), out)
     assert err(out, torch.cat(wants)) < 1.5e-2
     # the plan that attend() followed (memoised in the step's context)
     from inferx_amd.parts import attention

@@ -8,7 +8,7 @@ import tiny
 
 pytestmark = pytest.mark.gpu
 
-PROMPT_LENGTHS = {"A": (5, 9, 17, 70), "B": (7, 23, 40, 75), "C": (11, 50), "D": (3, 37, 66)}
+PROMPT_LENGTHS = {"A": (5, 9, 17, 70), "B": (7, 23, 40, 75), "C": (11, 50, 29, 70), "D": (3, 37, 66)}
 
 
 @pytest.fixture(scope="module")
@@ -82,7 +82,7 @@ def test_bfloat16_run_keeps_tensors_stored_in_32_bits(folders, name):
     from inferx_amd.engine.runner import ModelRunner
     runner = ModelRunner.from_directory(folders[(name, "float32")], dtype="bfloat16", page_size=16, num_pages=64,
                                         max_requests=4, max_seq_len=1024)
-    assert runner.model.embedding.dtype == torch.float32
+    assert runner.model.embedding.weight.dtype == torch.float32
     assert runner.model.blocks[-1].mixer.w_qkv.dtype == torch.float32
     prompts = prompts_for(name)
     for steps in (ru.whole(prompts), ru.tail_decoded(prompts, 8), ru.mixed(prompts, seed=3)):
@@ -115,9 +115,13 @@ def test_mixed_with_few_pages(folders, name, dtype):
     # room for about two of the longer requests: pages are given back and used again
     max_tokens = 192
     runner = make_runner(folders, name, dtype, num_pages=max_tokens // 16)
-    used = set()
-    steps = ru.mixed(prompts, seed=5, max_tokens=max_tokens)
-    got = ru.replay(runner, steps)
+    owners = {}
+    steps = ru.mixed(prompts, seed=8, max_tokens=max_tokens)
+    assert any(len(s["entries"]) > 1 and {len(e[1]) for e in s["entries"]} & {1} and
+               max(len(e[1]) for e in s["entries"]) > 1 for s in steps), "no step mixes a portion with a single token"
+    got = ru.replay(runner, steps, page_owners=owners)
+    reused = [key for key, rids in owners.items() if len(rids) > 1]
+    assert reused, "no physical page served two requests: the pool is too large for this test to bite"
     ru.compare(got, expected_for(folders, name, dtype), tol_of(dtype), f"mixed {name} {dtype}",
                ties_for(folders, name, dtype))
     assert all(p.used_pages == 0 for p in runner.cache.pools)
@@ -188,3 +192,27 @@ def test_random_configurations(tmp_path, seed, dtype, monkeypatch):
         runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=page, num_pages=4 * (160 // page + 2),
                                             max_requests=4, max_seq_len=256)
         ru.compare(ru.replay(runner, steps), want, (ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL), f"seed {seed} {dtype} {how}", skip=skip)
+
+
+@pytest.mark.parametrize("use_graphs", [True, False])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_an_entry_without_tokens_beside_one_with_two(folders, dtype, use_graphs):
+    """A step may name a request that brings no token.  Beside a request that brings two, the step then has as
+    many tokens as requests without being a step of one token each: it must not be taken for a decoding step
+    (whose tiles and graphs assume row i = request i)."""
+    from inferx_amd.engine.runner import ModelRunner
+    name = "B"
+    runner = ModelRunner.from_directory(folders[(name, dtype)], dtype=dtype, page_size=16, num_pages=64,
+                                        max_requests=4, max_seq_len=1024, use_graphs=use_graphs)
+    prompts = {k: v for k, v in list(prompts_for(name).items())[1:3]}
+    (a, ta), (b, tb) = prompts.items()
+    steps = [{"entries": [(a, ta[:9], list(range(9)))], "end": []},
+             {"entries": [(b, tb[:20], list(range(20)))], "end": []},
+             {"entries": [(a, [], []), (b, tb[20:22], [0, 1])], "end": []},       # 2 tokens, 2 requests
+             {"entries": [(a, ta[9:11], [0, 1]), (b, [], [])], "end": []},
+             {"entries": [(a, ta[11:12], [0]), (b, tb[22:23], [0])], "end": []},  # a true step of one token each
+             {"entries": [(a, ta[12:], list(range(len(ta) - 12))), (b, tb[23:], list(range(len(tb) - 23)))],
+              "end": [a, b]}]
+    got = ru.replay(runner, steps)
+    expected = {k: v for k, v in expected_for(folders, name, dtype).items() if k in prompts}
+    ru.compare(got, expected, tol_of(dtype), f"empty entry {dtype} graphs={use_graphs}", ties_for(folders, name, dtype))

@@ -20,8 +20,8 @@ DEV = "cuda:0"
 # ---- the toy mixer: a leaky running sum over the request's tokens -----------------------------
 #   s_t = decay * s_{t-1} + W_in x_t ;  y_t = W_out s_t          (s carried across steps in a state slot)
 def define_toy():
-    from inferx_amd.config import ModelSpec, PartSpec, ScheduleEntry, register_architecture
-    from inferx_amd.config.spec import LayerSpec
+    from inferx_amd.config import (LayerSpec, ModelSpec, PartSpec, ScheduleEntry, linear_head, register_architecture,
+                                   token_embedding)
     from inferx_amd.parts import Mixer, ParamSpec, StateNeed, register_part
 
     class RunningSumMixer(Mixer):
@@ -38,9 +38,19 @@ def define_toy():
         def bind(self, tensors, rt):
             self.w_in, self.w_out = tensors["in.weight"].float(), tensors["out.weight"].float()
 
+        # A step of one token per request only launches work on the device (its state slots come from the step's
+        # device arrays), so the part may be captured into a graph; other steps walk their requests on the host,
+        # which no captured step ever does.
+        graph_safe = True
+
         def forward(self, ctx, x, cache):
-            batch = ctx.host  # host arrays of the step: which rows belong to which request, and its state slot
             u = x.float() @ self.w_in.T
+            if ctx.one_token_each:
+                slots = ctx.state_slots.long()
+                s_all = self.decay * cache.state.index_select(0, slots) + u
+                cache.state.index_copy_(0, slots, s_all)
+                return (s_all @ self.w_out.T).to(x.dtype)
+            batch = ctx.host  # host arrays of the step: which rows belong to which request, and its state slot
             s_all = torch.empty_like(u)
             for r in range(batch.num_requests):
                 b, e, slot = int(batch.q_start[r]), int(batch.q_start[r + 1]), int(batch.state_slots[r])
@@ -80,10 +90,12 @@ def define_toy():
                                                    "position": PartSpec("rope", {"theta": 1e4, "rotary_dim": 16})},
                                      prefix=p + "attn.")
                 ffn = PartSpec("dense_mlp", {"hidden_size": H, "width": r["width"], "init_std": 0.2}, prefix=p + "mlp.")
-                layers.append(LayerSpec("prenorm", mixer, ffn, norm(p + "norm1."), norm(p + "norm2.")))
-            return ModelSpec("ToyStateForCausalLM", H, r["vocab_size"], 0, layers,
-                             [ScheduleEntry(l) for l in range(len(layers))], "embed.weight", norm("final_norm."),
-                             None, init_std=0.5)
+                layers.append(LayerSpec("prenorm", {"mixer": mixer, "feed_forward": ffn, "mixer_norm": norm(p + "norm1."),
+                                                    "feed_forward_norm": norm(p + "norm2.")}))
+            V = r["vocab_size"]
+            return ModelSpec("ToyStateForCausalLM", H, V, 0, layers, [ScheduleEntry(l) for l in range(len(layers))],
+                             token_embedding("embed.weight", V, H, 0.5), norm("final_norm."),
+                             linear_head("embed.weight", V, H, 0.5), init_std=0.5)
 
     register_architecture("ToyStateForCausalLM", ToyConfig)
     return ToyConfig
@@ -138,10 +150,13 @@ def test_a_mixer_with_state_of_its_own(tmp_path, dtype, tol):
                         ("chunked", ru.chunked(prompts)), ("mixed", ru.mixed(prompts, seed=2, max_live=2))]:
         runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=16, num_pages=8, max_requests=2,
                                             max_seq_len=128)
-        assert not runner.use_graphs  # the toy mixer plans on the host: it does not claim to be graph-safe
-        assert sum(b.state is not None for b in runner.bindings) == 2 and len(runner.kv) == 1
+        assert runner.use_graphs  # a model with a stateful part of its own still replays its decoding steps
+        assert sum(b.state is not None for bound in runner.bindings for b in bound.values()) == 2
+        assert len(runner.pages) == 1 and runner.group_owners == [[(1, "mixer")]]
         got = ru.replay(runner, steps)
         ru.compare(got, expected, tol, f"toy {name} {dtype}")
+        if name != "mixed":  # (a mixed trace may or may not hold a step of one token each)
+            assert bool(runner._graphs) == (name == "tail"), f"{name}: graphs {list(runner._graphs)}"
 
 
 @pytest.mark.parametrize("dtype,tol", [("float32", ru.FP32_TOL), ("bfloat16", ru.BF16_TOL)])
@@ -170,7 +185,10 @@ def test_layer_order_is_data(tmp_path, dtype, tol):
     model = build_model(config.model_spec())
     runner = ModelRunner(config, load_weights(model, str(tmp_path), rt), rt, page_size=16, num_pages=16,
                          max_requests=2, max_seq_len=128, model=model)
-    assert runner.kv[0].shape[0] == 3  # three executions own a cache; the fourth reads the first one's
+    # three executions own a cache; the fourth reads the first one's
+    assert runner.group_owners == [[(0, "mixer"), (1, "mixer"), (2, "mixer")]] and runner.pages[0]["k"].shape[0] == 3
+    assert runner.bindings[3]["mixer"].k.data_ptr() == runner.bindings[0]["mixer"].k.data_ptr()
+    assert not runner.bindings[3]["mixer"].writes
     prompts = {"a": tiny.random_tokens(40, 256, 7), "b": tiny.random_tokens(9, 256, 8)}
     expected = {rid: pm.forward(cfg, weights, toks, schedule=schedule) for rid, toks in prompts.items()}
     for steps in (ru.whole(prompts), ru.chunked(prompts), ru.tail_decoded(prompts, 12)):
@@ -182,8 +200,8 @@ def test_layer_order_is_data(tmp_path, dtype, tol):
 #   feed-forward: every token goes to ONE of a few small experts, the one whose router score is largest:
 #                 y_t = W2[e_t] relu(W1[e_t] x_t),  e_t = argmax_e (Wr x_t)_e
 def define_toy_routed():
-    from inferx_amd.config import ModelSpec, PartSpec, ScheduleEntry, register_architecture
-    from inferx_amd.config.spec import LayerSpec
+    from inferx_amd.config import (LayerSpec, ModelSpec, PartSpec, ScheduleEntry, linear_head, register_architecture,
+                                   token_embedding)
     from inferx_amd.parts import FeedForward, LazyNorm, ParamSpec, PositionEncoding, register_part, resolve_input
 
     class StretchedRotary(PositionEncoding):
@@ -250,10 +268,12 @@ def define_toy_routed():
                                  prefix=p + "attn.")
                 ffn = PartSpec("toy_switch", {"hidden_size": H, "width": r["width"], "num_experts": r["experts"]},
                                prefix=p + "ffn.")
-                layers.append(LayerSpec("prenorm", mixer, ffn, norm(p + "norm1."), norm(p + "norm2.")))
-            return ModelSpec("ToyRoutedForCausalLM", H, r["vocab_size"], 0, layers,
-                             [ScheduleEntry(l) for l in range(len(layers))], "embed.weight", norm("final_norm."),
-                             None, init_std=0.5)
+                layers.append(LayerSpec("prenorm", {"mixer": mixer, "feed_forward": ffn, "mixer_norm": norm(p + "norm1."),
+                                                    "feed_forward_norm": norm(p + "norm2.")}))
+            V = r["vocab_size"]
+            return ModelSpec("ToyRoutedForCausalLM", H, V, 0, layers, [ScheduleEntry(l) for l in range(len(layers))],
+                             token_embedding("embed.weight", V, H, 0.5), norm("final_norm."),
+                             linear_head("embed.weight", V, H, 0.5), init_std=0.5)
 
     register_architecture("ToyRoutedForCausalLM", ToyRoutedConfig)
     return ToyRoutedConfig
@@ -325,3 +345,233 @@ def test_a_routed_feed_forward_and_another_position_encoding(tmp_path, dtype, to
         assert not runner.use_graphs  # the toy parts do not claim to be graph-safe
         got = ru.replay(runner, steps)
         ru.compare(got, expected, tol, f"toy routed {name} {dtype}")
+
+
+# ---- other arrangements, another kind of cache, other ends of the model: all defined HERE ----------------------
+#   sandwich block: four norms     h += post1(mixer(pre1(h)));  h += post2(ffn(pre2(h)))
+#   parallel block: one norm       x = norm(h);  h += mixer(x) + ffn(x)
+#   latent mixer: keeps ONE array of `rank` numbers per token (c_t = Wc x_t) instead of keys and values, and reads
+#       it back through the block table:  y_t = Wo sum_{j<=t} softmax_j(q_t . c_j / sqrt(rank)) c_j,  q_t = Wq x_t
+#   embedding: table[id] * scale + learned_position[position];  head: cap * tanh((x . W^T + bias) / cap)
+def define_toy_shapes():
+    from inferx_amd.config import LayerSpec, ModelSpec, PartSpec, ScheduleEntry, register_architecture
+    from inferx_amd.parts import (Block, CacheArray, CacheNeed, Embedding, Head, Mixer, ParamSpec, register_part,
+                                  resolve_delta)
+
+    class SandwichBlock(Block):
+        part_kinds = {"mixer": "mixer", "feed_forward": "feed_forward", "pre_mixer": "norm", "post_mixer": "norm",
+                      "pre_ffn": "norm", "post_ffn": "norm"}
+
+        def forward(self, ctx, h, pending, caches):
+            zero = lambda: torch.zeros_like(h)
+            x = self.pre_mixer.forward(ctx, h, pending)
+            a = resolve_delta(ctx, self.mixer.forward(ctx, x, caches.get("mixer")))
+            a = self.post_mixer.forward(ctx, a.float().contiguous(), None)     # a norm of the delta, not of h
+            x = self.pre_ffn.forward(ctx, h, a)
+            f = resolve_delta(ctx, self.feed_forward.forward(ctx, x))
+            return self.post_ffn.forward(ctx, f.float().contiguous(), None)
+
+    class ParallelBlock(Block):
+        part_kinds = {"mixer": "mixer", "feed_forward": "feed_forward", "norm": "norm"}
+
+        def forward(self, ctx, h, pending, caches):
+            x = self.norm.forward(ctx, h, pending)
+            a = resolve_delta(ctx, self.mixer.forward(ctx, x, caches.get("mixer")))
+            f = resolve_delta(ctx, self.feed_forward.forward(ctx, x))
+            return a + f
+
+    class LatentMixer(Mixer):
+        def __init__(self, hidden_size, rank):
+            self.hidden_size, self.rank = hidden_size, rank
+
+        def cache_need(self):
+            return CacheNeed((CacheArray("latent", 1, self.rank, dtype="float32"),))
+
+        def param_specs(self):
+            H, r = self.hidden_size, self.rank
+            return [ParamSpec("c.weight", (r, H), std=0.15), ParamSpec("q.weight", (r, H), std=0.15),
+                    ParamSpec("o.weight", (H, r), std=0.4)]
+
+        def bind(self, tensors, rt):
+            self.wc, self.wq, self.wo = (tensors[n].float() for n in ("c.weight", "q.weight", "o.weight"))
+
+        def forward(self, ctx, x, cache):
+            pages = cache.arrays["latent"]                     # [pages, 1, page_size, rank], as the need says
+            page_size = pages.shape[2]
+            flat = pages.view(-1, self.rank)                   # slot = page * page_size + offset
+            xf = x.float()
+            flat.index_copy_(0, ctx.slots[cache.group].long(), xf @ self.wc.T)
+            q = xf @ self.wq.T
+            batch, table = ctx.host, ctx.block_tables[cache.group]
+            out = torch.empty_like(q)
+            for t in range(batch.num_tokens):
+                s, p = int(batch.seq_of_token[t]), int(batch.positions[t])
+                keys = torch.arange(p + 1, device=x.device)
+                slots = table[s, keys // page_size].long() * page_size + keys % page_size
+                c = flat[slots]
+                out[t] = torch.softmax(c @ q[t] / self.rank ** 0.5, 0) @ c
+            return (out @ self.wo.T).to(x.dtype)
+
+    class ScaledPositionalEmbedding(Embedding):
+        def __init__(self, vocab_size, hidden_size, max_positions, scale):
+            self.vocab_size, self.hidden_size, self.max_positions, self.scale = vocab_size, hidden_size, max_positions, scale
+
+        def param_specs(self):
+            return [ParamSpec("tokens.weight", (self.vocab_size, self.hidden_size), std=0.5),
+                    ParamSpec("positions.weight", (self.max_positions, self.hidden_size), std=0.5)]
+
+        def bind(self, tensors, rt):
+            self.tokens, self.positions = tensors["tokens.weight"].float(), tensors["positions.weight"].float()
+
+        def forward(self, ctx):
+            return (self.tokens[ctx.token_ids.long()] * self.scale + self.positions[ctx.positions.long()]).contiguous()
+
+    class CappedHead(Head):
+        def __init__(self, vocab_size, hidden_size, cap):
+            self.vocab_size, self.hidden_size, self.cap = vocab_size, hidden_size, cap
+
+        def param_specs(self):
+            return [ParamSpec("weight", (self.vocab_size, self.hidden_size), std=0.5),
+                    ParamSpec("bias", (self.vocab_size,), std=0.5)]
+
+        def bind(self, tensors, rt):
+            self.weight, self.bias = tensors["weight"].float(), tensors["bias"].float()
+
+        def forward(self, ctx, x):
+            return self.cap * torch.tanh((x.float() @ self.weight.T + self.bias) / self.cap)
+
+    register_part("block", "toy_sandwich", SandwichBlock)
+    register_part("block", "toy_parallel", ParallelBlock)
+    register_part("mixer", "toy_latent", LatentMixer)
+    register_part("embedding", "toy_scaled_positional", ScaledPositionalEmbedding)
+    register_part("head", "toy_capped", CappedHead)
+
+    class ToyShapesConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def validate(self):
+            pass
+
+        def model_spec(self):
+            r = self.raw
+            H, V = r["hidden_size"], r["vocab_size"]
+            norm = lambda p: PartSpec("rmsnorm", {"width": H, "eps": r["eps"]}, prefix=p)
+            layers = []
+            for l, (block, mixer_kind) in enumerate(r["layers"]):
+                p = f"layers.{l}."
+                if mixer_kind == "latent":
+                    mixer = PartSpec("toy_latent", {"hidden_size": H, "rank": r["rank"]}, prefix=p + "latent.")
+                else:
+                    mixer = PartSpec("attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 2, "head_dim": 16,
+                                                   "qkv_bias": True, "init_std": 0.2,
+                                                   "position": PartSpec("rope", {"theta": 1e4, "rotary_dim": 16})},
+                                     prefix=p + "attn.")
+                ffn = PartSpec("dense_mlp", {"hidden_size": H, "width": r["width"], "init_std": 0.2}, prefix=p + "mlp.")
+                parts = {"mixer": mixer, "feed_forward": ffn}
+                if block == "toy_sandwich":
+                    parts.update({n: norm(p + n + ".") for n in ("pre_mixer", "post_mixer", "pre_ffn", "post_ffn")})
+                else:
+                    parts["norm"] = norm(p + "norm.")
+                layers.append(LayerSpec(block, parts))
+            embedding = PartSpec("toy_scaled_positional", {"vocab_size": V, "hidden_size": H,
+                                                           "max_positions": r["max_positions"], "scale": r["scale"]},
+                                 prefix="embed.")
+            head = PartSpec("toy_capped", {"vocab_size": V, "hidden_size": H, "cap": r["cap"]}, prefix="head.")
+            return ModelSpec("ToyShapesForCausalLM", H, V, r["max_positions"], layers,
+                             [ScheduleEntry(l) for l in range(len(layers))], embedding, norm("final_norm."), head)
+
+    register_architecture("ToyShapesForCausalLM", ToyShapesConfig)
+    return ToyShapesConfig
+
+
+SHAPES = {"architectures": ["ToyShapesForCausalLM"], "hidden_size": 32, "eps": 1e-5, "width": 48, "rank": 12,
+          "vocab_size": 70, "max_positions": 96, "scale": 3.0, "cap": 30.0,
+          "layers": [["toy_sandwich", "latent"], ["toy_parallel", "attention"], ["toy_sandwich", "attention"],
+                     ["toy_parallel", "latent"]]}
+
+
+def toy_shapes_reference(w, tokens):
+    """The toy model, whole sequence, float64."""
+    w = {k: v.double() for k, v in w.items()}
+    r, T = SHAPES, len(tokens)
+    eps = r["eps"]
+    pos = torch.arange(T)
+    h = w["embed.tokens.weight"][torch.tensor(tokens)] * r["scale"] + w["embed.positions.weight"][pos]
+    for l, (block, mixer_kind) in enumerate(r["layers"]):
+        p = f"layers.{l}."
+
+        def mixer(x):
+            if mixer_kind == "latent":
+                c, q = x @ w[p + "latent.c.weight"].T, x @ w[p + "latent.q.weight"].T
+                rows = [torch.softmax(c[:t + 1] @ q[t] / r["rank"] ** 0.5, 0) @ c[:t + 1] for t in range(T)]
+                return torch.stack(rows) @ w[p + "latent.o.weight"].T
+            a = p + "attn."
+            q = pm.apply_rope((x @ w[a + "q_proj.weight"].T + w[a + "q_proj.bias"]).view(T, 2, 16), pos, 1e4)
+            k = pm.apply_rope((x @ w[a + "k_proj.weight"].T + w[a + "k_proj.bias"]).view(T, 2, 16), pos, 1e4)
+            v = (x @ w[a + "v_proj.weight"].T + w[a + "v_proj.bias"]).view(T, 2, 16)
+            return pm.attention(q, k, v, pos, 0.25).reshape(T, 32) @ w[a + "o_proj.weight"].T
+
+        ffn = lambda x: pm.gated_mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                                     w[p + "mlp.down_proj.weight"])
+        n = lambda name, x: pm.rms_norm(x, w[p + name + ".weight"], eps)
+        if block == "toy_sandwich":
+            h = h + n("post_mixer", mixer(n("pre_mixer", h)))
+            h = h + n("post_ffn", ffn(n("pre_ffn", h)))
+        else:
+            x = n("norm", h)
+            h = h + mixer(x) + ffn(x)
+    logits = pm.rms_norm(h, w["final_norm.weight"], eps) @ w["head.weight"].T + w["head.bias"]
+    return r["cap"] * torch.tanh(logits / r["cap"])
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", ru.FP32_TOL), ("bfloat16", ru.BF16_TOL)])
+def test_other_arrangements_caches_and_ends(tmp_path, dtype, tol):
+    """Blocks with four norms and with one, a mixer whose cache is one array per token (beside attention's two, in a
+    page group of its own), an embedding with a scale and learned positions and a head with a bias and a cap: all
+    registered from here, built, loaded from a folder and stepped four ways without a change to the framework."""
+    ToyShapesConfig = define_toy_shapes()
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.parts import build_model
+    from inferx_amd.weights import random_tensors, write_safetensors
+    model = build_model(ToyShapesConfig(SHAPES).model_spec())
+    assert [type(b).__name__ for b in model.blocks] == ["SandwichBlock", "ParallelBlock"] * 2
+    assert sorted(model.blocks[0].parts) == ["feed_forward", "mixer", "post_ffn", "post_mixer", "pre_ffn", "pre_mixer"]
+    weights = random_tensors(model, 9, dtype)
+    assert "head.bias" in weights and "embed.positions.weight" in weights and "layers.0.post_ffn.weight" in weights
+    write_safetensors(os.path.join(str(tmp_path), "model.safetensors"), weights)
+    with open(os.path.join(str(tmp_path), "config.json"), "w") as f:
+        json.dump(SHAPES, f)
+    prompts = {"a": tiny.random_tokens(50, 70, 1), "b": tiny.random_tokens(19, 70, 2), "c": tiny.random_tokens(34, 70, 3)}
+    expected = {rid: toy_shapes_reference(weights, toks) for rid, toks in prompts.items()}
+    for name, steps in [("whole", ru.whole(prompts)), ("tail", ru.tail_decoded(prompts, 8)),
+                        ("chunked", ru.chunked(prompts)), ("mixed", ru.mixed(prompts, seed=6, max_live=2))]:
+        runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=16, num_pages=9, max_requests=2,
+                                            max_seq_len=96)
+        # two page groups, laid out from the parts' own descriptions: one float32 array of `rank` per token for the
+        # latent mixers, keys and values in the run's type for attention
+        assert runner.group_owners == [[(0, "mixer"), (3, "mixer")], [(1, "mixer"), (2, "mixer")]]
+        assert {n: tuple(t.shape) for n, t in runner.pages[0].items()} == {"latent": (2, 9, 1, 16, 12)}
+        assert runner.pages[0]["latent"].dtype == torch.float32 and runner.pages[1]["v"].shape == (2, 9, 2, 16, 16)
+        assert runner.kv_bytes_per_token() == 2 * 12 * 4 + 2 * 2 * 2 * 16 * runner.pages[1]["k"].element_size()
+        got = ru.replay(runner, steps)
+        ru.compare(got, expected, tol, f"toy shapes {name} {dtype}")
+
+
+def test_a_block_says_which_parts_it_misses_or_does_not_know():
+    define_toy_shapes()
+    from inferx_amd.config import PartSpec
+    from inferx_amd.parts import build_block
+    norm = PartSpec("rmsnorm", {"width": 8, "eps": 1e-5})
+    ffn = PartSpec("dense_mlp", {"hidden_size": 8, "width": 8})
+    with pytest.raises(KeyError, match=r"missing: \['mixer'\]"):
+        build_block("toy_parallel", {"feed_forward": ffn, "norm": norm})
+    with pytest.raises(KeyError, match=r"not known to it: \['post_ffn'\]"):
+        build_block("prenorm", {"feed_forward": ffn, "mixer_norm": norm, "feed_forward_norm": norm, "post_ffn": norm,
+                                "mixer": PartSpec("toy_latent", {"hidden_size": 8, "rank": 4})})
+    with pytest.raises(KeyError, match="no block registered"):
+        build_block("no_such_block", {})

@@ -44,6 +44,25 @@ def test_rope_is_a_complex_rotation_of_half_split_pairs():
     assert f[0] == 1.0 and abs(float(f[1]) - 10000.0 ** (-2.0 / d)) < 1e-7 and float(f[-1]) > 1e-4
 
 
+def test_rope_fixed_vector_worked_by_hand():
+    """d = 4, theta = 10000, position 1: frequencies 1 and 0.01; the row (1, 2, 3, 4) is the pairs (1, 3) at angle 1
+    and (2, 4) at angle 0.01 (pairs (j, j + d/2), as the reference's own host twin pairs them,
+    tests/kernel/mla_test.cc:239-263).  The numbers below were worked out by hand from cos 1 = 0.5403023058681398,
+    sin 1 = 0.8414709848078965, cos 0.01 = 0.9999500004166653, sin 0.01 = 0.009999833334166664.  Interleaved pairs
+    ((1, 2) at angle 1, (3, 4) at angle 0.01) give -1.1426..., a swapped sign gives +3.0647...: both fail."""
+    x = torch.tensor([[[1.0, 2.0, 3.0, 4.0]]], dtype=F64)
+    got = pm.apply_rope(x, torch.tensor([1]), 10000.0)[0, 0]
+    want = torch.tensor([1 * 0.5403023058681398 - 3 * 0.8414709848078965,          # -1.98411064855...
+                         2 * 0.9999500004166653 - 4 * 0.009999833334166664,        #  1.95990066749...
+                         3 * 0.5403023058681398 + 1 * 0.8414709848078965,          #  2.46237790241...
+                         4 * 0.9999500004166653 + 2 * 0.009999833334166664], dtype=F64)  # 4.01979966833...
+    assert torch.allclose(want, torch.tensor([-1.98411064855555, 1.95990066749666, 2.46237790241231,
+                                              4.01979966833500], dtype=F64), atol=1e-12)
+    assert torch.allclose(got, want, atol=1e-6)  # frequency and angle are rounded to float32, as on the device
+    interleaved = 1 * 0.5403023058681398 - 2 * 0.8414709848078965
+    assert abs(float(got[0]) - interleaved) > 0.5
+
+
 def test_attention_without_rotation_or_window_is_library_attention():
     T, heads, kv, d = 9, 6, 2, 8
     q, k, v = rnd(T, heads, d), rnd(T, kv, d, seed=1), rnd(T, kv, d, seed=2)

@@ -97,6 +97,8 @@ def random_config(seed: int) -> dict:
         "tie_word_embeddings": rnd.random() < 0.3, "qkv_bias": rnd.random() < 0.7,
         "_page_size": rnd.choice([16, 16, 32, 64]),
     }
+    if rnd.random() < 0.3:  # the windowed layers named outright
+        cfg["layer_types"] = [rnd.choice(["full_attention", "sliding_attention"]) for _ in range(layers)]
     sparse = [l for l in range(layers)
               if (l + 1) % cfg["decoder_sparse_step"] == 0 and l not in cfg["mlp_only_layers"]]
     if not sparse:  # the architecture wants at least one layer of experts
