@@ -4,6 +4,7 @@ Option names and meanings are the reference server's where it has them
 (src/support/options.cc:47-227: --model, --dtype, --max-num-seqs, --max-model-len,
 --max-num-batched-tokens, --block-size, --num-gpu-blocks-override,
 --kv-cache-memory-bytes, --gpu-memory-utilization, --enforce-eager, --device);
+--dump-logits writes the file format of the reference's scripts/gen_reference_logits.py;
 exit code 0 for --help and 2 for a bad command line (include/inferx/support/options.h:17-22).
 There is no tokenizer and no server: prompts are token ids, output is one JSON
 line per prompt.
@@ -12,6 +13,7 @@ from __future__ import annotations
 
 import argparse
 import json
+import struct
 import sys
 import tempfile
 from typing import List, Optional
@@ -56,6 +58,9 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--logprobs", type=int, default=None, metavar="N",
                     help="report each token's log-probability and those of the N most probable (0 to 20)")
     ap.add_argument("--seed", type=int, default=0, help="fixes the sampling draws")
+    ap.add_argument("--dump-logits", metavar="FILE",
+                    help="also write the float32 logits at every position of every prompt to FILE, one record per "
+                         "prompt: 'IXRL', u32 version 1, u32 tokens, u32 vocab, i32 ids[tokens], f32 logits[tokens * vocab]")
     return ap
 
 
@@ -105,6 +110,14 @@ def main(argv: Optional[List[str]] = None) -> int:
                                 repetition_penalty=args.repetition_penalty, stop_tokens=stop, seed=args.seed,
                                 min_tokens=args.min_tokens, ignore_eos=args.ignore_eos,
                                 want_logprobs=args.logprobs is not None, top_logprobs=args.logprobs or 0)
+        if args.dump_logits:
+            # the reference's logits file (scripts/gen_reference_logits.py:15-23), one record after the other
+            with open(args.dump_logits, "wb") as f:
+                for p in prompts:
+                    logits = engine.prompt_logits(p).numpy().astype("<f4")
+                    f.write(b"IXRL" + struct.pack("<III", 1, logits.shape[0], logits.shape[1]))
+                    f.write(struct.pack(f"<{len(p)}i", *p))
+                    f.write(logits.tobytes())
         results = engine.generate(prompts, params, with_reasons=True)
     except (ConfigError, CheckpointError, ValueError, OSError) as e:
         print(f"inferx-generate: {e}", file=sys.stderr)

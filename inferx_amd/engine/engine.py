@@ -187,6 +187,30 @@ class LLMEngine:
         self.stats.step_seconds += time.perf_counter() - t0
         return self.scheduler.take_completed()
 
+    def prompt_logits(self, prompt_token_ids: Sequence[int]) -> torch.Tensor:
+        """float32 logits [len(prompt), vocab] (on the CPU) at every position of a prompt, run through the step
+        function in portions under the token budget, as a request of its own that holds pages only meanwhile
+        (what the reference's scripts/gen_reference_logits.py:15-23 writes for its own model).  Not to be called
+        while requests are in flight."""
+        if self.scheduler.has_work():
+            raise RuntimeError("prompt_logits runs beside no other request")
+        ids = [int(t) for t in prompt_token_ids]
+        vocab = self.runner.spec.vocab_size
+        if not ids or any(not 0 <= t < vocab for t in ids):
+            raise ValueError("prompt_logits needs a non-empty prompt of token ids inside the vocabulary")
+        rid = ("prompt_logits", self._next_id)
+        self._next_id += 1
+        self.runner.add_request(rid)
+        rows = []
+        try:
+            budget = self.scheduler.max_batch_tokens
+            for at in range(0, len(ids), budget):
+                part = ids[at:at + budget]
+                rows.append(self.runner.run_entries([(rid, part, list(range(len(part))))]).cpu())
+        finally:
+            self.runner.end_request(rid)
+        return torch.cat(rows)
+
     def generate(self, prompts: Sequence[Sequence[int]],
                  params: Union[SamplingParams, Sequence[SamplingParams], None] = None,
                  with_reasons: bool = False):

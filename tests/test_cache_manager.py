@@ -81,6 +81,23 @@ def test_window_rule_exactly():
     assert m.block_row("a", 0)[1] == -1
 
 
+def test_a_windowed_group_may_keep_every_page():
+    # the switch for differential tests: the same window, but passed pages stay until the request ends
+    keep = CacheManager([GroupLayout(5, release_passed=False)], [16], page_size=4, max_requests=1, max_seq_len=64)
+    give = CacheManager([GroupLayout(5)], [16], page_size=4, max_requests=1, max_seq_len=64)
+    for m in (keep, give):
+        m.add("a")
+        m.reserve("a", 40)
+        m.commit("a", 40)
+    assert keep.groups[0].window == 5 and keep.pools[0].used_pages == 10 and -1 not in keep.block_row("a", 0)[:10]
+    # the next query, at position 40, reads keys 36..40: pages 0..8 (tokens 0..35) are dead
+    assert give.pools[0].used_pages == 1 and give.block_row("a", 0)[:9] == [-1] * 9
+    for m in (keep, give):
+        m.free("a")
+        m.check()
+        assert m.pools[0].used_pages == 0
+
+
 def test_reset_keeps_the_slot():
     m = CacheManager([GroupLayout(0)], [4], 4, 2, 16)
     slot = m.add("a")

@@ -260,6 +260,63 @@ def test_command_line(tmp_path):
     assert missing.returncode == 1 and "config.json" in missing.stderr
 
 
+def test_command_line_sizes_the_cache_by_memory_and_dumps_logits(tmp_path):
+    """The command line without --num-gpu-blocks-override (the pool is sized from the memory that is free), with
+    --kv-cache-memory-bytes, and --dump-logits: the reference's logits file, against the plain implementation."""
+    import struct
+    model = tmp_path / "m"
+    tiny.make_folder(tiny.CONFIG_B, 41, str(model), "float32")
+    cfg, weights = tiny.read_folder(str(model))
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 60 + n) for n in (9, 40)]
+    want = [plain_greedy(cfg, weights, p, 4)[0] for p in prompts]
+    base = [sys.executable, os.path.join(ROOT, "bin", "inferx-generate"), str(model), "--dtype", "float32",
+            "--max-tokens", "4", "--max-model-len", "96", "--max-num-seqs", "2", "--max-num-batched-tokens", "16"]
+    for p in prompts:
+        base += ["--prompt-ids", ",".join(map(str, p))]
+    dump = tmp_path / "logits.bin"
+    out = subprocess.run(base + ["--dump-logits", str(dump)], capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    recs = [json.loads(l) for l in out.stdout.strip().splitlines()]
+    assert [r["output_token_ids"] for r in recs] == want
+    raw = dump.read_bytes()
+    at = 0
+    for p in prompts:
+        assert raw[at:at + 4] == b"IXRL"
+        version, tokens, vocab = struct.unpack_from("<III", raw, at + 4)
+        assert (version, tokens, vocab) == (1, len(p), cfg["vocab_size"])
+        assert list(struct.unpack_from(f"<{tokens}i", raw, at + 16)) == p
+        at += 16 + 4 * tokens
+        rows = torch.from_numpy(np.frombuffer(raw, dtype="<f4", count=tokens * vocab, offset=at).copy()).view(tokens, vocab)
+        at += 4 * tokens * vocab
+        expect = pm.forward(cfg, weights, p)
+        assert float((rows.double() - expect).abs().max()) <= ru.FP32_TOL * float(expect.abs().max())
+    assert at == len(raw)
+    # an explicit budget in bytes: 6 pages of 16 tokens are just enough for one sequence of 96
+    page_bytes = 16 * 4 * 2 * 1 * 32 * 4  # tokens x layers x (k, v) x kv heads x head size x float32
+    sized = subprocess.run(base + ["--kv-cache-memory-bytes", str(6 * page_bytes)], capture_output=True, text=True,
+                           timeout=300)
+    assert sized.returncode == 0, sized.stderr
+    assert [json.loads(l)["output_token_ids"] for l in sized.stdout.strip().splitlines()] == want
+    small = subprocess.run(base + ["--kv-cache-memory-bytes", str(5 * page_bytes)], capture_output=True, text=True,
+                           timeout=300)
+    assert small.returncode == 1 and "--kv-cache-memory-bytes" in small.stderr and "--max-model-len" in small.stderr
+
+
+def test_a_prompt_larger_than_the_pool_ends_out_of_memory(tmp_path):
+    """Two pages and a prompt of 40: the request ends out_of_memory at once and the next one runs; the loop does
+    not wait for pages that nobody will give back."""
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_A, 43, str(tmp_path), "float32")
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    engine = LLMEngine(str(tmp_path), "float32", max_num_seqs=2, max_model_len=64, num_gpu_blocks_override=2)
+    big, small = tiny.random_tokens(40, cfg["vocab_size"], 1), tiny.random_tokens(9, cfg["vocab_size"], 2)
+    got = engine.generate([big, small], SamplingParams(max_tokens=3), with_reasons=True)
+    assert got[0] == ([], "out_of_memory")
+    assert got[1] == (plain_greedy(cfg, weights, small, 3)[0], "max_tokens")
+    assert engine.runner.cache.pools[0].used_pages == 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_trace_run_program(tmp_path, dtype):
     """bin/trace_run as a user calls it: steps on standard input, logits in files, `done <step>` per step."""

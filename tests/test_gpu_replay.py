@@ -216,3 +216,29 @@ def test_an_entry_without_tokens_beside_one_with_two(folders, dtype, use_graphs)
     got = ru.replay(runner, steps)
     expected = {k: v for k, v in expected_for(folders, name, dtype).items() if k in prompts}
     ru.compare(got, expected, tol_of(dtype), f"empty entry {dtype} graphs={use_graphs}", ties_for(folders, name, dtype))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_giving_passed_pages_back_changes_no_logit(folders, name, dtype):
+    """The windowed layers' pages with and without the early release: the kernels mask by the window either way,
+    so the logits are the same bit for bit, while the pages held (summed over the steps) differ."""
+    from inferx_amd.engine.runner import ModelRunner
+    prompts = prompts_for(name)
+    steps = ru.chunked(prompts) + ru.mixed({k + "m": v for k, v in prompts.items()}, seed=8, max_live=3)
+    got, held = {}, {}
+    for release in (True, False):
+        runner = ModelRunner.from_directory(folders[(name, dtype)], dtype=dtype, page_size=16, num_pages=24,
+                                            max_requests=4, max_seq_len=128, release_window_pages=release)
+        windowed = [g for g, need in enumerate(runner.group_needs) if need.window > 0]
+        assert windowed and runner.cache.groups[windowed[0]].release_passed is release
+        held[release] = 0
+        rows = {}
+        for step in steps:
+            rows.update(ru.replay(runner, [step]))
+            held[release] += runner.cache.pools[windowed[0]].used_pages
+        got[release] = rows
+    assert held[True] < held[False]
+    assert got[True].keys() == got[False].keys()
+    for key in got[True]:
+        assert torch.equal(got[True][key], got[False][key]), f"{key} differs with the release switched off"
