@@ -16,6 +16,32 @@ import torch
 F64 = torch.float64
 
 
+class Widened:
+    """A checkpoint's tensors in float64, each widened when it is first used (of a model with many experts only
+    those that some token chose).  `forward` takes plain tensors too; handing it one of these keeps the widened
+    tensors from one call to the next."""
+
+    def __init__(self, tensors: Dict[str, torch.Tensor]):
+        self._stored, self._wide = tensors, {}
+
+    def __contains__(self, name: str) -> bool:
+        return name in self._stored
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        if name not in self._wide:
+            self._wide[name] = self._stored[name].to(F64)
+        return self._wide[name]
+
+
+def no_rounding(t: torch.Tensor) -> torch.Tensor:
+    return t
+
+
+def to_bfloat16_and_back(t: torch.Tensor) -> torch.Tensor:
+    """Rounds to bfloat16 (nearest even) and widens again: what a tensor stored in bfloat16 holds."""
+    return t.to(torch.bfloat16).to(F64)
+
+
 # --------------------------------------------------------------------------
 def rms_norm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     """y_i = x_i * rsqrt(sum(x^2)/H + eps) * w_i
@@ -73,18 +99,22 @@ def silu(g: torch.Tensor) -> torch.Tensor:
     return g / (1.0 + torch.exp(-g))
 
 
-def gated_mlp(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
-    """y = (silu(x Wg^T) * (x Wu^T)) Wd^T.   src/model/qwen2.cc:1042-1048; weights [out, in], gemm.h:51-57."""
-    return (silu(x @ w_gate.T) * (x @ w_up.T)) @ w_down.T
+def gated_mlp(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down: torch.Tensor,
+              rnd=no_rounding) -> torch.Tensor:
+    """y = (silu(x Wg^T) * (x Wu^T)) Wd^T.   src/model/qwen2.cc:1042-1048; weights [out, in], gemm.h:51-57.
+    `rnd`: what a stored activation goes through (the reference stores the two products, the activation and the
+    result in bfloat16; the sums themselves are 32-bit)."""
+    return rnd(rnd(silu(rnd(x @ w_gate.T)) * rnd(x @ w_up.T)) @ w_down.T)
 
 
 def route(x: torch.Tensor, w_router: torch.Tensor, top_k: int, renormalize: bool,
-          scale: float = 1.0) -> Tuple[torch.Tensor, torch.Tensor]:
+          scale: float = 1.0, rnd=no_rounding) -> Tuple[torch.Tensor, torch.Tensor]:
     """p = softmax(x Wr^T) over all experts; k rounds of argmax with strict '>' (lowest index wins a tie),
     chosen weight = p_e, chosen expert masked to -inf; optional division by the sum of the chosen; times scale.
     src/backends/cuda/ops/moe.cu:36-127 (RouteTopKKernel); src/model/moe_ffn.cc:200-221.
-    Returns weights [T, k] and experts [T, k], slots in descending score."""
-    z = x @ w_router.T
+    Returns weights [T, k] and experts [T, k], slots in descending score.  `rnd`: the reference stores the scores
+    z in bfloat16 (moe_ffn.cc:200-207) before the 32-bit softmax."""
+    z = rnd(x @ w_router.T)
     T, E = z.shape
     weights = torch.zeros(T, top_k, dtype=x.dtype)
     experts = torch.zeros(T, top_k, dtype=torch.int64)
@@ -119,24 +149,30 @@ def router_margin(x: torch.Tensor, w_router: torch.Tensor, top_k: int) -> torch.
 
 
 def moe_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, num_experts: int, top_k: int,
-              renormalize: bool, shared_width: int) -> torch.Tensor:
+              renormalize: bool, shared_width: int, rnd=no_rounding) -> torch.Tensor:
     """Every chosen expert applied per token and summed in slot order, plus the sigmoid-gated shared expert:
     out_t = sum_slot w_{t,slot} * MLP_e(x_t)  +  sigmoid(x_t . Wsg) * MLP_shared(x_t).
     src/model/moe_ffn.cc:158-367 (route, experts, combine :305-306, shared :308-351);
     moe.cu:237-255 (CombineRowsKernel), :275-287 (AddSharedExpertKernel: 1/(1+exp(-g)))."""
-    weights, experts = route(x, w[prefix + "gate.weight"], top_k, renormalize)
+    weights, experts = route(x, w[prefix + "gate.weight"], top_k, renormalize, rnd=rnd)
+    # every expert is applied once, to the tokens that chose it (rows of a product do not depend on each other) ...
+    applied = {}
+    for e in sorted(set(experts.flatten().tolist())):
+        p = f"{prefix}experts.{e}."
+        tokens = torch.nonzero((experts == e).any(dim=1)).flatten()
+        y = gated_mlp(x[tokens], w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"], rnd)
+        applied[e] = dict(zip(tokens.tolist(), y))
+    # ... and each token sums its experts' results in slot order
     out = torch.zeros_like(x)
     for t in range(x.shape[0]):
         for slot in range(top_k):
-            e = int(experts[t, slot])
-            p = f"{prefix}experts.{e}."
-            out[t] += weights[t, slot] * gated_mlp(x[t:t + 1], w[p + "gate_proj.weight"], w[p + "up_proj.weight"],
-                                                   w[p + "down_proj.weight"])[0]
+            out[t] += weights[t, slot] * applied[int(experts[t, slot])][t]
+    out = rnd(out)
     if shared_width > 0:
         p = prefix + "shared_expert."
-        shared = gated_mlp(x, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
-        gate = 1.0 / (1.0 + torch.exp(-(x @ w[prefix + "shared_expert_gate.weight"].T)))  # [T, 1]
-        out = out + gate * shared
+        shared = gated_mlp(x, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"], rnd)
+        gate = 1.0 / (1.0 + torch.exp(-rnd(x @ w[prefix + "shared_expert_gate.weight"].T)))  # [T, 1]
+        out = rnd(out + gate * shared)
     return out
 
 
@@ -164,13 +200,23 @@ def window_of_layer(cfg: dict, layer: int) -> int:
 def forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequence[int],
             positions: Optional[Sequence[int]] = None,
             schedule: Optional[List[Tuple[int, Optional[int]]]] = None,
-            margins: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+            margins: Optional[List[torch.Tensor]] = None, rnd=no_rounding,
+            router_scores: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence.  Layer order and the place of every norm and residual:
     src/model/qwen2.cc:902-1066 (embed :902; input norm :912; qkv + bias :920-923; rope :925-926; attention
     :1021-1023; o_proj + residual :1026-1030; post norm :1036; feed-forward :1042-1048; residual :1051; final norm
     and head :1059-1066).  `schedule`: (layer, cache_from) per execution, default each layer once.
-    `margins`: if a list, the router margin per token of every sparse layer run is appended to it."""
-    w = {k: v.to(F64) for k, v in weights.items()}
+    `margins`: if a list, the router margin per token of every sparse layer run is appended to it; `router_scores`
+    likewise takes the router's scores [T, experts] of every sparse layer.
+
+    `rnd` is what every stored activation goes through.  With `to_bfloat16_and_back` this is the reference's
+    bfloat16 model: every tensor it keeps between kernels is bfloat16 (norm outputs layers.cu:50-76; the q/k/v
+    product, then again after the bias :485-510; rotated q and k :80-115; attention output :256-318; the output
+    product and the residual sum :542-548; feed-forward activations; the router's scores, moe_ffn.cc:200-207) while
+    every sum inside a kernel is 32-bit.  The difference between that model and this one in float64 is the error
+    that bfloat16 storage alone brings: the measure for what a bfloat16 engine may differ by (the reference derives
+    its own tolerance so, scripts/gen_reference_logits.py:51-55).  The logits themselves are left unrounded."""
+    w = weights if isinstance(weights, Widened) else Widened(weights)
     H = cfg["hidden_size"]
     heads = cfg["num_attention_heads"]
     kv_heads = cfg.get("num_key_value_heads", heads)
@@ -180,38 +226,40 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequence[int
     T = len(token_ids)
     pos = torch.arange(T) if positions is None else torch.tensor(list(positions))
     scale = 1.0 / math.sqrt(d)  # qwen2.cc:890
-    h = w["model.embed_tokens.weight"][torch.tensor(list(token_ids))]  # layers.cu:465-481
+    h = rnd(w["model.embed_tokens.weight"][torch.tensor(list(token_ids))])  # layers.cu:465-481
     if schedule is None:
         schedule = [(l, None) for l in range(cfg["num_hidden_layers"])]
     kept: List[Tuple[torch.Tensor, torch.Tensor]] = []
     for layer, cache_from in schedule:
         p = f"model.layers.{layer}."
-        x = rms_norm(h, w[p + "input_layernorm.weight"], eps)
+        x = rnd(rms_norm(h, w[p + "input_layernorm.weight"], eps))
         a = p + "self_attn."
-        q = x @ w[a + "q_proj.weight"].T
-        k = x @ w[a + "k_proj.weight"].T
-        v = x @ w[a + "v_proj.weight"].T
+        q = rnd(x @ w[a + "q_proj.weight"].T)
+        k = rnd(x @ w[a + "k_proj.weight"].T)
+        v = rnd(x @ w[a + "v_proj.weight"].T)
         if a + "q_proj.bias" in w:  # SplitQkvKernel adds the bias after the product, layers.cu:485-510
-            q, k, v = q + w[a + "q_proj.bias"], k + w[a + "k_proj.bias"], v + w[a + "v_proj.bias"]
-        q = apply_rope(q.view(T, heads, d), pos, theta)
-        k = apply_rope(k.view(T, kv_heads, d), pos, theta)  # rotated keys are what is cached, qwen2.cc:928-969
+            q, k, v = rnd(q + w[a + "q_proj.bias"]), rnd(k + w[a + "k_proj.bias"]), rnd(v + w[a + "v_proj.bias"])
+        q = rnd(apply_rope(q.view(T, heads, d), pos, theta))
+        k = rnd(apply_rope(k.view(T, kv_heads, d), pos, theta))  # rotated keys are what is cached, qwen2.cc:928-969
         v = v.view(T, kv_heads, d)
         if cache_from is not None:
             k, v = kept[cache_from]
         kept.append((k, v))
-        att = attention(q, k, v, pos, scale, window_of_layer(cfg, layer))
-        h = h + att.reshape(T, heads * d) @ w[a + "o_proj.weight"].T
-        x = rms_norm(h, w[p + "post_attention_layernorm.weight"], eps)
+        att = rnd(attention(q, k, v, pos, scale, window_of_layer(cfg, layer)))
+        h = rnd(h + rnd(att.reshape(T, heads * d) @ w[a + "o_proj.weight"].T))
+        x = rnd(rms_norm(h, w[p + "post_attention_layernorm.weight"], eps))
         m = p + "mlp."
         if is_moe_layer(cfg, layer):
             if margins is not None:
                 margins.append(router_margin(x, w[m + "gate.weight"], cfg["num_experts_per_tok"]))
+            if router_scores is not None:
+                router_scores.append(rnd(x @ w[m + "gate.weight"].T))
             f = moe_block(x, w, m, cfg["num_experts"], cfg["num_experts_per_tok"],
-                          bool(cfg.get("norm_topk_prob", False)), cfg.get("shared_expert_intermediate_size", 0))
+                          bool(cfg.get("norm_topk_prob", False)), cfg.get("shared_expert_intermediate_size", 0), rnd)
         else:
-            f = gated_mlp(x, w[m + "gate_proj.weight"], w[m + "up_proj.weight"], w[m + "down_proj.weight"])
-        h = h + f
-    x = rms_norm(h, w["model.norm.weight"], eps)
+            f = gated_mlp(x, w[m + "gate_proj.weight"], w[m + "up_proj.weight"], w[m + "down_proj.weight"], rnd)
+        h = rnd(h + f)
+    x = rnd(rms_norm(h, w["model.norm.weight"], eps))
     head = w["model.embed_tokens.weight"] if cfg.get("tie_word_embeddings", False) else w["lm_head.weight"]
     return x @ head.T
 

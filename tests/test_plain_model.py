@@ -242,3 +242,18 @@ def test_norms_and_residuals_sit_where_the_reference_puts_them(model_b):
                            w[p + "mlp.down_proj.weight"].double())
     want = pm.rms_norm(h2, w["model.norm.weight"].double(), cfg["rms_norm_eps"]) @ w["model.embed_tokens.weight"].double().T
     assert torch.allclose(pm.forward(one, w, toks[:1]), want, atol=1e-12)
+
+
+def test_bfloat16_storage_mode(model_b):
+    """The plain implementation with every stored activation rounded to bfloat16: the same model up to rounding
+    (a few parts in a thousand of the largest logit), not bit-equal, and untouched when nothing is rounded."""
+    cfg, w = model_b
+    toks = tiny.random_tokens(24, cfg["vocab_size"], 9)
+    base = pm.forward(cfg, w, toks)
+    assert torch.equal(pm.forward(cfg, w, toks, rnd=pm.no_rounding), base)
+    scores = []
+    stored = pm.forward(cfg, w, toks, rnd=pm.to_bfloat16_and_back, router_scores=scores)
+    moved = float((stored - base).abs().max()) / float(base.abs().max())
+    assert 1e-5 < moved < 3e-2
+    assert len(scores) == 2 and scores[0].shape == (24, cfg["num_experts"])  # config B has two sparse layers
+    assert torch.equal(scores[0], pm.to_bfloat16_and_back(scores[0]))       # the scores are stored rounded too
