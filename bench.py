@@ -4,9 +4,12 @@
 
 A step is one decode step of the whole batch through the engine (scheduler,
 batch layout, upload, every kernel, greedy choice of the next tokens).  Prints ONE
-JSON line: decoded tokens a second at the default batch, the prefill of one
-2,048-token prompt, the decode step's HBM roofline fraction, and decode at
-batch 1 and 64.  One GPU only.
+JSON line: decoded tokens a second at the default batch (with the smallest and the
+median time of single steps), the prefill of one 2,048-token prompt, the decode
+step's HBM roofline fraction, and decode at batch 1 and 64.  Fractions are given
+against the published peaks and against what two probe kernels measure on this
+machine at the start of the run (a pure read of 4 GiB, pure matrix-core
+products).  One GPU only.
 
 Two further workloads at the Qwen2-57B-A14B shape, each with a JSON line of the same form:
 
@@ -267,6 +270,9 @@ def main() -> int:
     cfg = config_from_dict(raw)
     rt = Runtime(args.dtype, "cuda:0")
     elt = 2 if args.dtype == "bfloat16" else 4
+    from inferx_amd import ops
+    ceilings = ops.measured_ceilings("cuda:0")  # before the weights take the memory
+    log(f"measured on this machine: {ceilings}")
     points = [int(p) for p in args.points.split(",") if p]
     max_batch = max([args.batch] + points)
     log(f"drawing random weights on the device ({args.layers} layers, {args.dtype})")
@@ -284,12 +290,14 @@ def main() -> int:
     def prompt():
         return torch.randint(0, cfg.vocab_size, (PROMPT,), generator=gen).tolist()
 
-    def run_decode(batch, steps, warmup):
+    def run_decode(batch, steps, warmup, single=0):
         """`batch` requests with prompts of PROMPT tokens through the engine (scheduler, step function, sampler):
-        first their prompts, then `warmup` untimed and `steps` timed decode steps of the whole batch."""
+        first their prompts, then `warmup` untimed and `steps` timed decode steps of the whole batch; then `single`
+        more steps, each timed on its own (the device is waited for after every one of them, so they are a little
+        slower than steps that follow each other).  Returns the time of the `steps` and the list of single times."""
         engine = LLMEngine("", runner=runner, max_num_seqs=batch, max_model_len=CONTEXT, max_num_batched_tokens=PROMPT)
         # (requests decode while the later prompts are still being read: room for those tokens too)
-        params = SamplingParams(max_tokens=warmup + steps + 3 * batch + 16, ignore_eos=True)
+        params = SamplingParams(max_tokens=warmup + steps + single + 3 * batch + 16, ignore_eos=True)
         ids = [engine.add_request(prompt(), params) for _ in range(batch)]
         while any(engine.scheduler.sequence(i).generated() == 0 for i in ids):  # the prompts, one a step
             engine.step()
@@ -303,12 +311,18 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         assert engine.stats.tokens_out - before == batch * steps, "a timed step was not a decode step of the whole batch"
+        singles = []
+        for _ in range(single):
+            t = time.perf_counter()
+            engine.step()
+            torch.cuda.synchronize()
+            singles.append(time.perf_counter() - t)
         for i in ids:
             engine.cancel(i)
         while engine.has_unfinished():
             engine.step()
         assert runner.cache.pools[0].used_pages == 0
-        return dt
+        return dt, singles
 
     # ---- prefill of one 2,048-token prompt ---------------------------------
     prefill = None
@@ -327,12 +341,15 @@ def main() -> int:
         sec = min(times[1:])
         flops = prefill_flops(cfg, PROMPT)
         prefill = {"value": round(PROMPT / sec, 1), "tokens": PROMPT, "ms": round(sec * 1e3, 3),
-                   "frac": round(flops / sec / (PEAK_TFLOPS["bf16" if elt == 2 else "fp32"] * 1e12), 5)}
+                   "frac": round(flops / sec / (PEAK_TFLOPS["bf16" if elt == 2 else "fp32"] * 1e12), 5),
+                   "tflops": round(flops / sec / 1e12, 1),
+                   "frac_measured": round(flops / sec / (ceilings["mfma_bf16_tflops"] * 1e12), 5) if elt == 2 else None}
         log(f"prefill {prefill}")
 
     # ---- decode ----------------------------------------------------------------
     log(f"decode at batch {args.batch}")
-    dt = run_decode(args.batch, args.steps, args.warmup)
+    dt, singles = run_decode(args.batch, args.steps, args.warmup, single=args.steps)
+    singles.sort()
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     context = PROMPT + args.warmup + args.steps // 2
@@ -341,13 +358,15 @@ def main() -> int:
     for b in points:
         log(f"decode at batch {b}")
         steps = max(8, args.steps // 2)
-        d = run_decode(b, steps, max(2, args.warmup // 2))
+        d, _ = run_decode(b, steps, max(2, args.warmup // 2))
         pts[f"decode_b{b}"] = round(b * steps / d, 1)
 
     line = {
         "metric": f"Qwen1.5-MoE-A2.7B decode tok/s @ batch {args.batch} (2048-token prompts)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": round(ms, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": round(ms, 3),
+        "step_ms": {"min": round(singles[0] * 1e3, 3), "median": round(singles[len(singles) // 2] * 1e3, 3)},
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if elt == 2 else "fp32", "data": "synthetic: seeded random weights and token ids",
         "config": {
             "model": "Qwen1.5-MoE-A2.7B shape", "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT,
@@ -359,7 +378,8 @@ def main() -> int:
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(gbs / PEAK_HBM_GBS, 5)},
+                     "frac": round(gbs / PEAK_HBM_GBS, 5), "frac_measured": round(gbs / ceilings["hbm_read_gbs"], 5)},
+        "ceilings": ceilings,
         "points": pts,
     }
     print(json.dumps(line), flush=True)

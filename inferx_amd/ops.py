@@ -622,3 +622,36 @@ def apply_penalties(logits: torch.Tensor, hist_begin: torch.Tensor, hist_ids: to
         _need(t.dtype == torch.float32 and t.numel() >= R, "penalties must be float32 [rows]")
     _call("ix_apply_penalties", _ptr(logits), _ptr(hist_begin), _ptr(hist_ids), _ptr(hist_counts), _ptr(presence),
           _ptr(frequency), _ptr(repetition), _ptr(mask_begin), _ptr(mask_ids), _i64(R), _i64(V), _stream())
+
+
+def measured_ceilings(device=None, read_bytes: int = 4 << 30) -> dict:
+    """What this machine gives a kernel that only reads memory (GB/s, over a buffer far larger than any cache)
+    and one that only issues bfloat16 matrix-core products (TFLOP/s): the measured ceilings that results are
+    priced against beside the published peaks.  Takes a few tens of milliseconds and `read_bytes` of memory."""
+    device = torch.device(device or "cuda:0")
+    cus = torch.cuda.get_device_properties(device).multi_processor_count
+    buf = torch.empty(read_bytes // 4, dtype=torch.int32, device=device)
+    buf.fill_(1)
+    out = torch.zeros(1024, dtype=torch.int32, device=device)
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    best_read = 0.0
+    for blocks in (cus * 8, cus * 16, cus * 32):
+        _call("ix_probe_read", _ptr(buf), _i64(read_bytes), _ptr(out), _i32(blocks), _i32(1), _stream())  # warm
+        start.record()
+        _call("ix_probe_read", _ptr(buf), _i64(read_bytes), _ptr(out), _i32(blocks), _i32(4), _stream())
+        stop.record()
+        stop.synchronize()
+        best_read = max(best_read, 4 * read_bytes / (start.elapsed_time(stop) * 1e-3) / 1e9)
+    del buf
+    sink = torch.zeros(1, dtype=torch.float32, device=device)
+    flops = ctypes.c_double(0.0)
+    best_mfma = 0.0
+    for waves_per_simd in (2, 4):
+        blocks, iters = cus * waves_per_simd, 100000
+        _call("ix_probe_mfma", _i32(blocks), _i32(200), _ptr(sink), ctypes.byref(flops), _stream())  # warm
+        start.record()
+        _call("ix_probe_mfma", _i32(blocks), _i32(iters), _ptr(sink), ctypes.byref(flops), _stream())
+        stop.record()
+        stop.synchronize()
+        best_mfma = max(best_mfma, flops.value / (start.elapsed_time(stop) * 1e-3) / 1e12)
+    return {"hbm_read_gbs": round(best_read, 1), "mfma_bf16_tflops": round(best_mfma, 1)}
