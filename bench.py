@@ -16,6 +16,12 @@ Two further workloads at the Qwen2-57B-A14B shape, each with a JSON line of the 
     python bench.py --workload mixed [--layers L]   # 32 decodes at a context of 4,096 beside 2 prompt portions of 512
     python bench.py --workload long [--layers L]    # batch 8, prompts of 16,384 to 32,000 tokens in portions of
                                                     # 2,048, then --steps decode steps (default there: 256)
+
+and a small mixed step at the Qwen1.5-MoE-A2.7B shape, which is launched kernel by kernel (only steps of one token
+per request are replayed from HIP graphs): under `rocprofv3 --kernel-trace` it shows whether such steps wait for
+the host:
+
+    python bench.py --workload mixed-small          # 8 decodes at a context of 2,048 beside 1 prompt portion of 64
 """
 from __future__ import annotations
 
@@ -114,15 +120,17 @@ def run_57b(args) -> int:
     from inferx_amd.sampling import SamplingParams
     from inferx_amd.weights import random_tensors
 
-    layers = args.layers or SHAPE_57B["num_hidden_layers"]
-    raw = dict(SHAPE_57B)
+    shape = SHAPE if args.workload == "mixed-small" else SHAPE_57B
+    shape_name = "Qwen1.5-MoE-A2.7B shape" if args.workload == "mixed-small" else "Qwen2-57B-A14B shape"
+    layers = args.layers or shape["num_hidden_layers"]
+    raw = dict(shape)
     raw["num_hidden_layers"] = layers
     cfg = config_from_dict(raw)
     rt = Runtime(args.dtype, "cuda:0")
     elt = 2 if args.dtype == "bfloat16" else 4
     peak = PEAK_TFLOPS["bf16" if elt == 2 else "fp32"] * 1e12
-    mixed = args.workload == "mixed"
-    context = 8192 if mixed else 32768
+    mixed = args.workload in ("mixed", "mixed-small")
+    context = {"mixed": 8192, "mixed-small": 4096, "long": 32768}[args.workload]
     log(f"drawing random weights on the device ({layers} layers, {args.dtype})")
     t0 = time.time()
     model = build_model(cfg.model_spec())
@@ -132,13 +140,14 @@ def run_57b(args) -> int:
     base = {"metric": None, "value": None, "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
             "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
             "dtype": "bf16" if elt == 2 else "fp32", "data": "synthetic: seeded random weights and token ids"}
-    sizes = {"layers": layers, "layers_of_shape": SHAPE_57B["num_hidden_layers"], "hidden": cfg.hidden_size,
+    sizes = {"layers": layers, "layers_of_shape": shape["num_hidden_layers"], "hidden": cfg.hidden_size,
              "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
              "experts": cfg.num_experts, "top_k": cfg.num_experts_per_tok, "moe_intermediate": cfg.moe_intermediate_size,
              "shared_intermediate": cfg.shared_expert_intermediate_size, "vocab": cfg.vocab_size, "page_size": PAGE}
 
     if mixed:
-        n_dec, dec_ctx, n_pre, portion, pre_ctx = 32, 4096, 2, 512, 2048
+        n_dec, dec_ctx, n_pre, portion, pre_ctx = (32, 4096, 2, 512, 2048) if args.workload == "mixed" else \
+            (8, 2048, 1, 64, 0)
         pages = (n_dec * context + n_pre * context) // PAGE
         runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=n_dec + n_pre,
                              max_seq_len=context, model=model)
@@ -150,7 +159,7 @@ def run_57b(args) -> int:
             for s in range(0, dec_ctx if r in dec else pre_ctx, 2048):
                 runner.run_entries([(r, rnd(2048), [])])
         total = args.warmup + args.steps
-        assert pre_ctx + total * portion <= context and dec_ctx + total <= context, "fewer steps: the context is 8,192"
+        assert pre_ctx + total * portion <= context and dec_ctx + total <= context, f"fewer steps: the context is {context}"
         entries = lambda: [(r, rnd(1), [0]) for r in dec] + [(r, rnd(portion), []) for r in pre]
         for _ in range(args.warmup):
             runner.run_entries(entries())
@@ -167,10 +176,10 @@ def run_57b(args) -> int:
         flops = linear_flops(cfg, tokens, n_dec) + n_dec * attention_flops(cfg, 1, dec_ctx + mid) \
             + n_pre * attention_flops(cfg, portion, pre_ctx + mid * portion)
         gbs = step_bytes(cfg, tokens, cache_tokens, elt) / dt / 1e9
-        line = dict(base, metric="Qwen2-57B-A14B shape, mixed step (32 decodes at context 4096 beside 2 prompt "
-                                 "portions of 512) through the step function, tokens/s",
+        line = dict(base, metric=f"{shape_name}, mixed step ({n_dec} decodes at context {dec_ctx} beside {n_pre} prompt "
+                                 f"portions of {portion}) through the step function, tokens/s",
                     value=round(tokens / dt, 1), ms_per_step=round(dt * 1e3, 3),
-                    config=dict(sizes, model="Qwen2-57B-A14B shape", global_batch=n_dec + n_pre, seq_len=context,
+                    config=dict(sizes, model=shape_name, global_batch=n_dec + n_pre, seq_len=context,
                                 tokens_per_step=tokens, parallelism="single GPU"),
                     prefill=None,
                     compute={"flops_per_step": flops, "frac": round(flops / dt / peak, 5)},
@@ -237,8 +246,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (4; 2 for mixed)")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the configuration has (sizes of a layer are never reduced)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long"],
-                    help="decode: the Qwen1.5-MoE-A2.7B shape (default); mixed, long: the Qwen2-57B-A14B shape")
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long", "mixed-small"],
+                    help="decode, mixed-small: the Qwen1.5-MoE-A2.7B shape (decode is the default); mixed, long: the "
+                         "Qwen2-57B-A14B shape")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
@@ -248,9 +258,9 @@ def main() -> int:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
         return 2
     if args.steps is None:
-        args.steps = {"decode": 32, "mixed": 8, "long": 256}[args.workload]
+        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24}[args.workload]
     if args.warmup is None:
-        args.warmup = {"decode": 4, "mixed": 2, "long": 4}[args.workload]
+        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4}[args.workload]
     if args.workload != "decode":
         return run_57b(args)
     if args.layers is None:

@@ -164,6 +164,19 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
 #pragma unroll
       for (int i = 0; i < 3; ++i) pg[i] = pg_next[i];
     }
+    // Values of keys that no query of the tile may read (past the tile's last key in the same page, or on a page
+    // that the window has passed, read from wherever the table's filler points) are made zero: their probability
+    // is zero, but zero times whatever an earlier request left there need not be.  Only rounds at the edges.
+    if (kb + ATTN_KEYS_PER_ITER > hi || kb < lo) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int key = (min(kb + 8 * g, hi - 1) & ~7) + j;
+        if (key >= hi || key < lo) {
+#pragma unroll
+          for (int b = 0; b < NB; ++b) vf[b][j] = (__bf16)0.f;
+        }
+      }
+    }
 #pragma unroll
     for (int t = 0; t < QT; ++t) {
       if (QT > 1 && (16 * t >= rows || kb > pos0 + 16 * t + 15)) continue;  // no query of this block reads these keys

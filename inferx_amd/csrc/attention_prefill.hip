@@ -102,11 +102,11 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
   // and V_PER of value rows; piece c of a group is (key c / 2NB, piece c % 2NB of its row) for keys and
   // (row c / 2, keys 8 (c % 2) ..) for values, so that neighbouring threads read neighbouring memory.
   // Keys past the tile's last one, and pages that a window has passed (-1 in the table), are read from some page of
-  // the pool and masked where they are used: memory of the pool is finite everywhere (it starts as zeros and only
-  // ever holds what was appended), so a masked value times a probability of zero is zero.
+  // the pool and masked where they are used; their values are written to LDS as zeros (see stage), because a
+  // probability of zero times whatever an earlier request left in a page need not be zero.
   constexpr int GROUPS = PF_KEYS / 16, GROUP_CHUNKS = 32 * NB;
   __builtin_assume(tid < 256);
-  int k_grp[K_PER], k_src[K_PER], k_dst[K_PER], v_grp[V_PER], v_src[V_PER], v_dst[V_PER];
+  int k_grp[K_PER], k_src[K_PER], k_dst[K_PER], v_grp[V_PER], v_src[V_PER], v_dst[V_PER], v_key[V_PER];
 #pragma unroll
   for (int i = 0; i < K_PER; ++i) {
     const int c = min(tid + 256 * i, K_CHUNKS - 1), w = c % GROUP_CHUNKS;
@@ -125,6 +125,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
     const int half = (w >> 4) & 1, dd = (w & 15) | ((w >> 5) << 4);
     v_grp[i] = c / GROUP_CHUNKS;
     v_src[i] = dd * page_size + half * 8;
+    v_key[i] = 16 * (c / GROUP_CHUNKS) + 8 * half;  // the piece's first key within the tile
     v_dst[i] = dd * VS + (((2 * (c / GROUP_CHUNKS) + half) ^ ((dd >> 1) & 7)) << 3);
   }
   const int64_t page_elems = static_cast<int64_t>(kv_heads) * page_size * D;
@@ -165,12 +166,23 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
     for (int i = 0; i < V_PER; ++i) vreg[i] = *reinterpret_cast<const bf16x8*>(v_head + pick(v_at, v_grp[i]) + v_src[i]);
   };
   auto key_place = [&](int row, int d0) { return row * KS + ((d0 >> 3) ^ ((row & 3) | (((row >> 3) & 3) << 2))) * 8; };
-  auto stage = [&](int buf) {
+  // `tile_kb`: the first key of the tile that the registers hold.  At the tile's edges (uniform) the values of keys
+  // that no query may read become zeros on their way into LDS.
+  auto stage = [&](int buf, int tile_kb) {
     __bf16* ks = k_tiles[buf];
     __bf16* vs = v_tiles[buf];
 #pragma unroll
     for (int i = 0; i < K_PER; ++i)
       if (tid + 256 * i < K_CHUNKS) *reinterpret_cast<bf16x8*>(ks + k_dst[i]) = kreg[i];
+    if (tile_kb + PF_KEYS > hi_tile || tile_kb < lo) {
+#pragma unroll
+      for (int i = 0; i < V_PER; ++i)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int key = tile_kb + v_key[i] + j;
+          if (key >= hi_tile || key < lo) vreg[i][j] = (__bf16)0.f;
+        }
+    }
 #pragma unroll
     for (int i = 0; i < V_PER; ++i)
       if (tid + 256 * i < V_CHUNKS) *reinterpret_cast<bf16x8*>(vs + v_dst[i]) = vreg[i];
@@ -183,7 +195,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
   locate(kb0);
   fetch();
   ask_pages(kb0 + PF_KEYS);
-  stage(0);
+  stage(0, kb0);
   if (kb0 + PF_KEYS < hi) {
     locate(kb0 + PF_KEYS);
     fetch();
@@ -196,7 +208,7 @@ attn_prefill_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_c
     // The registers hold tile kb + 64 (loaded while tile kb - 64 was multiplied): it goes into the buffer that
     // the previous round read, which every wavefront has left (the barrier below); then tile kb + 128 is asked for.
     if (kb + PF_KEYS < hi) {
-      stage(buf ^ 1);
+      stage(buf ^ 1, kb + PF_KEYS);
       if (kb + 2 * PF_KEYS < hi) {
         locate(kb + 2 * PF_KEYS);
         fetch();

@@ -250,3 +250,85 @@ def test_attention_finds_one_far_key():
             want = attention_reference(p, [L], [1], heads, heads, d ** -0.5, 0)
             close(out, want, TOL[torch.bfloat16], f"far key {far}")
             assert float((out[0].float().cpu() - v[far].float()).abs().max()) < 0.05 * float(v[far].abs().max())
+
+
+def poison_what_no_query_may_read(p, seq_lens, q_lens, page_size, window):
+    """Everything in the pool that the requests do not own becomes NaN, as an earlier request that went wrong
+    might have left it: unused pages, the part of each request's last page past its last token, page 0 (which is
+    freed for it and read as a filler), and, with a window, the pages that all of a request's queries have passed,
+    whose table entries become -1 as the cache manager leaves them."""
+    table = p["table"].cpu().clone()
+    k_cache, v_cache = p["k_cache"], p["v_cache"]
+    pages = k_cache.shape[0]
+    used = set(int(x) for x in table.flatten() if x >= 0)
+    spare = [i for i in range(pages) if i not in used]
+    if 0 in used:  # move page 0's content elsewhere so that page 0 is nobody's
+        to = spare.pop()
+        k_cache[to], v_cache[to] = k_cache[0].clone(), v_cache[0].clone()
+        table[table == 0] = to
+    nan = float("nan")
+    for s, (L, n) in enumerate(zip(seq_lens, q_lens)):
+        last = (L - 1) // page_size
+        tail = L - last * page_size
+        pg = int(table[s, last])
+        k_cache[pg, :, tail:, :] = nan
+        v_cache[pg, :, :, tail:] = nan
+        if window > 0:
+            first_read = max(0, (L - n) + 1 - window)  # the lowest key that the request's first query reads
+            for j in range(first_read // page_size):
+                pg = int(table[s, j])
+                k_cache[pg], v_cache[pg] = nan, nan
+                table[s, j] = -1
+    owned = set(int(x) for x in table.flatten() if x >= 0)
+    for i in range(pages):
+        if i not in owned:
+            k_cache[i], v_cache[i] = nan, nan
+    p["table"] = table.to(DEV)
+
+
+NAN_CASES = [
+    # seq_lens, q_lens, heads, kv_heads, d, page, window
+    ([700, 33, 1], [1, 1, 1], 8, 8, 128, 16, 0),
+    ([1000, 999, 70], [1, 3, 2], 8, 2, 64, 64, 100),       # window: passed pages are -1 and hold NaN
+    ([513, 260, 45], [200, 17, 45], 4, 1, 64, 32, 0),      # portions whose last page is partly filled
+    ([900, 450], [500, 450], 2, 2, 96, 32, 70),
+]
+
+
+@pytest.mark.parametrize("case", NAN_CASES)
+def test_attention_kernels_ignore_what_other_requests_left_in_the_pool(case):
+    """A request that once wrote NaN into its keys or values leaves them in its freed pages.  Whoever gets such a
+    page, or reads page 0 as a filler for a page the window has passed, must not be touched by them: a masked
+    key's probability is zero, and zero times NaN is NaN unless the value is masked too."""
+    from inferx_amd import ops
+    seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    scale = d ** -0.5
+    p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, torch.bfloat16, seed=12)
+    want = attention_reference(p, seq_lens, q_lens, heads, kv_heads, scale, window)
+    poison_what_no_query_may_read(p, seq_lens, q_lens, page, window)
+    T = p["q"].shape[0]
+    runs = []
+    for n_splits in (1, 4):
+        work = torch.empty(T * heads * n_splits * (d + 2), dtype=torch.float32, device=DEV)
+        for prefetch in (False, True):
+            out = torch.full_like(p["q"], float("nan"))
+            ops.attention_mfma(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for(q_lens), p["positions"], out,
+                               n_splits, work, scale, window, 16, prefetch)
+            runs.append((f"wavefront-level, {n_splits} slices, prefetch {prefetch}", out))
+        if max(q_lens) < heads // kv_heads or all(n == 1 for n in q_lens):
+            out = torch.full_like(p["q"], float("nan"))
+            ops.attention_mfma(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for(q_lens, 1), p["positions"],
+                               out, n_splits, work, scale, window, 16, True, grouped=heads > kv_heads)
+            runs.append((f"one token per tile, {n_splits} slices", out))
+        out = torch.full_like(p["q"], float("nan"))
+        tiles = tiles_for(q_lens, 64)
+        ops.attention_prefill(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles, p["positions"], out, scale,
+                              window, 64, None, n_splits, work if n_splits > 1 else None)
+        runs.append((f"LDS-sharing, {n_splits} slices", out))
+    out = torch.full_like(p["q"], float("nan"))
+    ops.attention_plain(p["q"], p["k_cache"], p["v_cache"], p["table"], p["seq_of_token"], p["positions"], out, scale,
+                        window)
+    runs.append(("plain", out))
+    for what, out in runs:
+        assert torch.isfinite(out.float()).all(), f"{what}: NaN from the pool reached the output"
+        close(out, want, TOL[torch.bfloat16], what)
