@@ -45,7 +45,7 @@ def host_lib():
         i32p, i64p = ctypes.POINTER(ctypes.c_int32), ctypes.POINTER(ctypes.c_int64)
         vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
         sig = {
-            "ixh_cache_create": (vp, [ci, i32p, i32p, ci, ci, i64]),
+            "ixh_cache_create": (vp, [ci, i32p, i32p, ci, ci, i64, i64]),
             "ixh_cache_destroy": (None, [vp]),
             "ixh_cache_error": (ctypes.c_char_p, [vp]),
             "ixh_cache_max_blocks": (ci, [vp]),
@@ -181,11 +181,25 @@ RESERVE_OK, RESERVE_POOL_EMPTY, RESERVE_CONTEXT_FULL = "ok", "pool_empty", "cont
 _RESERVE = {0: RESERVE_OK, 1: RESERVE_POOL_EMPTY, 2: RESERVE_CONTEXT_FULL}
 
 
+def pages_for_window(window: int, page_size: int, max_requests: int, max_step_tokens: int) -> int:
+    """Pages that a windowed group can ever hold at once when no step brings more than `max_step_tokens` tokens
+    of a request: per request the pages that cover the window behind its next position and the step in front of
+    it (plus the two that the ends may straddle), for every request slot.  A pool of this size never runs out."""
+    return max_requests * (-(-(window + max_step_tokens) // page_size) + 2)
+
+
 class CacheManager:
+    """`max_step_tokens`: the most tokens of one request that a step will ever bring, if the caller can promise one
+    (a scheduler's token budget).  With it, a windowed group that gives passed pages back takes a request's pages as
+    the steps reach them instead of at reservation, so its pool may be as small as `pages_for_window` says however
+    long the prompts are; a step that brings more is refused.  Without it every group holds what is reserved."""
+
     def __init__(self, groups: Sequence[GroupLayout], pages_per_group: Sequence[int], page_size: int,
-                 max_requests: int, max_seq_len: int):
+                 max_requests: int, max_seq_len: int, max_step_tokens: Optional[int] = None):
         if page_size <= 0 or max_requests <= 0 or max_seq_len <= 0:
             raise CacheError("page_size, max_requests and max_seq_len must be positive")
+        if max_step_tokens is not None and max_step_tokens <= 0:
+            raise CacheError("max_step_tokens must be positive")
         if len(groups) != len(pages_per_group):
             raise CacheError("one page count per group is needed")
         if any(n <= 0 for n in pages_per_group):
@@ -199,7 +213,9 @@ class CacheManager:
         G = len(self.groups)
         windows = (ctypes.c_int32 * max(G, 1))(*[g.release_window for g in self.groups])
         pages = (ctypes.c_int32 * max(G, 1))(*pages_per_group)
-        self._h = self._lib.ixh_cache_create(G, windows, pages, page_size, max_requests, max_seq_len)
+        self.max_step_tokens = max_step_tokens
+        self._h = self._lib.ixh_cache_create(G, windows, pages, page_size, max_requests, max_seq_len,
+                                             int(max_step_tokens or 0))
         if not self._h:
             raise CacheError("the cache manager could not be created")
         self.pools = [_PoolView(self, g) for g in range(G)]

@@ -53,6 +53,7 @@ struct Cache {
   std::vector<Pool> pools;
   int32_t page_size = 0, max_requests = 0, max_blocks = 0;
   int64_t max_seq_len = 0;
+  int64_t step_cap = 0;  // > 0: no step brings more tokens of a request than this (see reserve)
   std::vector<int32_t> free_slots;
   std::unordered_map<int64_t, Request> requests;
   std::vector<int64_t> order;  // live requests in the order they were added
@@ -102,21 +103,31 @@ struct Cache {
     }
     return ok;
   }
+  // Pages of group g that a request which has `cached` tokens and a reservation up to `upto` holds now.  A group
+  // that keeps every token holds all of them.  A windowed group, when the largest step is known (step_cap), holds
+  // only what the next step can touch, cached + step_cap tokens at most: its pages beyond that are taken when the
+  // steps get there (its pool is sized so that they are there, see pages_for_window in cache/manager.py), so
+  // that a long prompt does not claim a context's worth of pages in a group that only ever reads a window.
+  int64_t pages_held(size_t g, int64_t cached, int64_t upto) const {
+    if (windows[g] > 0 && step_cap > 0 && upto > cached + step_cap) upto = cached + step_cap;
+    return (upto + page_size - 1) / page_size;
+  }
   // 0 ok, 1 pool empty, 2 context full, -1 error
   int reserve(int64_t rid, int64_t new_len) {
     Request* r = get(rid);
     if (!r) return -1;
     if (new_len > max_seq_len) return 2;
-    if (new_len <= r->reserved) return 0;
     if (!release_passed(*r)) return -1;
-    const int64_t want_pages = (new_len + page_size - 1) / page_size;
+    const int64_t upto = new_len > r->reserved ? new_len : r->reserved;
     for (size_t g = 0; g < pools.size(); ++g) {
-      const int64_t need = want_pages - static_cast<int64_t>(r->blocks[g].size());
+      const int64_t need = pages_held(g, r->cached, upto) - static_cast<int64_t>(r->blocks[g].size());
       if (need > pools[g].free_pages()) return 1;  // all groups or nothing
     }
-    for (size_t g = 0; g < pools.size(); ++g)
+    for (size_t g = 0; g < pools.size(); ++g) {
+      const int64_t want_pages = pages_held(g, r->cached, upto);
       while (static_cast<int64_t>(r->blocks[g].size()) < want_pages) r->blocks[g].push_back(pools[g].allocate());
-    r->reserved = new_len;
+    }
+    r->reserved = upto;
     return 0;
   }
 };
@@ -128,8 +139,8 @@ Cache* C(void* h) { return static_cast<Cache*>(h); }
 extern "C" {
 
 void* ixh_cache_create(int n_groups, const int32_t* windows, const int32_t* pages, int page_size, int max_requests,
-                       int64_t max_seq_len) {
-  if (n_groups < 0 || page_size <= 0 || max_requests <= 0 || max_seq_len <= 0) return nullptr;
+                       int64_t max_seq_len, int64_t step_cap) {
+  if (n_groups < 0 || page_size <= 0 || max_requests <= 0 || max_seq_len <= 0 || step_cap < 0) return nullptr;
   for (int g = 0; g < n_groups; ++g)
     if (pages[g] <= 0) return nullptr;
   Cache* c = new Cache();
@@ -138,6 +149,7 @@ void* ixh_cache_create(int n_groups, const int32_t* windows, const int32_t* page
   c->page_size = page_size;
   c->max_requests = max_requests;
   c->max_seq_len = max_seq_len;
+  c->step_cap = step_cap;
   c->max_blocks = static_cast<int32_t>((max_seq_len + page_size - 1) / page_size);
   for (int32_t s = max_requests - 1; s >= 0; --s) c->free_slots.push_back(s);
   return c;
@@ -317,6 +329,11 @@ int ixh_build_batch(void* h, int n, const int64_t* rids, const int32_t* n_tokens
       if (!seen.insert(rids[s]).second) { c->error = "appears twice in one step"; return -1; }
       if (!c->requests.count(rids[s])) { c->error = "is not live"; return -1; }
       if (n_tokens[s] < 0) { c->error = "negative token count"; return -1; }
+      if (c->step_cap > 0 && n_tokens[s] > c->step_cap) {
+        c->error = "brings " + std::to_string(n_tokens[s]) + " tokens in one step, the cache was made for " +
+                   std::to_string(c->step_cap) + " at most";
+        return -1;
+      }
       for (int i = 0; i < n_want[s]; ++i)
         if (want_flat[w_at + i] < 0 || want_flat[w_at + i] >= n_tokens[s]) {
           c->error = "wanted place " + std::to_string(want_flat[w_at + i]) + " is outside its " +

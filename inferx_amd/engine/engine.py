@@ -89,13 +89,21 @@ class LLMEngine:
             weights = load_weights(net, model, rt)
             # page count needs the per-token bytes, which need the cache plan: lay out with one page, then size
             probe = ModelRunner(config, weights, rt, page_size=block_size, num_pages=1, max_requests=max_num_seqs,
-                                max_seq_len=max_model_len, model=net, use_graphs=not enforce_eager)
+                                max_seq_len=max_model_len, model=net, use_graphs=not enforce_eager,
+                                max_step_tokens=max_num_batched_tokens)
             block_bytes = probe.kv_bytes_per_token() * block_size
             free, total = torch.cuda.mem_get_info(rt.device)
             pages = resolve_kv_blocks(max(block_bytes, 1), explicit_blocks=num_gpu_blocks_override,
                                       kv_cache_memory_bytes=kv_cache_memory_bytes,
                                       gpu_memory_utilization=gpu_memory_utilization, total_bytes=total,
                                       used_bytes=total - free, min_blocks=-(-max_model_len // block_size))
+            if num_gpu_blocks_override is None:
+                # Windowed groups take no more than window + step per request, whatever the page count: what they
+                # leave of the budget goes to the groups that keep every token.
+                growing = sum(probe.page_bytes(g) for g, n in enumerate(probe.group_needs)
+                              if probe.pages_of_group(n, pages + 1) > probe.pages_of_group(n, pages))
+                if growing:
+                    pages += max(0, pages * block_bytes - probe.cache_bytes(pages)) // growing
             pages = min(pages, max_num_seqs * -(-max_model_len // block_size))  # more could never be used
             probe._lay_out_cache(pages)
             runner = probe

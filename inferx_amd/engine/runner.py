@@ -21,7 +21,7 @@ from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..cache.manager import CacheManager, GroupLayout
+from ..cache.manager import CacheManager, GroupLayout, pages_for_window
 from ..config import config_from_directory
 from ..parts import build_model
 from ..weights import load_weights
@@ -47,7 +47,8 @@ def _pack(batch: StepBatch, out: Optional[np.ndarray] = None) -> Tuple[List[int]
 class ModelRunner:
     def __init__(self, config, weights: Dict[str, torch.Tensor], rt: Runtime, *, page_size: int = 16,
                  num_pages: int = 256, max_requests: int = 8, max_seq_len: Optional[int] = None, model=None,
-                 use_graphs: bool = True, release_window_pages: bool = True):
+                 use_graphs: bool = True, release_window_pages: bool = True,
+                 max_step_tokens: Optional[int] = None):
         self.config = config
         self.rt = rt
         self.spec = config.model_spec()
@@ -61,6 +62,9 @@ class ModelRunner:
         self.use_graphs = bool(use_graphs) and self.model.graph_safe()
         # False: windowed groups keep every page until the request ends (for differential tests of the release)
         self.release_window_pages = bool(release_window_pages)
+        # the most tokens of one request that a step will bring, if the caller promises one (the scheduler's budget):
+        # windowed groups then get pools sized by window + step instead of by context
+        self.max_step_tokens = max_step_tokens
         self._lay_out_cache(int(num_pages))
 
     @classmethod
@@ -91,13 +95,14 @@ class ModelRunner:
                     owners.append([])
                 owners[needs.index(need)].append((i, name))
         self.group_needs, self.group_owners = needs, owners
+        self.group_pages = [self.pages_of_group(n, num_pages) for n in needs]
         dtype_of = lambda name: rt.dtype if name is None else {"float32": torch.float32, "bfloat16": torch.bfloat16}[name]
         self.pages: List[Dict[str, torch.Tensor]] = []
         for g, need in enumerate(needs):
             arrays = {}
             for a in need.arrays:
                 shape = (a.heads, a.width, self.page_size) if a.transposed else (a.heads, self.page_size, a.width)
-                arrays[a.name] = torch.zeros((len(owners[g]), num_pages) + shape, dtype=dtype_of(a.dtype),
+                arrays[a.name] = torch.zeros((len(owners[g]), self.group_pages[g]) + shape, dtype=dtype_of(a.dtype),
                                              device=rt.device)
             self.pages.append(arrays)
         self.bindings: List[Dict[str, CacheBinding]] = []
@@ -122,14 +127,31 @@ class ModelRunner:
             self.bindings.append(bound)
         self._states = [b.state for bound in self.bindings for b in bound.values() if b.state is not None]
         self.cache = CacheManager([GroupLayout(n.window, self.release_window_pages) for n in needs],
-                                  [num_pages] * len(needs), self.page_size, self.max_requests, self.max_seq_len)
+                                  self.group_pages, self.page_size, self.max_requests, self.max_seq_len,
+                                  self.max_step_tokens)
         self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
         self._graph_pool = None
+
+    def pages_of_group(self, need, num_pages: int) -> int:
+        """A group that keeps every token gets `num_pages`; a windowed one that gives passed pages back, when the
+        largest step is known, no more than it can ever hold."""
+        if need.window > 0 and self.release_window_pages and self.max_step_tokens:
+            return min(num_pages, pages_for_window(need.window, self.page_size, self.max_requests, self.max_step_tokens))
+        return num_pages
 
     def kv_bytes_per_token(self) -> int:
         """Bytes that one token takes in the pages of all groups."""
         return sum(t.shape[0] * t.shape[2] * t.shape[3] * t.shape[4] // self.page_size * t.element_size()
                    for arrays in self.pages for t in arrays.values())
+
+    def page_bytes(self, group: int) -> int:
+        """Bytes of one page of a group, all its owners' arrays together."""
+        return sum(t.shape[0] * t.shape[2] * t.shape[3] * t.shape[4] * t.element_size()
+                   for t in self.pages[group].values())
+
+    def cache_bytes(self, num_pages: int) -> int:
+        """Bytes of all pools if the groups that keep every token get `num_pages` pages."""
+        return sum(self.pages_of_group(n, num_pages) * self.page_bytes(g) for g, n in enumerate(self.group_needs))
 
     # ---- the step ------------------------------------------------------------
     def step(self, batch: StepBatch) -> torch.Tensor:

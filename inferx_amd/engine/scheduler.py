@@ -134,6 +134,9 @@ class Scheduler:
         self.max_running = min(max_running, cache.max_requests)
         self.max_batch_tokens = max_batch_tokens
         self.max_seq_len = min(max_seq_len or cache.max_seq_len, cache.max_seq_len)
+        if cache.max_step_tokens is not None and max_batch_tokens > cache.max_step_tokens:
+            raise ValueError(f"the cache was made for steps of at most {cache.max_step_tokens} tokens of a request, "
+                             f"the token budget is {max_batch_tokens}")
         self._lib = host_lib()
         self._h = self._lib.ixh_sched_create(cache._h, self.max_running, self.max_batch_tokens, self.max_seq_len)
         if not self._h:

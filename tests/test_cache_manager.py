@@ -5,7 +5,8 @@ import random
 import pytest
 
 from inferx_amd.cache.manager import (RESERVE_CONTEXT_FULL, RESERVE_OK, RESERVE_POOL_EMPTY, CacheError, CacheManager,
-                                      GroupLayout, PagePool)
+                                      GroupLayout, PagePool, pages_for_window)
+from inferx_amd.engine.batch import BatchError, build_step_batch
 
 
 def test_pool_lifo_and_double_free():
@@ -96,6 +97,69 @@ def test_a_windowed_group_may_keep_every_page():
         m.free("a")
         m.check()
         assert m.pools[0].used_pages == 0
+
+
+def test_a_windowed_group_takes_pages_as_the_steps_reach_them():
+    # window 8, pages of 4, steps of at most 6 tokens: whatever is reserved, the windowed group holds the pages
+    # for the window behind and one step ahead, the full group everything
+    per_request = pages_for_window(8, 4, 1, 6)
+    assert per_request == 6  # ceil((8 + 6) / 4) + 2
+    m = CacheManager([GroupLayout(0), GroupLayout(8)], [32, per_request], page_size=4, max_requests=1, max_seq_len=128,
+                     max_step_tokens=6)
+    m.add("a")
+    assert m.reserve("a", 100) == RESERVE_OK          # a long prompt, reserved whole (as a scheduler admits it)
+    assert m.pools[0].used_pages == 25 and m.pools[1].used_pages == 2   # 6 tokens ahead: 2 pages
+    fed = 0
+    while fed < 100:
+        n = min(6, 100 - fed)
+        batch = build_step_batch(m, [("a", [1] * n, [])])
+        assert batch.slots[1].min() >= 0 and m.pools[1].used_pages <= per_request
+        batch.validate(10, [p.num_pages for p in m.pools], 4)           # every slot under its table, both groups
+        m.commit("a", n)
+        fed += n
+        m.check()
+    assert m.pools[0].used_pages == 25 and m.pools[1].used_pages <= 3
+    with pytest.raises(BatchError, match="6 at most"):
+        m.reserve("a", 120)
+        build_step_batch(m, [("a", [1] * 7, [])])
+    m.free("a")
+    assert all(p.used_pages == 0 for p in m.pools)
+    # without the promise of a largest step the windowed group holds what is reserved, as before
+    m = CacheManager([GroupLayout(8)], [32], page_size=4, max_requests=1, max_seq_len=128)
+    m.add("a")
+    m.reserve("a", 100)
+    assert m.pools[0].used_pages == 25
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_a_windowed_pool_of_the_computed_size_never_runs_out(seed):
+    rng = random.Random(seed)
+    window, page, slots, cap = 24, 8, 5, 20
+    m = CacheManager([GroupLayout(0), GroupLayout(window)], [400, pages_for_window(window, page, slots, cap)],
+                     page_size=page, max_requests=slots, max_seq_len=600, max_step_tokens=cap)
+    live = {}
+    for i in range(800):
+        if len(live) < slots and rng.random() < 0.3:
+            rid = f"r{i}"
+            m.add(rid)
+            target = rng.randint(1, 600)
+            if m.reserve(rid, target) == RESERVE_OK:  # (only the full group can refuse)
+                live[rid] = [0, target]
+            else:
+                m.free(rid)
+        for rid in list(live):
+            done, target = live[rid]
+            n = min(rng.randint(1, cap), target - done)
+            build_step_batch(m, [(rid, [0] * n, [])])  # raises if any group is out of pages
+            m.commit(rid, n)
+            live[rid][0] = done + n
+            if done + n == target:
+                m.free(rid)
+                del live[rid]
+        m.check()
+    for rid in live:
+        m.free(rid)
+    assert all(p.used_pages == 0 for p in m.pools)
 
 
 def test_reset_keeps_the_slot():

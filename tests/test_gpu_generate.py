@@ -302,6 +302,24 @@ def test_command_line_sizes_the_cache_by_memory_and_dumps_logits(tmp_path):
     assert small.returncode == 1 and "--kv-cache-memory-bytes" in small.stderr and "--max-model-len" in small.stderr
 
 
+def test_generation_with_a_small_token_budget_and_windowed_layers(tmp_path):
+    """The engine promises its token budget to the cache: the windowed layers' pool is sized by window + budget,
+    prompts longer than that pool run through it in portions, and the tokens are the plain implementation's."""
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.sampling import SamplingParams
+    tiny.make_folder(tiny.CONFIG_B, 47, str(tmp_path), "float32")
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    engine = LLMEngine(str(tmp_path), "float32", max_num_seqs=2, max_model_len=192, max_num_batched_tokens=16,
+                       num_gpu_blocks_override=24)
+    pools = engine.runner.cache.pools
+    assert [p.num_pages for p in pools] == [24, 2 * (2 + 2)]  # window 16, budget 16, pages of 16, two requests
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 70 + n) for n in (150, 90, 33)]
+    got = engine.generate(prompts, SamplingParams(max_tokens=5))
+    for p, out in zip(prompts, got):
+        assert out == plain_greedy(cfg, weights, p, 5)[0]
+    assert all(p.used_pages == 0 for p in pools)
+
+
 def test_a_prompt_larger_than_the_pool_ends_out_of_memory(tmp_path):
     """Two pages and a prompt of 40: the request ends out_of_memory at once and the next one runs; the loop does
     not wait for pages that nobody will give back."""

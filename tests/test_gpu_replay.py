@@ -242,3 +242,29 @@ def test_giving_passed_pages_back_changes_no_logit(folders, name, dtype):
     assert got[True].keys() == got[False].keys()
     for key in got[True]:
         assert torch.equal(got[True][key], got[False][key]), f"{key} differs with the release switched off"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_a_windowed_pool_sized_by_window_and_step(folders, name, dtype):
+    """With the largest step promised, the windowed layers' pool holds window + step per request instead of a
+    context's worth, pages are taken as the steps reach them, and no logit changes."""
+    from inferx_amd.engine.runner import ModelRunner
+    prompts = prompts_for(name)
+    steps = ru.mixed(prompts, seed=8, max_live=3)           # no entry brings more than 33 tokens
+    assert max(len(e[1]) for s in steps for e in s["entries"]) <= 33
+    got = {}
+    for cap in (None, 33):
+        runner = ModelRunner.from_directory(folders[(name, dtype)], dtype=dtype, page_size=16, num_pages=24,
+                                            max_requests=3, max_seq_len=128, max_step_tokens=cap)
+        windowed = [g for g, need in enumerate(runner.group_needs) if need.window > 0][0]
+        W = runner.group_needs[windowed].window
+        want_pages = 24 if cap is None else 3 * (-(-(W + 33) // 16) + 2)
+        assert runner.cache.pools[windowed].num_pages == want_pages < (25 if cap is None else 24)
+        assert runner.pages[windowed]["k"].shape[1] == want_pages
+        got[cap] = ru.replay(runner, steps)
+        assert all(p.used_pages == 0 for p in runner.cache.pools)
+    ru.compare(got[33], expected_for(folders, name, dtype), tol_of(dtype), f"windowed pool {name} {dtype}",
+               ties_for(folders, name, dtype))
+    for key in got[None]:
+        assert torch.equal(got[None][key], got[33][key]), f"{key} differs with the smaller pool"
