@@ -5,6 +5,7 @@ Option names and meanings are the reference server's where it has them
 --max-num-batched-tokens, --block-size, --num-gpu-blocks-override,
 --kv-cache-memory-bytes, --gpu-memory-utilization, --enforce-eager, --device);
 --dump-logits writes the file format of the reference's scripts/gen_reference_logits.py;
+--log-level, --log-json, --log-file are the reference's (options.cc:218-227);
 exit code 0 for --help and 2 for a bad command line (include/inferx/support/options.h:17-22).
 There is no tokenizer and no server: prompts are token ids, output is one JSON
 line per prompt.
@@ -23,6 +24,23 @@ def _ids(text: str) -> List[int]:
     return [int(x) for x in text.replace(",", " ").split()]
 
 
+def _set_up_logging(level: str, as_json: bool, path: Optional[str]) -> None:
+    """--log-level, --log-json, --log-file as the reference's server has them (src/support/options.cc:218-227)."""
+    import logging
+
+    class JsonLines(logging.Formatter):
+        def format(self, record):
+            return json.dumps({"time": round(record.created, 3), "level": record.levelname.lower(),
+                               "logger": record.name, "message": record.getMessage()})
+
+    handler = logging.FileHandler(path) if path else logging.StreamHandler(sys.stderr)
+    handler.setFormatter(JsonLines() if as_json else logging.Formatter("%(levelname).1s %(name)s: %(message)s"))
+    root = logging.getLogger("inferx_amd")
+    root.handlers[:] = [handler]
+    root.setLevel(getattr(logging, level.upper()))
+    root.propagate = False
+
+
 def build_parser() -> argparse.ArgumentParser:
     ap = argparse.ArgumentParser(prog="inferx-generate", description=__doc__,
                                  formatter_class=argparse.RawDescriptionHelpFormatter)
@@ -30,13 +48,14 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--model", help="checkpoint directory (config.json + model.safetensors)")
     ap.add_argument("--random-config", help="a config.json: make a folder of random weights from it and run that")
     ap.add_argument("--random-seed", type=int, default=0, help="seed of the random weights")
-    ap.add_argument("--dtype", default="auto", choices=["auto", "bfloat16", "float", "float32"],
+    ap.add_argument("--dtype", default="auto", choices=["auto", "bfloat16", "bf16", "float", "float32", "fp32"],
                     help="auto and bfloat16 run the serving kernels; float32 runs everything in true 32-bit")
     ap.add_argument("--max-num-seqs", type=int, default=8, help="concurrent sequences")
     ap.add_argument("--max-model-len", type=int, default=2048, help="prompt + generation cap")
     ap.add_argument("--max-num-batched-tokens", type=int, default=None, help="token budget per scheduler step")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page")
-    ap.add_argument("--num-gpu-blocks-override", type=int, default=None, help="cache pages (overrides sizing by memory)")
+    ap.add_argument("--num-gpu-blocks-override", "--num-blocks", type=int, default=None,
+                    help="cache pages (overrides sizing by memory)")
     ap.add_argument("--kv-cache-memory-bytes", type=int, default=None, help="explicit cache budget in bytes")
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.92,
                     help="fraction of GPU memory the engine may use")
@@ -58,14 +77,63 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--logprobs", type=int, default=None, metavar="N",
                     help="report each token's log-probability and those of the N most probable (0 to 20)")
     ap.add_argument("--seed", type=int, default=0, help="fixes the sampling draws")
+    ap.add_argument("--config", metavar="FILE", help="a TOML (.toml) or INI file of options by name; the command line wins")
+    ap.add_argument("--log-level", default="warning", choices=["debug", "info", "warning", "error"],
+                    help="what the engine reports on standard error (info: how the cache was sized; debug: every step)")
+    ap.add_argument("--log-json", action="store_true", help="write the log as JSON lines")
+    ap.add_argument("--log-file", help="append the log to a file instead of standard error")
     ap.add_argument("--dump-logits", metavar="FILE",
                     help="also write the float32 logits at every position of every prompt to FILE, one record per "
                          "prompt: 'IXRL', u32 version 1, u32 tokens, u32 vocab, i32 ids[tokens], f32 logits[tokens * vocab]")
     return ap
 
 
+def _config_file_defaults(ap: argparse.ArgumentParser, path: str) -> dict:
+    """Options from a TOML or INI file whose keys are the options' names (with dashes or underscores, without the
+    leading ones); what the command line says wins.  (The reference's server takes such a file through --config,
+    src/support/options.cc.)"""
+    known = {a.dest: a for a in ap._actions if a.option_strings}
+    try:
+        with open(path, "rb") as f:
+            raw = f.read()
+        if path.endswith(".toml"):
+            import tomli
+            table = tomli.loads(raw.decode("utf-8"))
+        else:
+            import configparser
+            cp = configparser.ConfigParser()
+            cp.read_string("[options]\n" + raw.decode("utf-8") if not raw.lstrip().startswith(b"[") else raw.decode("utf-8"))
+            table = {k: v for section in cp.sections() for k, v in cp.items(section)}
+    except (OSError, ValueError, Exception) as e:  # noqa: B014  (any parser's complaint is a bad command line)
+        ap.error(f"cannot read --config {path}: {e}")
+    out = {}
+    for key, value in table.items():
+        dest = key.replace("-", "_")
+        if dest not in known or dest == "config":
+            ap.error(f"--config {path}: unknown option {key!r}")
+        action = known[dest]
+        if isinstance(action, argparse._StoreTrueAction):
+            value = value if isinstance(value, bool) else str(value).strip().lower() in ("1", "true", "yes", "on")
+        elif isinstance(action, argparse._AppendAction):
+            value = [str(v) for v in (value if isinstance(value, list) else [value])]
+        elif action.type is not None and not isinstance(value, bool):
+            try:
+                value = action.type(value)
+            except (TypeError, ValueError):
+                ap.error(f"--config {path}: {key} = {value!r} is not {action.type.__name__}")
+        elif isinstance(value, (int, float)) and action.type is None:
+            value = str(value)
+        if action.choices and value not in action.choices:
+            ap.error(f"--config {path}: {key} must be one of {', '.join(map(str, action.choices))}")
+        out[dest] = value
+    return out
+
+
 def main(argv: Optional[List[str]] = None) -> int:
     ap = build_parser()
+    first, _ = ap.parse_known_args(argv)
+    if first.config:
+        ap.set_defaults(**_config_file_defaults(ap, first.config))
     args = ap.parse_args(argv)
     model = args.model or args.model_tag
     if (model is None) == (args.random_config is None):
@@ -85,6 +153,7 @@ def main(argv: Optional[List[str]] = None) -> int:
     if not prompts or any(not p for p in prompts):
         ap.error("give at least one non-empty prompt (--prompt-ids or --prompt-file)")
 
+    _set_up_logging(args.log_level, args.log_json, args.log_file)
     from ..config import ConfigError
     from ..sampling import SamplingParams
     from ..weights import CheckpointError
@@ -96,9 +165,9 @@ def main(argv: Optional[List[str]] = None) -> int:
             with open(args.random_config) as f:
                 cfg = config_from_json(f.read())
             model = tempfile.mkdtemp(prefix="inferx_random_")
-            store = "float32" if args.dtype in ("float", "float32") else "bfloat16"
+            store = "float32" if args.dtype in ("float", "float32", "fp32") else "bfloat16"
             write_model_folder(cfg, args.random_seed, model, store)
-        dtype = "float32" if args.dtype in ("float", "float32") else "bfloat16"
+        dtype = "float32" if args.dtype in ("float", "float32", "fp32") else "bfloat16"
         engine = LLMEngine(model, dtype, max_num_seqs=args.max_num_seqs, max_model_len=args.max_model_len,
                            max_num_batched_tokens=args.max_num_batched_tokens, block_size=args.block_size,
                            num_gpu_blocks_override=args.num_gpu_blocks_override,

@@ -12,7 +12,7 @@ ids out: tokenizers and servers are not part of this engine.
 from __future__ import annotations
 
 import dataclasses
-
+import logging
 import time
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence, Union
@@ -29,6 +29,7 @@ from .runtime import Runtime
 from .scheduler import Completion, Scheduler
 
 KV_HEADROOM_BYTES = 1 << 30
+log = logging.getLogger("inferx_amd.engine")
 
 
 def resolve_kv_blocks(block_bytes: int, *, explicit_blocks: Optional[int] = None,
@@ -105,6 +106,10 @@ class LLMEngine:
                 if growing:
                     pages += max(0, pages * block_bytes - probe.cache_bytes(pages)) // growing
             pages = min(pages, max_num_seqs * -(-max_model_len // block_size))  # more could never be used
+            # (the reference logs the same figures: AutosizeKvBlocksOnDevice, src/engine/kv_autosize.cc:65-71)
+            log.info("cache: %d bytes on the device, %d already in use, utilization %s, page %d bytes -> %d pages of "
+                     "%d tokens (%d bytes) in %d group(s)", total, total - free, gpu_memory_utilization, block_bytes,
+                     pages, block_size, probe.cache_bytes(pages), len(probe.group_needs))
             probe._lay_out_cache(pages)
             runner = probe
         self.runner = runner
@@ -193,7 +198,12 @@ class LLMEngine:
         self.stats.tokens_out += len(sampled)
         self.stats.preemptions = self.scheduler.preemptions
         self.stats.step_seconds += time.perf_counter() - t0
-        return self.scheduler.take_completed()
+        done = self.scheduler.take_completed()
+        if log.isEnabledFor(logging.DEBUG):
+            log.debug("step %d: %d tokens of %d requests in, %d sampled, %d finished, %.3f ms", self.stats.steps,
+                      plan.num_tokens, len(plan.contributions), len(sampled), len(done),
+                      (time.perf_counter() - t0) * 1e3)
+        return done
 
     def prompt_logits(self, prompt_token_ids: Sequence[int]) -> torch.Tensor:
         """float32 logits [len(prompt), vocab] (on the CPU) at every position of a prompt, run through the step

@@ -274,8 +274,11 @@ def test_command_line_sizes_the_cache_by_memory_and_dumps_logits(tmp_path):
     for p in prompts:
         base += ["--prompt-ids", ",".join(map(str, p))]
     dump = tmp_path / "logits.bin"
-    out = subprocess.run(base + ["--dump-logits", str(dump)], capture_output=True, text=True, timeout=300)
+    out = subprocess.run(base + ["--dump-logits", str(dump), "--log-level", "info", "--log-json"], capture_output=True,
+                         text=True, timeout=300)
     assert out.returncode == 0, out.stderr
+    sized = [json.loads(l) for l in out.stderr.splitlines() if l.startswith("{")]
+    assert any(r["level"] == "info" and "pages of 16 tokens" in r["message"] for r in sized), out.stderr
     recs = [json.loads(l) for l in out.stdout.strip().splitlines()]
     assert [r["output_token_ids"] for r in recs] == want
     raw = dump.read_bytes()
