@@ -194,6 +194,61 @@ def test_random_configurations(tmp_path, seed, dtype, monkeypatch):
         ru.compare(ru.replay(runner, steps), want, (ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL), f"seed {seed} {dtype} {how}", skip=skip)
 
 
+def _edge(**over):
+    base = {"architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "decoder_sparse_step": 1,
+            "mlp_only_layers": [], "norm_topk_prob": False, "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
+            "max_position_embeddings": 1024, "use_sliding_window": False, "tie_word_embeddings": False,
+            "intermediate_size": 40}
+    base.update(over)
+    return base
+
+
+# the ends of what the architecture allows: one expert, one head, every expert chosen, a head of 256, a width of 16
+# and of 1,000, a vocabulary of 17, a window of one key and one that no prompt reaches, six layers of three kinds
+EDGE_CONFIGS = {
+    "one_of_everything": (_edge(num_hidden_layers=2, hidden_size=16, num_attention_heads=1, num_key_value_heads=1,
+                                head_dim=16, num_experts=1, num_experts_per_tok=1, moe_intermediate_size=8,
+                                shared_expert_intermediate_size=0, vocab_size=17, use_sliding_window=True,
+                                sliding_window=1, max_window_layers=1), 16, (2, 3, 64, 65)),
+    "every_expert_chosen": (_edge(num_hidden_layers=2, hidden_size=1000, num_attention_heads=7, num_key_value_heads=1,
+                                  head_dim=256, num_experts=7, num_experts_per_tok=7, moe_intermediate_size=200,
+                                  shared_expert_intermediate_size=512, vocab_size=5003, norm_topk_prob=True,
+                                  use_sliding_window=True, sliding_window=4096, max_window_layers=0,
+                                  tie_word_embeddings=True, rms_norm_eps=1e-3), 64, (129, 300, 40)),
+    "six_layers_three_kinds": (_edge(num_hidden_layers=6, hidden_size=320, num_attention_heads=16,
+                                     num_key_value_heads=8, head_dim=32, num_experts=64, num_experts_per_tok=3,
+                                     moe_intermediate_size=16, shared_expert_intermediate_size=8, vocab_size=64,
+                                     decoder_sparse_step=3, mlp_only_layers=[2], intermediate_size=640, rope_theta=100.0,
+                                     use_sliding_window=True, sliding_window=5, max_window_layers=3, qkv_bias=False),
+                               16, (33, 257, 16, 90)),
+    "window_of_two_in_pages_of_64": (_edge(num_hidden_layers=2, hidden_size=48, num_attention_heads=8,
+                                           num_key_value_heads=8, head_dim=64, num_experts=4, num_experts_per_tok=3,
+                                           moe_intermediate_size=384, shared_expert_intermediate_size=16,
+                                           vocab_size=32000, use_sliding_window=True, sliding_window=2,
+                                           max_window_layers=0), 64, (129, 500, 40)),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", list(EDGE_CONFIGS))
+def test_configurations_at_the_ends(tmp_path, name, dtype):
+    """Whole, last tokens one by one, portions down to two tokens, and mixed, at the ends of the sizes."""
+    from inferx_amd.engine.runner import ModelRunner
+    cfg, page, lengths = EDGE_CONFIGS[name]
+    tiny.make_folder(cfg, seed=3, out_dir=str(tmp_path), dtype=dtype)
+    raw, weights = tiny.read_folder(str(tmp_path))
+    prompts = {f"r{i}": tiny.random_tokens(n, cfg["vocab_size"], seed=50 + i) for i, n in enumerate(lengths)}
+    want = ru.expected_logits(raw, weights, prompts)
+    skip = ru.near_ties(raw, weights, prompts) if dtype == "bfloat16" else set()
+    for how, steps in (("whole", ru.whole(prompts)), ("tail", ru.tail_decoded(prompts, 32)),
+                       ("portions", ru.chunked(prompts, (256, 130, 2, 17, 200, 3))),
+                       ("mixed", ru.mixed(prompts, seed=4, max_live=4))):
+        runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=page, num_pages=4 * (512 // page + 2),
+                                            max_requests=4, max_seq_len=1024)
+        ru.compare(ru.replay(runner, steps), want, (ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL),
+                   f"{name} {dtype} {how}", skip=skip)
+
+
 @pytest.mark.parametrize("use_graphs", [True, False])
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_an_entry_without_tokens_beside_one_with_two(folders, dtype, use_graphs):
