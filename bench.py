@@ -253,6 +253,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--prompt-len", type=int, default=PROMPT,
+                    help="tokens of every request's prompt before it decodes (the context of the decode steps)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
@@ -290,24 +292,30 @@ def main() -> int:
     model = build_model(cfg.model_spec())
     weights = random_tensors(model, seed=0, dtype=args.dtype, device="cuda:0")
     weights = {k: rt.place(v) for k, v in weights.items()}
-    pages = max_batch * CONTEXT // PAGE
+    prompt_len = args.prompt_len
+    # a request's prompt, the tokens it decodes while the later prompts are read (a step each portion), the steps
+    reading = max_batch * -(-prompt_len // PROMPT)
+    context_cap = max(CONTEXT, -(-(prompt_len + reading + 2 * args.steps + args.warmup + 3 * max_batch + 32) // PAGE) * PAGE)
+    pages = max_batch * context_cap // PAGE
     runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=max_batch,
-                         max_seq_len=CONTEXT, model=model)
+                         max_seq_len=context_cap, model=model)
     torch.cuda.synchronize()
     log(f"model ready in {time.time() - t0:.1f}s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB on the device")
     gen = torch.Generator().manual_seed(1234)
 
-    def prompt():
-        return torch.randint(0, cfg.vocab_size, (PROMPT,), generator=gen).tolist()
+    def prompt(n=None):
+        return torch.randint(0, cfg.vocab_size, (n or prompt_len,), generator=gen).tolist()
 
     def run_decode(batch, steps, warmup, single=0):
-        """`batch` requests with prompts of PROMPT tokens through the engine (scheduler, step function, sampler):
+        """`batch` requests with prompts of `prompt_len` tokens through the engine (scheduler, step function, sampler):
         first their prompts, then `warmup` untimed and `steps` timed decode steps of the whole batch; then `single`
         more steps, each timed on its own (the device is waited for after every one of them, so they are a little
         slower than steps that follow each other).  Returns the time of the `steps` and the list of single times."""
-        engine = LLMEngine("", runner=runner, max_num_seqs=batch, max_model_len=CONTEXT, max_num_batched_tokens=PROMPT)
+        engine = LLMEngine("", runner=runner, max_num_seqs=batch, max_model_len=context_cap,
+                           max_num_batched_tokens=max(PROMPT, batch))
         # (requests decode while the later prompts are still being read: room for those tokens too)
-        params = SamplingParams(max_tokens=warmup + steps + single + 3 * batch + 16, ignore_eos=True)
+        params = SamplingParams(max_tokens=warmup + steps + single + batch * -(-prompt_len // PROMPT) + 3 * batch + 16,
+                                ignore_eos=True)
         ids = [engine.add_request(prompt(), params) for _ in range(batch)]
         while any(engine.scheduler.sequence(i).generated() == 0 for i in ids):  # the prompts, one a step
             engine.step()
@@ -341,7 +349,7 @@ def main() -> int:
         times = []
         for i in range(3):
             runner.add_request("p")
-            toks = prompt()
+            toks = prompt(PROMPT)
             torch.cuda.synchronize()
             t = time.perf_counter()
             runner.run_entries([("p", toks, [PROMPT - 1])])
@@ -362,7 +370,7 @@ def main() -> int:
     singles.sort()
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
-    context = PROMPT + args.warmup + args.steps // 2
+    context = prompt_len + args.warmup + args.steps // 2
     gbs = decode_bytes(cfg, args.batch, context, elt) / (dt / args.steps) / 1e9
     pts = {}
     for b in points:
@@ -372,14 +380,14 @@ def main() -> int:
         pts[f"decode_b{b}"] = round(b * steps / d, 1)
 
     line = {
-        "metric": f"Qwen1.5-MoE-A2.7B decode tok/s @ batch {args.batch} (2048-token prompts)",
+        "metric": f"Qwen1.5-MoE-A2.7B decode tok/s @ batch {args.batch} ({prompt_len}-token prompts)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 3),
         "step_ms": {"min": round(singles[0] * 1e3, 3), "median": round(singles[len(singles) // 2] * 1e3, 3)},
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if elt == 2 else "fp32", "data": "synthetic: seeded random weights and token ids",
         "config": {
-            "model": "Qwen1.5-MoE-A2.7B shape", "global_batch": args.batch, "seq_len": CONTEXT, "prompt_len": PROMPT,
+            "model": "Qwen1.5-MoE-A2.7B shape", "global_batch": args.batch, "seq_len": context_cap, "prompt_len": prompt_len,
             "parallelism": "single GPU", "layers": args.layers, "layers_of_shape": SHAPE["num_hidden_layers"],
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "experts": cfg.num_experts, "top_k": cfg.num_experts_per_tok,
