@@ -253,6 +253,8 @@ def main() -> int:
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--points", default="1,64", help="further decode batch sizes, comma separated ('' for none)")
     ap.add_argument("--no-prefill", action="store_true")
+    ap.add_argument("--prefill-tokens", type=int, default=PROMPT,
+                    help="tokens of the prompt whose reading in one step is timed (2,048 is the contract's)")
     ap.add_argument("--prompt-len", type=int, default=PROMPT,
                     help="tokens of every request's prompt before it decodes (the context of the decode steps)")
     args = ap.parse_args()
@@ -295,7 +297,7 @@ def main() -> int:
     prompt_len = args.prompt_len
     # a request's prompt, the tokens it decodes while the later prompts are read (a step each portion), the steps
     reading = max_batch * -(-prompt_len // PROMPT)
-    context_cap = max(CONTEXT, -(-(prompt_len + reading + 2 * args.steps + args.warmup + 3 * max_batch + 32) // PAGE) * PAGE)
+    context_cap = max(CONTEXT, args.prefill_tokens, -(-(prompt_len + reading + 2 * args.steps + args.warmup + 3 * max_batch + 32) // PAGE) * PAGE)
     pages = max_batch * context_cap // PAGE
     runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=max_batch,
                          max_seq_len=context_cap, model=model)
@@ -346,19 +348,20 @@ def main() -> int:
     prefill = None
     if not args.no_prefill:
         log("prefill")
+        n_pre = args.prefill_tokens
         times = []
         for i in range(3):
             runner.add_request("p")
-            toks = prompt(PROMPT)
+            toks = prompt(n_pre)
             torch.cuda.synchronize()
             t = time.perf_counter()
-            runner.run_entries([("p", toks, [PROMPT - 1])])
+            runner.run_entries([("p", toks, [n_pre - 1])])
             torch.cuda.synchronize()
             times.append(time.perf_counter() - t)
             runner.end_request("p")
         sec = min(times[1:])
-        flops = prefill_flops(cfg, PROMPT)
-        prefill = {"value": round(PROMPT / sec, 1), "tokens": PROMPT, "ms": round(sec * 1e3, 3),
+        flops = prefill_flops(cfg, n_pre)
+        prefill = {"value": round(n_pre / sec, 1), "tokens": n_pre, "ms": round(sec * 1e3, 3),
                    "frac": round(flops / sec / (PEAK_TFLOPS["bf16" if elt == 2 else "fp32"] * 1e12), 5),
                    "tflops": round(flops / sec / 1e12, 1),
                    "frac_measured": round(flops / sec / (ceilings["mfma_bf16_tflops"] * 1e12), 5) if elt == 2 else None}
