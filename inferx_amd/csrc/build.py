@@ -31,6 +31,9 @@ FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}", "-Xclang", "-ta
 FILE_FLAGS = {"attention_prefill.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
               "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
 
+# the vendor's library for dense products (csrc/gemm.hip calls its C interface)
+LINK_LIBS = ["-lhipblaslt"]
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -48,7 +51,7 @@ def _digest() -> str:
         h.update(name.encode())
         with open(os.path.join(HERE, name), "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + LINK_LIBS).encode())
     h.update(repr(sorted(FILE_FLAGS.items())).encode())
     return h.hexdigest()[:16]
 
@@ -125,7 +128,7 @@ def build(verbose: bool = True) -> str:
                 _say(f"  [{done}/{len(srcs)}] {name} ({time.time() - t0:.0f}s)")
     lib = os.path.join(out_dir, LIB_NAME)
     tmp = lib + f".tmp{os.getpid()}"
-    p = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp] + sorted(objs),
+    p = subprocess.run([hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", "-o", tmp] + sorted(objs) + LINK_LIBS,
                        capture_output=True, text=True, env=env)
     if p.returncode != 0:
         raise BuildError(f"hipcc failed to link:\n{p.stdout}\n{p.stderr}")
@@ -204,14 +207,53 @@ def load_host() -> ctypes.CDLL:
     return _host_lib
 
 
+_C_TYPES = {"int": ctypes.c_int, "int32_t": ctypes.c_int, "int64_t": ctypes.c_int64, "float": ctypes.c_float,
+            "double": ctypes.c_double, "size_t": ctypes.c_size_t, "hipStream_t": ctypes.c_void_p}
+
+
+def signatures() -> dict:
+    """name -> (result type, argument types) of every `extern "C"` entry point, read from the sources: with the
+    argument types set, ctypes converts plain Python numbers itself (a pointer is an int or None), which costs a
+    fraction of building a ctypes object per argument."""
+    import re
+    out = {}
+    for path in sources():
+        with open(os.path.join(HERE, path)) as f:
+            text = f.read()
+        for m in re.finditer(r'extern\s+"C"\s+([\w\s\*]+?)\s*\b(ix_\w+)\s*\(([^)]*)\)\s*\{', text):
+            result, name, params = m.group(1).strip(), m.group(2), m.group(3)
+            args = []
+            for prm in (q.strip() for q in params.split(",")):
+                if not prm or prm == "void":
+                    continue
+                if "*" in prm:
+                    args.append(ctypes.c_void_p)
+                    continue
+                words = [w for w in prm.split() if w != "const"]
+                if len(words) != 2 or words[0] not in _C_TYPES:
+                    raise BuildError(f"{os.path.basename(path)}: cannot read parameter {prm!r} of {name}")
+                args.append(_C_TYPES[words[0]])
+            if "*" in result:
+                res = ctypes.c_char_p
+            elif result in _C_TYPES:
+                res = _C_TYPES[result]
+            else:
+                raise BuildError(f"{os.path.basename(path)}: cannot read result type {result!r} of {name}")
+            out[name] = (res, args)
+    return out
+
+
 def load() -> ctypes.CDLL:
     """The library, built first if no current build exists.  Raises if it cannot be had."""
     global _lib
     if _lib is None:
         path = find_built() or build()
         try:
-            _lib = ctypes.CDLL(path)
+            lib = ctypes.CDLL(path)
         except OSError as e:
             raise BuildError(f"cannot load {path}: {e}") from None
-        _lib.ix_last_error.restype = ctypes.c_char_p
+        for name, (res, args) in signatures().items():
+            fn = getattr(lib, name)  # every entry point of the sources must be in the library
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
     return _lib

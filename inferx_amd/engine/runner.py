@@ -131,6 +131,7 @@ class ModelRunner:
                                   self.max_step_tokens)
         self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
         self._graph_pool = None
+        self._capture_stream = None
 
     def pages_of_group(self, need, num_pages: int) -> int:
         """A group that keeps every token gets `num_pages`; a windowed one that gives passed pages back, when the
@@ -245,7 +246,11 @@ class _DecodeGraph:
         # The warm-up run really executes the step.  What it appends to the pages the replay writes again, the same
         # values to the same places; per-request state, though, would be advanced twice, so it is put back.
         kept = [state.clone() for state in runner._states]
-        side = torch.cuda.Stream()
+        # Warm-up and capture run on one stream that all of the runner's graphs share: what a library keeps per
+        # stream (the dense products' workspace) is there before the capture, and once for all graphs.
+        if runner._capture_stream is None:
+            runner._capture_stream = torch.cuda.Stream()
+        side = runner._capture_stream
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             runner.model.forward(ctx, runner.bindings)  # warm-up: library plans, allocator
@@ -255,7 +260,7 @@ class _DecodeGraph:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         self.graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(self.graph, pool=runner._graph_pool):
+        with torch.cuda.graph(self.graph, pool=runner._graph_pool, stream=side):
             self.logits = runner.model.forward(ctx, runner.bindings)
         if runner._graph_pool is None:
             runner._graph_pool = self.graph.pool()

@@ -34,14 +34,16 @@ def _dt(t: torch.Tensor) -> int:
         raise KernelError(f"dtype {t.dtype} is not float32 or bfloat16") from None
 
 
+# The entry points' argument types are set when the library is loaded (csrc/build.py `signatures`), so the
+# helpers below hand over plain Python values: an address or None for a pointer, ints and floats for numbers.
 def _ptr(t: Optional[torch.Tensor]):
     if t is None:
-        return ctypes.c_void_p(0)
+        return None
     if not t.is_cuda:
         raise KernelError("kernel operands must live on the GPU (no CPU path exists)")
     if not t.is_contiguous():
         raise KernelError("kernel operands must be contiguous")
-    return ctypes.c_void_p(t.data_ptr())
+    return t.data_ptr()
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
@@ -50,26 +52,21 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 def _stream():
     """The current HIP stream of the current device (what torch launches on, also under graph capture)."""
     if _raw_stream is not None:  # the same value as below, without building a Stream object (17 us a call)
-        return ctypes.c_void_p(_raw_stream(torch.cuda.current_device()))
-    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+        return _raw_stream(torch.cuda.current_device())
+    return torch.cuda.current_stream().cuda_stream
 
 
-def _i64(v):
-    return ctypes.c_int64(int(v))
-
-
-def _i32(v):
-    return ctypes.c_int(int(v))
-
-
-def _f32(v):
-    return ctypes.c_float(float(v))
+_i64 = int
+_i32 = int
+_f32 = float
+_functions = {}
 
 
 def _call(name: str, *args):
-    fn = getattr(lib(), name)
-    rc = fn(*args)
-    if rc != 0:
+    fn = _functions.get(name)
+    if fn is None:
+        fn = _functions[name] = getattr(lib(), name)
+    if fn(*args) != 0:
         raise KernelError(lib().ix_last_error().decode("utf-8", "replace"))
 
 
@@ -473,6 +470,32 @@ def moe_grouped_dual(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offset
     _call("ix_moe_grouped_dual", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
           _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i32(tile_rows), _i64(n_out), _i64(K),
           _ptr(a_s), _ptr(w_s), _ptr(out_s), _i32(T), _i64(n_out_s), _i64(K_s), _i32(1 if gate_up else 0), _stream())
+
+
+_no_library_kernel = set()  # shapes that the vendor's library has no kernel for
+
+
+def gemm_bf16(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+    """out [T, N] = x [T, K] . w[N, K]^T, bfloat16 operands, 32-bit accumulation, out bfloat16 or float32, through the
+    vendor library's C interface.  False if that library has no kernel for the shape: nothing was queued then."""
+    T, K = x.shape
+    N = w.shape[0]
+    key = (T, N, K, out.dtype)
+    if key in _no_library_kernel:
+        return False
+    _need(x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and out.dtype in (torch.bfloat16, torch.float32),
+          "bfloat16 operands and a bfloat16 or float32 result")
+    _need(w.dim() == 2 and w.shape[1] == K and out.shape == (T, N), "shapes do not fit")
+    fn = _functions.get("ix_gemm_bf16")
+    if fn is None:
+        fn = _functions["ix_gemm_bf16"] = lib().ix_gemm_bf16
+    rc = fn(_ptr(x), _ptr(w), _ptr(out), T, N, K, 1 if out.dtype == torch.float32 else 0, _stream())
+    if rc == 2:
+        _no_library_kernel.add(key)
+        return False
+    if rc != 0:
+        raise KernelError(lib().ix_last_error().decode("utf-8", "replace"))
+    return True
 
 
 def linear_skinny_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> None:

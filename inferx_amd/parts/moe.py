@@ -19,7 +19,11 @@ from .base import FeedForward, LazyDelta, LazyNorm, ParamSpec, register_part
 from .dense_mlp import stack_rows
 
 
-SHARED_BESIDE_TOKENS = 256  # from here on the shared expert runs on a second stream beside the routed ones
+# From here on the shared expert runs on a second stream beside the routed ones.  Below it a step of 24 layers
+# waits for the host, which the two streams' hand-overs cost 21 us a layer (measured at the A2.7B shape, beside
+# against one after the other: 8.1 against 7.0 ms at 256 tokens, 8.3 against 8.3 at 512, 9.0 against 9.8 at 768,
+# 15.1 against 15.4 at 2,048).
+SHARED_BESIDE_TOKENS = 512
 # From this width on the LDS-staged expert products run in their wide form (256 weight rows per workgroup) and the
 # shared expert stays on the main stream (a wide workgroup fills a compute unit's LDS, the library's kernels find
 # no place beside it).  Measured, prompt portions at a width of 3,584 (64 experts of 2,560, 8 per token): 14.9 against

@@ -355,3 +355,61 @@ def test_penalties_and_masks():
     out = torch.empty(2, dtype=torch.int32, device=DEV)
     ops.argmax(logits, out)
     assert out.tolist()[0] == 2
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("T,N,K", [(33, 2048, 2048), (300, 1000, 136), (512, 6144, 2048), (64, 131, 100), (1, 17, 16),
+                                   (200, 5003, 72), (2048, 2048, 5632)])
+def test_library_product(T, N, K, out_dtype):
+    """The vendor library's dense product through its C interface: right, or refused with nothing written."""
+    from inferx_amd import ops
+    x, w = rnd(T, K, dtype=torch.bfloat16), rnd(N, K, seed=1, dtype=torch.bfloat16, scale=0.05)
+    out = torch.full((T, N), 7.0, dtype=out_dtype, device=DEV)
+    if not ops.gemm_bf16(x, w, out):
+        torch.cuda.synchronize()
+        assert bool((out == 7.0).all()), "a refused product must not write"
+        assert not ops.gemm_bf16(x, w, out)  # and stays refused
+        return
+    want = x.double().cpu() @ w.double().cpu().T
+    assert rel_err(out, want) < (1e-5 if out_dtype == torch.float32 else 8e-3)
+
+
+def test_library_product_in_a_graph_and_on_two_streams():
+    """Replays of a captured product follow their inputs; products on two streams at once keep to their own
+    workspaces (a shape whose kernel splits the reduction and sums the parts through the workspace)."""
+    from inferx_amd import ops
+    T, N, K = 48, 2048, 5632
+    w = rnd(N, K, seed=1, dtype=torch.bfloat16, scale=0.05)
+    x = rnd(T, K, dtype=torch.bfloat16)
+    out = torch.empty(T, N, dtype=torch.bfloat16, device=DEV)
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        assert ops.gemm_bf16(x, w, out)  # the stream's first product, not recorded: it allocates the workspace
+    s.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        ops.gemm_bf16(x, w, out)
+    for seed in (3, 4, 5):
+        x.copy_(rnd(T, K, seed=seed, dtype=torch.bfloat16))
+        g.replay()
+        torch.cuda.synchronize()
+        eager = torch.empty_like(out)
+        assert ops.gemm_bf16(x, w, eager)
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), f"replay with seed {seed} differs from the eager product"
+        assert rel_err(out, x.double().cpu() @ w.double().cpu().T) < 8e-3
+    # two streams at once, many products each
+    a, b = torch.cuda.Stream(), torch.cuda.Stream()
+    xa, xb = rnd(T, K, seed=8, dtype=torch.bfloat16), rnd(T, K, seed=9, dtype=torch.bfloat16)
+    oa, ob = [torch.empty_like(out) for _ in range(20)], [torch.empty_like(out) for _ in range(20)]
+    torch.cuda.synchronize()
+    for i in range(20):
+        with torch.cuda.stream(a):
+            ops.gemm_bf16(xa, w, oa[i])
+        with torch.cuda.stream(b):
+            ops.gemm_bf16(xb, w, ob[i])
+    torch.cuda.synchronize()
+    assert all(torch.equal(o, oa[0]) for o in oa) and all(torch.equal(o, ob[0]) for o in ob)
+    assert rel_err(oa[0], xa.double().cpu() @ w.double().cpu().T) < 8e-3
+    assert rel_err(ob[0], xb.double().cpu() @ w.double().cpu().T) < 8e-3

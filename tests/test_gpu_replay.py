@@ -194,6 +194,27 @@ def test_random_configurations(tmp_path, seed, dtype, monkeypatch):
         ru.compare(ru.replay(runner, steps), want, (ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL), f"seed {seed} {dtype} {how}", skip=skip)
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name,requests", [("A", 40), ("B", 64), ("D", 33)])
+def test_many_requests_decoding_together(folders, name, dtype, requests):
+    """More decoding requests in a step than the few-rows kernels take (so the dense products go to the vendor's
+    library, also inside the captured graph of the step): prompts of a few tokens, then six tokens each, one a step."""
+    from inferx_amd.engine.runner import ModelRunner
+    cfg = tiny.CONFIGS[name]
+    raw, weights = tiny.read_folder(folders[(name, dtype)])
+    prompts = {f"r{i}": tiny.random_tokens(4 + i % 5 + 6, cfg["vocab_size"], seed=300 + i) for i in range(requests)}
+    want = ru.expected_logits(raw, weights, prompts)
+    skip = ru.near_ties(raw, weights, prompts) if dtype == "bfloat16" else set()
+    steps = [{"entries": [(rid, toks[:-6], list(range(len(toks) - 6)))], "end": []} for rid, toks in prompts.items()]
+    for i in range(6):
+        steps.append({"entries": [(rid, toks[len(toks) - 6 + i:len(toks) - 5 + i], [0]) for rid, toks in prompts.items()],
+                      "end": list(prompts) if i == 5 else []})
+    runner = ModelRunner.from_directory(folders[(name, dtype)], dtype=dtype, page_size=16, num_pages=2 * requests,
+                                        max_requests=requests, max_seq_len=64)
+    ru.compare(ru.replay(runner, steps), want, tol_of(dtype), f"{requests} requests {name} {dtype}", skip)
+    assert runner._graphs, "the steps of one token per request were not replayed from a graph"
+
+
 def _edge(**over):
     base = {"architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "decoder_sparse_step": 1,
             "mlp_only_layers": [], "norm_topk_prob": False, "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
