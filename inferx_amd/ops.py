@@ -39,20 +39,22 @@ def _dt(t: torch.Tensor) -> int:
 def _ptr(t: Optional[torch.Tensor]):
     if t is None:
         return None
-    if not t.is_cuda:
-        raise KernelError("kernel operands must live on the GPU (no CPU path exists)")
-    if not t.is_contiguous():
-        raise KernelError("kernel operands must be contiguous")
-    return t.data_ptr()
+    if t.is_contiguous() and t.is_cuda:
+        return t.data_ptr()
+    raise KernelError("kernel operands must live on the GPU (no CPU path exists)" if not t.is_cuda
+                      else "kernel operands must be contiguous")
 
 
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
 def _stream():
     """The current HIP stream of the current device (what torch launches on, also under graph capture)."""
-    if _raw_stream is not None:  # the same value as below, without building a Stream object (17 us a call)
-        return _raw_stream(torch.cuda.current_device())
+    if _raw_stream is not None and _raw_device is not None:
+        # the same value as below, without building a Stream object (17 us a call) or the checks of
+        # torch.cuda.current_device (1 us)
+        return _raw_stream(_raw_device())
     return torch.cuda.current_stream().cuda_stream
 
 
