@@ -284,13 +284,13 @@ __global__ void qkv_rope_append_kernel(const T* __restrict__ qkv, const void* __
 
 // The same for bfloat16 with head_dim a multiple of 16: a thread takes eight consecutive elements of the
 // low half of a head and the eight of the high half that pair with them (16-byte loads and stores).
-__global__ void __launch_bounds__(256)
-qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
-                            const float2* __restrict__ cs, const int32_t* __restrict__ slots,
-                            uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache,
-                            uint16_t* __restrict__ v_cache, int heads, int kv_heads, int head_dim, int page_size,
-                            int64_t total_slots, int skip_v) {
-  const int64_t t = blockIdx.x;
+// (`t`: the token; `part` of `parts` workgroups share its elements)
+__device__ __forceinline__ void
+qkv_rope_append_vec8_body(int64_t t, int part, int parts, const uint16_t* __restrict__ qkv,
+                          const void* __restrict__ bias, int bias_dtype, const float2* __restrict__ cs,
+                          const int32_t* __restrict__ slots, uint16_t* __restrict__ q_out,
+                          uint16_t* __restrict__ k_cache, uint16_t* __restrict__ v_cache, int heads, int kv_heads,
+                          int head_dim, int page_size, int64_t total_slots, int skip_v) {
   const int half = head_dim / 2, per_head = half / 8;
   const int items = (heads + (skip_v ? 1 : 2) * kv_heads) * per_head;  // values may be left to the kernel below
   const int64_t in_width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
@@ -320,7 +320,7 @@ qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __rest
       for (int i = 0; i < 8; ++i) v[i] += ix_load_rt(bias, bias_dtype, c + i);
     }
   };
-  for (int p = blockIdx.y * blockDim.x + threadIdx.x; p < items; p += gridDim.y * blockDim.x) {
+  for (int p = part * blockDim.x + threadIdx.x; p < items; p += parts * blockDim.x) {
     const int head = p / per_head, j = (p - head * per_head) * 8;
     const int col = head * head_dim + j;
     const uint4 lo4 = *reinterpret_cast<const uint4*>(in + col);
@@ -385,18 +385,28 @@ qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __rest
   }
 }
 
+__global__ void __launch_bounds__(256)
+qkv_rope_append_vec8_kernel(const uint16_t* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
+                            const float2* __restrict__ cs, const int32_t* __restrict__ slots,
+                            uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache,
+                            uint16_t* __restrict__ v_cache, int heads, int kv_heads, int head_dim, int page_size,
+                            int64_t total_slots, int skip_v) {
+  qkv_rope_append_vec8_body(blockIdx.x, blockIdx.y, gridDim.y, qkv, bias, bias_dtype, cs, slots, q_out, k_cache, v_cache,
+                            heads, kv_heads, head_dim, page_size, total_slots, skip_v);
+}
+
 // Values of many tokens (bfloat16): the cache keeps them transposed, so a token's values are head_dim separate
 // 2-byte stores.  A workgroup takes 32 tokens of one kv head, turns the tile in LDS and stores with neighbouring
 // lanes on neighbouring tokens: tokens of one request have consecutive slots, so 32 lanes fill 64 contiguous bytes.
 #define V_TILE_TOKENS 32
-__global__ void __launch_bounds__(256)
-v_append_tile_kernel(const uint16_t* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
-                     const int32_t* __restrict__ slots, uint16_t* __restrict__ v_cache, int64_t tokens, int heads,
-                     int kv_heads, int head_dim, int page_size, int64_t total_slots) {
-  extern __shared__ __align__(16) uint16_t v_tile[];  // [32][head_dim + 2]
-  const int stride = head_dim + 2;
-  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * V_TILE_TOKENS;
-  const int g = blockIdx.y, tid = threadIdx.x;
+__device__ __forceinline__ void
+v_append_tile_body(int64_t tile, int g, uint16_t* v_tile, const uint16_t* __restrict__ qkv,
+                   const void* __restrict__ bias, int bias_dtype, const int32_t* __restrict__ slots,
+                   uint16_t* __restrict__ v_cache, int64_t tokens, int heads, int kv_heads, int head_dim, int page_size,
+                   int64_t total_slots) {
+  const int stride = head_dim + 2;  // v_tile is [32][head_dim + 2]
+  const int64_t t0 = tile * V_TILE_TOKENS;
+  const int tid = threadIdx.x;
   const int64_t in_width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
   const int col0 = (heads + kv_heads + g) * head_dim;
   const int pieces = head_dim / 8;
@@ -428,6 +438,27 @@ v_append_tile_kernel(const uint16_t* __restrict__ qkv, const void* __restrict__ 
     dst[static_cast<int64_t>(d) * page_size] = v_tile[i * stride + d];
 }
 
+// One launch for both: the first `rope_blocks` workgroups (`parts` per token) add the bias, rotate and store
+// queries and keys; the others turn tiles of values.  Neither half waits for the other, and a prompt portion
+// pays one launch instead of two.
+__global__ void __launch_bounds__(256)
+qkv_rope_append_tiles_kernel(const uint16_t* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
+                             const float2* __restrict__ cs, const int32_t* __restrict__ slots,
+                             uint16_t* __restrict__ q_out, uint16_t* __restrict__ k_cache,
+                             uint16_t* __restrict__ v_cache, int64_t tokens, int heads, int kv_heads, int head_dim,
+                             int page_size, int64_t total_slots, int parts, int64_t rope_blocks) {
+  extern __shared__ __align__(16) uint16_t v_tile[];
+  const int64_t b = blockIdx.x;
+  if (b < rope_blocks) {
+    qkv_rope_append_vec8_body(b / parts, static_cast<int>(b % parts), parts, qkv, bias, bias_dtype, cs, slots, q_out,
+                              k_cache, v_cache, heads, kv_heads, head_dim, page_size, total_slots, 1);
+  } else {
+    const int64_t v = b - rope_blocks;
+    v_append_tile_body(v / kv_heads, static_cast<int>(v % kv_heads), v_tile, qkv, bias, bias_dtype, slots, v_cache,
+                       tokens, heads, kv_heads, head_dim, page_size, total_slots);
+  }
+}
+
 extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const void* cs,
                                   const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int64_t tokens,
                                   int heads, int kv_heads, int head_dim, int page_size, int64_t total_slots,
@@ -444,17 +475,22 @@ extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, 
                        head_dim, page_size, total_slots);
   else if (dtype == IX_BF16 && head_dim % 16 == 0 && (reinterpret_cast<uintptr_t>(cs) & 15) == 0) {
     // from a few dozen tokens on, the values go through the kernel that turns tiles of them
-    const int skip_v = (tokens >= 2 * V_TILE_TOKENS && v_cache != nullptr && slots != nullptr && kv_heads <= 65535) ? 1 : 0;
+    const int skip_v = (tokens >= 2 * V_TILE_TOKENS && v_cache != nullptr && slots != nullptr) ? 1 : 0;
     const int items8 = (heads + (skip_v ? 1 : 2) * kv_heads) * (head_dim / 16);
-    dim3 grid8(tokens, std::min((items8 + 255) / 256, 8));
-    hipLaunchKernelGGL(qkv_rope_append_vec8_kernel, grid8, block, 0, stream, (const uint16_t*)qkv, bias, bias_dtype,
-                       (const float2*)cs, slots, (uint16_t*)q_out, (uint16_t*)k_cache, (uint16_t*)v_cache, heads,
-                       kv_heads, head_dim, page_size, total_slots, skip_v);
+    const int parts = std::min((items8 + 255) / 256, 8);
     if (skip_v) {
-      dim3 grid_v(static_cast<unsigned>((tokens + V_TILE_TOKENS - 1) / V_TILE_TOKENS), kv_heads);
+      const int64_t rope_blocks = tokens * parts;
+      const int64_t tile_blocks = (tokens + V_TILE_TOKENS - 1) / V_TILE_TOKENS * kv_heads;
+      IX_REQUIRE(rope_blocks + tile_blocks < (int64_t(1) << 31), "too many tokens for one launch");
       const size_t lds = static_cast<size_t>(V_TILE_TOKENS) * (head_dim + 2) * sizeof(uint16_t);
-      hipLaunchKernelGGL(v_append_tile_kernel, grid_v, block, lds, stream, (const uint16_t*)qkv, bias, bias_dtype,
-                         slots, (uint16_t*)v_cache, tokens, heads, kv_heads, head_dim, page_size, total_slots);
+      hipLaunchKernelGGL(qkv_rope_append_tiles_kernel, dim3(static_cast<unsigned>(rope_blocks + tile_blocks)), block, lds,
+                         stream, (const uint16_t*)qkv, bias, bias_dtype, (const float2*)cs, slots, (uint16_t*)q_out,
+                         (uint16_t*)k_cache, (uint16_t*)v_cache, tokens, heads, kv_heads, head_dim, page_size,
+                         total_slots, parts, rope_blocks);
+    } else {
+      hipLaunchKernelGGL(qkv_rope_append_vec8_kernel, dim3(tokens, parts), block, 0, stream, (const uint16_t*)qkv, bias,
+                         bias_dtype, (const float2*)cs, slots, (uint16_t*)q_out, (uint16_t*)k_cache,
+                         (uint16_t*)v_cache, heads, kv_heads, head_dim, page_size, total_slots, 0);
     }
   } else if (dtype == IX_BF16)
     hipLaunchKernelGGL(qkv_rope_append_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)qkv, bias, bias_dtype,
