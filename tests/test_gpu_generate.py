@@ -167,6 +167,44 @@ def test_long_decoding_and_first_tokens(tmp_path, dtype):
     assert runner.use_graphs and len(runner._graphs) >= 2  # captured steps were replayed, over several buckets
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_portions_whose_keys_are_cut_into_slices(tmp_path, dtype, monkeypatch):
+    """A prompt read in portions on top of a growing context, with the rule that cuts a portion's keys into slices
+    (a workgroup each; from about 6,000 keys on) brought down to 512 keys so that the plain implementation can
+    follow; then tokens one by one (keys in several slices there too), on layers with and without a window."""
+    from inferx_amd import ops
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.parts import attention
+    monkeypatch.setattr(attention, "PREFILL_SLICED_MIN_ROUNDS", 8)
+    monkeypatch.setattr(attention, "PREFILL_SLICE_ROUNDS", 2)
+    monkeypatch.setattr(attention, "PREFILL_MIN_WORKGROUPS", 0)
+    sliced = []
+    real = ops.attention_prefill
+
+    def spy(*args, **kwargs):
+        sliced.append(args[11] if len(args) > 11 else kwargs.get("n_splits", 1))
+        return real(*args, **kwargs)
+    monkeypatch.setattr(ops, "attention_prefill", spy)
+    raw = dict(tiny.CONFIG_B, max_position_embeddings=2048)
+    tiny.make_folder(raw, 37, str(tmp_path), dtype)
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    toks = tiny.random_tokens(1100, cfg["vocab_size"], 82)
+    whole = pm.forward(cfg, weights, toks)
+    runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=16, num_pages=72, max_requests=2,
+                                        max_seq_len=1152)
+    steps, at = [], 0
+    for n in (384, 384, 320):
+        steps.append({"entries": [("r", toks[at:at + n], [0, 1, n // 2, n - 2, n - 1])], "end": []})
+        at += n
+    steps += [{"entries": [("r", toks[i:i + 1], [0])], "end": []} for i in range(at, len(toks))]
+    got = ru.replay(runner, steps)
+    assert len(got) == 15 + 12
+    assert dtype == "float32" or any(n > 1 for n in sliced), "no portion's keys were cut into slices"
+    scale = float(whole.abs().max())
+    worst = max(float((row.double() - whole[pos]).abs().max()) / scale for (_, pos), row in got.items())
+    assert worst < (ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL), f"{dtype}: {worst:.3e} of the largest logit"
+
+
 def test_far_key_and_window_edge_show_in_the_logits(tmp_path):
     """Random weights attend almost uniformly and would hide a lost key.  With attention weights scaled up the
     scores are peaked, so a key lost at a page edge, a split boundary or the window's edge changes the logits."""
