@@ -205,6 +205,42 @@ def test_portions_whose_keys_are_cut_into_slices(tmp_path, dtype, monkeypatch):
     assert worst < (ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL), f"{dtype}: {worst:.3e} of the largest logit"
 
 
+def test_a_context_of_thousands_of_tokens_in_both_types(tmp_path):
+    """9,000 tokens: too many for the plain implementation, so the two kernel families check each other.  The same
+    bfloat16 weights run in float32 (plain kernels, every portion of 2,048 and the last tokens one by one) and in
+    bfloat16 (matrix-core kernels; keys cut into slices for portions and for single tokens, a captured graph for a
+    context of thousands): the logits at the portions' ends and of the last tokens agree within the bfloat16 bound."""
+    from inferx_amd.engine.runner import ModelRunner
+    raw = dict(tiny.CONFIG_B, max_position_embeddings=16384)
+    tiny.make_folder(raw, 38, str(tmp_path), "bfloat16")
+    # (random weights attend almost evenly, and one lost slice of 9,000 keys would hardly show: with the query and
+    # key weights scaled up the scores are peaked)
+    from safetensors.torch import save_file
+    _, weights = tiny.read_folder(str(tmp_path))
+    for k in weights:
+        if "q_proj.weight" in k or "k_proj.weight" in k:
+            weights[k] = weights[k] * 8.0
+    save_file(weights, os.path.join(str(tmp_path), "model.safetensors"))
+    toks = tiny.random_tokens(9006, raw["vocab_size"], 83)
+    steps, at = [], 0
+    for n in (2048, 2048, 2048, 2048, 808):
+        steps.append({"entries": [("r", toks[at:at + n], [n - 1])], "end": []})
+        at += n
+    steps += [{"entries": [("r", toks[i:i + 1], [0])], "end": []} for i in range(at, len(toks))]
+    got = {}
+    for dtype in ("float32", "bfloat16"):
+        runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=16, num_pages=576, max_requests=2,
+                                            max_seq_len=9216)
+        got[dtype] = ru.replay(runner, steps)
+        assert len(got[dtype]) == 5 + 6
+        if dtype == "bfloat16":
+            assert runner._graphs
+    scale = max(float(row.abs().max()) for row in got["float32"].values())
+    errs = {pos: float((got["bfloat16"][(rid, pos)].double() - row.double()).abs().max()) / scale
+            for (rid, pos), row in got["float32"].items()}
+    assert max(errs.values()) < ru.BF16_TOL, f"the two runs differ: {errs}"
+
+
 def test_far_key_and_window_edge_show_in_the_logits(tmp_path):
     """Random weights attend almost uniformly and would hide a lost key.  With attention weights scaled up the
     scores are peaked, so a key lost at a page edge, a split boundary or the window's edge changes the logits."""
