@@ -3,9 +3,9 @@
 // each operand per wavefront, which is right when the weights are the traffic
 // (decoding) and wasteful when dozens of rows share them.
 //
-// A workgroup owns up to 160 rows of one expert (a row tile of the grouping
-// kernel's map; with a few hundred tokens that is all rows of the expert, so
-// its weights are read once) x 128 weight rows: for the gate|up product 64 gate
+// A workgroup owns up to 160 rows of one expert, 192 in the wide form (a row
+// tile of the grouping kernel's map; with a few hundred tokens that is all rows
+// of the expert, so its weights are read once) x 128 weight rows: for the gate|up product 64 gate
 // rows and the 64 up rows that belong to them (64 output columns after SwiGLU),
 // for the down product 128 output columns.  Only the pairs of sixteens of rows
 // that the tile really holds are multiplied.  The reduction runs in stages of
@@ -31,7 +31,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-#define TL_ROWS 160   // the row-tile map is made for tiles of this many rows
+// the row-tile map is made for tiles of this many rows (the wide form has LDS for 192)
+#define TL_ROWS(NWW) ((NWW) == 2 ? 160 : 192)
 #define TL_K 64
 #define TL_STRIDE 64  // elements per LDS row: no padding; the eight 16-byte pieces of a row are stored permuted
 // NWW: wavefronts along the weight rows (2 or 4; two along the activation rows): 64 NWW weight rows and 128 NWW
@@ -289,18 +290,21 @@ moe_grouped_tiled_kernel(const __bf16* a, const __bf16* w, __bf16* out, const in
   const int e = tile_expert[tile];
   const int row0 = tile_row0[tile];
   const int row_end = offsets[e + 1];
-  const int held = min(TL_ROWS, row_end - row0);
+  const int held = min(TL_ROWS(NWW), row_end - row0);
   if (held <= 0) return;
   switch ((held + 31) >> 5) {  // pairs of sixteens of rows this tile holds
     case 1: tiled_body<GATE_UP, 1, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
     case 2: tiled_body<GATE_UP, 2, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
     case 3: tiled_body<GATE_UP, 3, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
     case 4: tiled_body<GATE_UP, 4, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
-    default: tiled_body<GATE_UP, 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    case 5: tiled_body<GATE_UP, 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs); break;
+    default:  // (six pairs of sixteens in the wide form only)
+      tiled_body<GATE_UP, NWW == 4 ? 6 : 5, NWW>(a, w, out, rows, n_out, width, e, row0, row_end, tile, col_block, ws, xs);
+      break;
   }
 }
 
-// The row-tile map must have been made for tiles of TL_ROWS (160) rows.  `wide`: see below.
+// The row-tile map must have been made for tiles of 160 rows, for the wide form of 192.  `wide`: see below.
 extern "C" int ix_moe_grouped_tiled(const void* a, const void* w, void* out, const int32_t* offsets,
                                     const int32_t* rows, const int32_t* tile_expert, const int32_t* tile_row0,
                                     const int32_t* tile_info, int max_tiles, int64_t a_rows, int64_t n_out,

@@ -511,12 +511,18 @@ def linear_skinny_f32(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> No
 
 
 MOE_TILED_ROWS = 160  # rows per tile of the LDS-staged grouped product
+MOE_TILED_ROWS_WIDE = 192  # ... of its wide form
+
+
+def moe_tiled_rows(wide: bool) -> int:
+    return MOE_TILED_ROWS_WIDE if wide else MOE_TILED_ROWS
 
 
 def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offsets: torch.Tensor,
                       rows: Optional[torch.Tensor], tile_map: torch.Tensor, gate_up: bool, wide: bool = False) -> None:
     """Grouped product staged through LDS (bfloat16, many rows per expert); `tile_map` made for tiles of
-    MOE_TILED_ROWS rows.  `wide`: 256 instead of 128 weight rows per workgroup (same results)."""
+    `moe_tiled_rows(wide)` rows.  `wide`: 256 instead of 128 weight rows per workgroup (the same sums in the same
+    order; which rows share a tile, and with it where a row's sum starts, differs)."""
     E = w.shape[0]
     A, n_out = out.shape
     K = a.shape[1]
@@ -530,7 +536,7 @@ def moe_grouped_tiled(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, offse
         _is_i32(rows, A)
     else:
         _need(a.shape[0] >= A, "a has fewer rows than out")
-    mt = moe_max_tiles(A, E, MOE_TILED_ROWS)
+    mt = moe_max_tiles(A, E, moe_tiled_rows(wide))
     _is_i32(tile_map, 2 * mt + 1)
     _call("ix_moe_grouped_tiled", _ptr(a), _ptr(w), _ptr(out), _ptr(offsets), _ptr(rows), _ptr(tile_map[:mt]),
           _ptr(tile_map[mt:2 * mt]), _ptr(tile_map[2 * mt:]), _i32(mt), _i64(a.shape[0]), _i64(n_out), _i64(K),

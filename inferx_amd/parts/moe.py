@@ -101,7 +101,7 @@ class MoeFeedForward(FeedForward):
         # From about three rows per expert on the LDS-staged kernel is faster (60 experts, 4 per token: 174 against
         # 173 us for both products at 48 tokens, 209 against 189 at 96, 316 against 195 at 256).
         per_expert = x.shape[0] * self.top_k / self.num_experts
-        return 16 if (x.shape[0] <= ctx.rt.SKINNY_ROWS or per_expert <= 3) else ops.MOE_TILED_ROWS
+        return 16 if (x.shape[0] <= ctx.rt.SKINNY_ROWS or per_expert <= 3) else ops.moe_tiled_rows(self.wide_tiles)
 
     def dispatch(self, ctx, topk_e, tile_rows: int = 0):
         rt, A = ctx.rt, topk_e.numel()
@@ -118,7 +118,7 @@ class MoeFeedForward(FeedForward):
         rt, A = ctx.rt, rows.numel()
         act = rt.empty((A, self.expert_width))
         y = rt.empty((A, self.hidden_size))
-        if tile_rows == ops.MOE_TILED_ROWS:  # many rows per expert: operands staged through LDS
+        if tile_rows == ops.moe_tiled_rows(self.wide_tiles):  # many rows per expert: operands staged through LDS
             ops.moe_grouped_tiled(x, self.w13, act, offsets, rows, tile_map, True, self.wide_tiles)
             ops.moe_grouped_tiled(act, self.w2, y, offsets, None, tile_map, False, self.wide_tiles)
         elif tile_rows:

@@ -237,7 +237,7 @@ def test_grouped_tiled(T, H, E, k, mi, wide):
     from inferx_amd import ops
     g = torch.Generator().manual_seed(1)
     topk_e = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
-    offsets, rows, dest, tile_map = dispatch(topk_e, E, ops.MOE_TILED_ROWS)
+    offsets, rows, dest, tile_map = dispatch(topk_e, E, ops.moe_tiled_rows(wide))  # tiles of 160 rows, wide 192
     x = rnd(T, H, dtype=torch.bfloat16)
     w13 = rnd(E, 2 * mi, H, seed=2, dtype=torch.bfloat16, scale=H ** -0.5)
     w2 = rnd(E, H, mi, seed=3, dtype=torch.bfloat16, scale=mi ** -0.5)
@@ -246,11 +246,17 @@ def test_grouped_tiled(T, H, E, k, mi, wide):
     y = torch.full((T * k, H), float("nan"), dtype=torch.bfloat16, device=DEV)
     ops.moe_grouped_tiled(act, w2, y, offsets, None, tile_map, False, wide)
     if wide:
+        _, _, _, narrow_map = dispatch(topk_e, E, ops.moe_tiled_rows(False))
         act_n, y_n = torch.empty_like(act), torch.empty_like(y)
-        ops.moe_grouped_tiled(x, w13, act_n, offsets, rows, tile_map, True, False)
-        ops.moe_grouped_tiled(act, w2, y_n, offsets, None, tile_map, False, False)
-        assert torch.equal(act.view(torch.int16), act_n.view(torch.int16))
-        assert torch.equal(y.view(torch.int16), y_n.view(torch.int16))
+        ops.moe_grouped_tiled(x, w13, act_n, offsets, rows, narrow_map, True, False)
+        ops.moe_grouped_tiled(act, w2, y_n, offsets, None, narrow_map, False, False)
+        if H % 512 and mi % 512:
+            # the same sums in the same order (rows of a multiple of 1,024 bytes start the reduction at a stage
+            # that depends on the tile, and the two forms cut tiles differently)
+            assert torch.equal(act.view(torch.int16), act_n.view(torch.int16))
+            assert torch.equal(y.view(torch.int16), y_n.view(torch.int16))
+        else:
+            assert rel_err(act, act_n) < 1e-2 and rel_err(y, y_n) < 1e-2
     if T <= 900:
         assert rel_err(act, grouped_reference(x, w13, offsets.cpu(), rows.cpu(), True)) < 1.5e-2
         assert rel_err(y, grouped_reference(act, w2, offsets.cpu(), None, False)) < 1.5e-2
