@@ -63,12 +63,14 @@ def log(msg):
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
 
 
-def decode_bytes(cfg, batch, context, elt):
-    """Bytes one decode step has to read: every weight it uses once, and the cache of the live requests."""
+def decode_bytes(cfg, batch, context, elt, distinct=None):
+    """Bytes one decode step has to read: every weight it uses once, and the cache of the live requests.
+    `distinct`: experts that a step's tokens choose, per layer (measured); without it what an even router gives."""
     H, L = cfg.hidden_size, cfg.num_hidden_layers
     qd, kvd = cfg.q_dim, cfg.kv_dim
     E, k, mi, si = cfg.num_experts, cfg.num_experts_per_tok, cfg.moe_intermediate_size, cfg.shared_expert_intermediate_size
-    distinct = E * (1.0 - (1.0 - k / E) ** batch)  # expected number of experts a batch touches
+    if distinct is None:
+        distinct = E * (1.0 - (1.0 - k / E) ** batch)  # expected number of experts a batch touches
     per_layer = (qd + 2 * kvd) * H + (qd + 2 * kvd) + H * qd + 2 * H  # attention + norms
     per_layer += E * H + distinct * 3 * mi * H + 3 * si * H + H      # router, routed, shared, shared gate
     weights = L * per_layer + H + cfg.vocab_size * H + batch * H     # final norm, head, embedding rows
@@ -331,6 +333,30 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         assert engine.stats.tokens_out - before == batch * steps, "a timed step was not a decode step of the whole batch"
+        hit = []
+        if single:  # how many experts the steps' tokens really choose: two steps without graphs, offsets read back
+            from inferx_amd import ops
+            seen, graphs = [], runner.use_graphs
+            real = ops.moe_route_dispatch, ops.moe_dispatch
+
+            def spy_small(*a, **k):
+                real[0](*a, **k)
+                seen.append(a[8])
+
+            def spy_wide(topk_e, offsets, *a, **k):
+                real[1](topk_e, offsets, *a, **k)
+                seen.append(offsets)
+            try:
+                runner.use_graphs = False
+                ops.moe_route_dispatch, ops.moe_dispatch = spy_small, spy_wide
+                for _ in range(2):
+                    seen.clear()
+                    engine.step()
+                    torch.cuda.synchronize()  # (the offsets of a layer are a buffer of their own until the step ends)
+                    hit += [int(((o[1:] - o[:-1]) > 0).sum()) for o in seen]
+            finally:
+                runner.use_graphs = graphs
+                ops.moe_route_dispatch, ops.moe_dispatch = real
         singles = []
         for _ in range(single):
             t = time.perf_counter()
@@ -342,7 +368,7 @@ def main() -> int:
         while engine.has_unfinished():
             engine.step()
         assert runner.cache.pools[0].used_pages == 0
-        return dt, singles
+        return dt, singles, (sum(hit) / len(hit) if hit else None)
 
     # ---- prefill of one 2,048-token prompt ---------------------------------
     prefill = None
@@ -369,17 +395,17 @@ def main() -> int:
 
     # ---- decode ----------------------------------------------------------------
     log(f"decode at batch {args.batch}")
-    dt, singles = run_decode(args.batch, args.steps, args.warmup, single=args.steps)
+    dt, singles, experts_hit = run_decode(args.batch, args.steps, args.warmup, single=args.steps)
     singles.sort()
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     context = prompt_len + args.warmup + args.steps // 2
-    gbs = decode_bytes(cfg, args.batch, context, elt) / (dt / args.steps) / 1e9
+    gbs = decode_bytes(cfg, args.batch, context, elt, experts_hit) / (dt / args.steps) / 1e9
     pts = {}
     for b in points:
         log(f"decode at batch {b}")
         steps = max(8, args.steps // 2)
-        d, _ = run_decode(b, steps, max(2, args.warmup // 2))
+        d, _, _ = run_decode(b, steps, max(2, args.warmup // 2))
         pts[f"decode_b{b}"] = round(b * steps / d, 1)
 
     line = {
@@ -399,7 +425,8 @@ def main() -> int:
         },
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                     "frac": round(gbs / PEAK_HBM_GBS, 5), "frac_measured": round(gbs / ceilings["hbm_read_gbs"], 5)},
+                     "frac": round(gbs / PEAK_HBM_GBS, 5), "frac_measured": round(gbs / ceilings["hbm_read_gbs"], 5),
+                     "experts_hit_per_layer": round(experts_hit, 1) if experts_hit else None},
         "ceilings": ceilings,
         "points": pts,
     }
