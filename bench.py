@@ -88,12 +88,43 @@ def prefill_flops(cfg, tokens):
     return linear + attention
 
 
-def step_bytes(cfg, tokens, cache_tokens, elt):
-    """Bytes a step of `tokens` tokens has to read: every weight it uses once, and `cache_tokens` of cache."""
+def experts_hit(run_step, runner, steps=2):
+    """How many experts the tokens of a step really choose, per layer: `steps` steps run without graphs, the
+    grouping's offsets read back."""
+    import torch
+    from inferx_amd import ops
+    seen, hit, graphs = [], [], runner.use_graphs
+    real = ops.moe_route_dispatch, ops.moe_dispatch
+
+    def spy_small(*a, **k):
+        real[0](*a, **k)
+        seen.append(a[8])
+
+    def spy_wide(topk_e, offsets, *a, **k):
+        real[1](topk_e, offsets, *a, **k)
+        seen.append(offsets)
+    try:
+        runner.use_graphs = False
+        ops.moe_route_dispatch, ops.moe_dispatch = spy_small, spy_wide
+        for _ in range(steps):
+            seen.clear()
+            run_step()
+            torch.cuda.synchronize()  # (the offsets of a layer are a buffer of their own until the step ends)
+            hit += [int(((o[1:] - o[:-1]) > 0).sum()) for o in seen]
+    finally:
+        runner.use_graphs = graphs
+        ops.moe_route_dispatch, ops.moe_dispatch = real
+    return sum(hit) / len(hit) if hit else None
+
+
+def step_bytes(cfg, tokens, cache_tokens, elt, distinct=None):
+    """Bytes a step of `tokens` tokens has to read: every weight it uses once, and `cache_tokens` of cache.
+    `distinct`: experts that the step's tokens choose, per layer (measured); without it what an even router gives."""
     H, L = cfg.hidden_size, cfg.num_hidden_layers
     qd, kvd = cfg.q_dim, cfg.kv_dim
     E, k, mi, si = cfg.num_experts, cfg.num_experts_per_tok, cfg.moe_intermediate_size, cfg.shared_expert_intermediate_size
-    distinct = E * (1.0 - (1.0 - k / E) ** tokens)
+    if distinct is None:
+        distinct = E * (1.0 - (1.0 - k / E) ** tokens)
     per_layer = (qd + 2 * kvd) * H + (qd + 2 * kvd) + H * qd + 2 * H + E * H + distinct * 3 * mi * H + 3 * si * H + H
     return (L * per_layer + H + cfg.vocab_size * H + L * 2 * kvd * cache_tokens) * elt
 
@@ -228,7 +259,8 @@ def run_57b(args) -> int:
     assert engine.stats.tokens_out - before == batch * steps, "a timed step was not a decode step of the whole batch"
     pre_flops = linear_flops(cfg, sum(lens), batch) + sum(attention_flops(cfg, n, 0) for n in lens)
     cache_tokens = sum(lens) + batch * (args.warmup + steps // 2 + batch)
-    gbs = step_bytes(cfg, batch, cache_tokens, elt) / dt / 1e9
+    hit = experts_hit(engine.step, runner)
+    gbs = step_bytes(cfg, batch, cache_tokens, elt, hit) / dt / 1e9
     line = dict(base, metric="Qwen2-57B-A14B shape, decode tok/s @ batch 8 after prompts of 16384-32000 tokens",
                 value=round(batch / dt, 1), ms_per_step=round(dt * 1e3, 3),
                 config=dict(sizes, model="Qwen2-57B-A14B shape", global_batch=batch, seq_len=context,
@@ -236,7 +268,8 @@ def run_57b(args) -> int:
                 prefill={"value": round(sum(lens) / t_pre, 1), "tokens": sum(lens), "ms": round(t_pre * 1e3, 1),
                          "frac": round(pre_flops / t_pre / peak, 5)},
                 roofline={"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                          "frac": round(gbs / PEAK_HBM_GBS, 5)}, points={})
+                          "frac": round(gbs / PEAK_HBM_GBS, 5),
+                          "experts_hit_per_layer": round(hit, 1) if hit else None}, points={})
     print(json.dumps(line), flush=True)
     return 0
 
@@ -333,30 +366,7 @@ def main() -> int:
         torch.cuda.synchronize()
         dt = time.perf_counter() - t
         assert engine.stats.tokens_out - before == batch * steps, "a timed step was not a decode step of the whole batch"
-        hit = []
-        if single:  # how many experts the steps' tokens really choose: two steps without graphs, offsets read back
-            from inferx_amd import ops
-            seen, graphs = [], runner.use_graphs
-            real = ops.moe_route_dispatch, ops.moe_dispatch
-
-            def spy_small(*a, **k):
-                real[0](*a, **k)
-                seen.append(a[8])
-
-            def spy_wide(topk_e, offsets, *a, **k):
-                real[1](topk_e, offsets, *a, **k)
-                seen.append(offsets)
-            try:
-                runner.use_graphs = False
-                ops.moe_route_dispatch, ops.moe_dispatch = spy_small, spy_wide
-                for _ in range(2):
-                    seen.clear()
-                    engine.step()
-                    torch.cuda.synchronize()  # (the offsets of a layer are a buffer of their own until the step ends)
-                    hit += [int(((o[1:] - o[:-1]) > 0).sum()) for o in seen]
-            finally:
-                runner.use_graphs = graphs
-                ops.moe_route_dispatch, ops.moe_dispatch = real
+        hit = experts_hit(engine.step, runner) if single else None
         singles = []
         for _ in range(single):
             t = time.perf_counter()
@@ -368,7 +378,7 @@ def main() -> int:
         while engine.has_unfinished():
             engine.step()
         assert runner.cache.pools[0].used_pages == 0
-        return dt, singles, (sum(hit) / len(hit) if hit else None)
+        return dt, singles, hit
 
     # ---- prefill of one 2,048-token prompt ---------------------------------
     prefill = None
@@ -395,12 +405,12 @@ def main() -> int:
 
     # ---- decode ----------------------------------------------------------------
     log(f"decode at batch {args.batch}")
-    dt, singles, experts_hit = run_decode(args.batch, args.steps, args.warmup, single=args.steps)
+    dt, singles, hit_per_layer = run_decode(args.batch, args.steps, args.warmup, single=args.steps)
     singles.sort()
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     context = prompt_len + args.warmup + args.steps // 2
-    gbs = decode_bytes(cfg, args.batch, context, elt, experts_hit) / (dt / args.steps) / 1e9
+    gbs = decode_bytes(cfg, args.batch, context, elt, hit_per_layer) / (dt / args.steps) / 1e9
     pts = {}
     for b in points:
         log(f"decode at batch {b}")
@@ -426,7 +436,7 @@ def main() -> int:
         "prefill": prefill,
         "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
                      "frac": round(gbs / PEAK_HBM_GBS, 5), "frac_measured": round(gbs / ceilings["hbm_read_gbs"], 5),
-                     "experts_hit_per_layer": round(experts_hit, 1) if experts_hit else None},
+                     "experts_hit_per_layer": round(hit_per_layer, 1) if hit_per_layer else None},
         "ceilings": ceilings,
         "points": pts,
     }
