@@ -355,3 +355,70 @@ def test_norm_route_and_dispatch_in_one_launch(T, H, E, k, dtype):
         o1, r1, d1, tm1 = dispatch(e1, E, tile_rows)
         assert torch.equal(e1, e2) and torch.equal(o1, o2) and torch.equal(r1, r2) and torch.equal(d1, d2)
         assert rel_err(w2, w1) < 1e-6 and rel_err(g2, g1) < 1e-6
+
+
+@pytest.mark.parametrize("T,H,E,k,mi,S", [(1, 64, 4, 2, 32, 48), (8, 2048, 60, 4, 1408, 5632), (16, 136, 60, 4, 40, 24),
+                                          (21, 96, 8, 3, 48, 80), (40, 72, 5, 1, 40, 200), (64, 264, 7, 2, 88, 1000)])
+def test_routed_and_shared_experts_in_one_launch(T, H, E, k, mi, S):
+    """The launch that holds the routed experts' product and the shared expert's: the routed part is bit for bit
+    the routed launch's, the shared part is the product of all tokens with the shared weights; both products
+    (gate|up with SwiGLU, down), every tile height that takes the token count."""
+    from inferx_amd import ops
+    g = torch.Generator().manual_seed(1)
+    topk_e = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    x = rnd(T, H, dtype=torch.bfloat16)
+    w13 = rnd(E, 2 * mi, H, seed=2, dtype=torch.bfloat16, scale=H ** -0.5)
+    w2 = rnd(E, H, mi, seed=3, dtype=torch.bfloat16, scale=mi ** -0.5)
+    ws13 = rnd(2 * S, H, seed=4, dtype=torch.bfloat16, scale=H ** -0.5)
+    ws2 = rnd(H, S, seed=5, dtype=torch.bfloat16, scale=S ** -0.5)
+    nan = lambda *shape: torch.full(shape, float("nan"), dtype=torch.bfloat16, device=DEV)
+    for tile_rows in (16, 32, 64):
+        offsets, rows, dest, tile_map = dispatch(topk_e, E, tile_rows)
+        act1, act2, sact = nan(T * k, mi), nan(T * k, mi), nan(T, S)
+        ops.moe_grouped_mfma(x, w13, act1, offsets, rows, tile_map, tile_rows, True, 4)
+        ops.moe_grouped_dual(x, w13, act2, offsets, rows, tile_map, tile_rows, x, ws13, sact, True)
+        assert torch.equal(act1.view(torch.int16), act2.view(torch.int16))
+        want = torch.nn.functional.silu(x.double() @ ws13[:S].double().T) * (x.double() @ ws13[S:].double().T)
+        assert rel_err(sact, want) < 1.5e-2
+        y1, y2, sout = nan(T * k, H), nan(T * k, H), nan(T, H)
+        ops.moe_grouped_mfma(act1, w2, y1, offsets, None, tile_map, tile_rows, False, 4)
+        ops.moe_grouped_dual(act2, w2, y2, offsets, None, tile_map, tile_rows, sact, ws2, sout, False)
+        assert torch.equal(y1.view(torch.int16), y2.view(torch.int16))
+        assert rel_err(sout, sact.double() @ ws2.double().T) < 1.5e-2
+        assert rel_err(y2, grouped_reference(act2, w2, offsets.cpu(), None, False)) < 1.5e-2
+
+
+@pytest.mark.parametrize("T,H,k,A", [(1, 64, 2, 2), (8, 2048, 4, 32), (21, 96, 3, 70), (5, 1000, 1, 5), (130, 72, 8, 1040)])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("with_shared,gated", [(False, False), (True, False), (True, True)])
+def test_expert_sum_add_and_norm_in_one_pass(T, H, k, A, dtype, with_shared, gated):
+    """h += sum_s w[t, s] y[dest[t, s]] + gate[t] shared[t]; out = rmsnorm(h) * weight: against the two kernels one
+    after the other (the sum rounded to the run's type in between, as they leave it) and against float64; with
+    picked rows the stream is left alone."""
+    from inferx_amd import ops
+    g = torch.Generator().manual_seed(5)
+    y = rnd(A, H, seed=1, dtype=dtype)
+    dest = torch.stack([torch.randperm(A, generator=g)[:k] for _ in range(T)]).to(torch.int32).to(DEV)
+    topk_w = torch.rand(T, k, generator=g).to(DEV)
+    shared = rnd(T, H, seed=2, dtype=dtype) if with_shared else None
+    gate = torch.rand(T, generator=g).to(DEV) if gated else None
+    weight = (1.0 + rnd(H, seed=3, scale=0.2)).to(dtype)
+    h0 = rnd(T, H, seed=4, scale=2.0)
+    eps = 1e-5
+    total = (topk_w.double()[:, :, None] * y.double()[dest.long()]).sum(1)
+    if with_shared:
+        total = total + (gate.double()[:, None] if gated else 1.0) * shared.double()
+    h_want = h0.double() + total
+    x_want = h_want * torch.rsqrt((h_want ** 2).mean(-1, keepdim=True) + eps) * weight.double()
+    tol = 1e-5 if dtype == torch.float32 else 1e-2
+    h1, out1 = h0.clone(), torch.empty(T, H, dtype=dtype, device=DEV)
+    ops.moe_combine_add_rmsnorm(h1, y, dest, topk_w, shared, gate, weight, out1, eps)
+    assert rel_err(h1, h_want) < (1e-6 if dtype == torch.float32 else 4e-3) and rel_err(out1, x_want) < tol
+    summed, h2, out2 = torch.empty(T, H, dtype=dtype, device=DEV), h0.clone(), torch.empty(T, H, dtype=dtype, device=DEV)
+    ops.moe_combine(y, dest, topk_w, shared, gate, summed)
+    ops.add_rmsnorm(h2, summed, weight, out2, eps)
+    assert rel_err(h1, h2) < (1e-6 if dtype == torch.float32 else 4e-3) and rel_err(out1, out2) < tol
+    rows = torch.tensor([T - 1, 0, T // 2, T // 2], dtype=torch.int32, device=DEV)
+    h3, picked = h0.clone(), torch.empty(4, H, dtype=dtype, device=DEV)
+    ops.moe_combine_add_rmsnorm(h3, y, dest, topk_w, shared, gate, weight, picked, eps, rows)
+    assert torch.equal(h3, h0) and rel_err(picked, x_want[rows.long()]) < tol
