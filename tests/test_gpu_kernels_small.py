@@ -413,3 +413,14 @@ def test_library_product_in_a_graph_and_on_two_streams():
     assert all(torch.equal(o, oa[0]) for o in oa) and all(torch.equal(o, ob[0]) for o in ob)
     assert rel_err(oa[0], xa.double().cpu() @ w.double().cpu().T) < 8e-3
     assert rel_err(ob[0], xb.double().cpu() @ w.double().cpu().T) < 8e-3
+
+
+def test_the_probes_of_the_machine_s_ceilings():
+    """The two probes that the benchmark prices its results against: a pure read and pure matrix-core products.
+    Their figures are rates, so only their sanity is checked: positive, finite, and within what one MI355X can do."""
+    import math
+    from inferx_amd import ops
+    got = ops.measured_ceilings(DEV, read_bytes=1 << 30)
+    read, mfma = got["hbm_read_gbs"], got["mfma_bf16_tflops"]
+    assert math.isfinite(read) and 200.0 < read < 30000.0
+    assert math.isfinite(mfma) and 50.0 < mfma < 5200.0
