@@ -93,6 +93,7 @@ class LLMEngine:
                                 max_seq_len=max_model_len, model=net, use_graphs=not enforce_eager,
                                 max_step_tokens=max_num_batched_tokens)
             block_bytes = probe.kv_bytes_per_token() * block_size
+            torch.cuda.empty_cache()  # what loading and restacking the weights left cached is free for the pages
             free, total = torch.cuda.mem_get_info(rt.device)
             pages = resolve_kv_blocks(max(block_bytes, 1), explicit_blocks=num_gpu_blocks_override,
                                       kv_cache_memory_bytes=kv_cache_memory_bytes,

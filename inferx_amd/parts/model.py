@@ -48,8 +48,18 @@ class DecoderModel:
                 out.setdefault(name, p)
         return out
 
-    def bind(self, weights: Dict[str, torch.Tensor], rt) -> None:
-        """Hand every part its tensors (already on the device).  `weights` is emptied."""
+    def shared_tensor_names(self) -> List[str]:
+        """Checkpoint names that more than one part claims (a head tied to the embedding)."""
+        seen: Dict[str, int] = {}
+        for pspec, part in self._part_specs:
+            for p in part.param_specs():
+                name = pspec.tensor_name(p.name)
+                seen[name] = seen.get(name, 0) + 1
+        return [n for n, c in seen.items() if c > 1]
+
+    def bind(self, weights, rt) -> None:
+        """Hand every part its tensors: `weights` maps checkpoint names to tensors on the device (a dict, or a
+        mapping that fetches each when it is asked for) and is emptied."""
         for pspec, part in self._part_specs:
             local = {p.name: weights[pspec.tensor_name(p.name)] for p in part.param_specs()}
             part.bind(local, rt)

@@ -10,7 +10,8 @@ run; integer tables become int32.
 """
 from __future__ import annotations
 
-from typing import Dict, List, Sequence
+from collections.abc import Mapping
+from typing import Callable, Dict, Iterable, Iterator, List, Sequence
 
 import torch
 
@@ -44,9 +45,47 @@ def check_names_and_shapes(expected: Dict[str, tuple], ckpt: Checkpoint, ignored
         + block("wrong shapes", wrong) + block("not floating point", bad_type))
 
 
-def load_weights(model, model_dir: str, rt) -> Dict[str, torch.Tensor]:
-    """All tensors the model needs, on the device, keyed by checkpoint name."""
+class LazyWeights(Mapping):
+    """The tensors a model needs, by checkpoint name, each brought to the device when it is asked for and not kept
+    here: a part that restacks what it is given (the experts of a mixture, gate|up of a dense feed-forward) then
+    holds its own layout only, and loading peaks at the size of the model plus one layer's tensors instead of
+    twice the model.  A tensor that more than one part claims (a head tied to the embedding) is kept after its
+    first use, so that all of them get the same one."""
+
+    def __init__(self, names: Iterable[str], fetch: Callable[[str], torch.Tensor], shared: Iterable[str] = ()):
+        self._names = list(names)
+        self._known = set(self._names)
+        self._fetch = fetch
+        self._shared = set(shared)
+        self._kept: Dict[str, torch.Tensor] = {}
+
+    def __getitem__(self, name: str) -> torch.Tensor:
+        if name not in self._known:
+            raise KeyError(name)
+        if name in self._kept:
+            return self._kept[name]
+        t = self._fetch(name)
+        if name in self._shared:
+            self._kept[name] = t
+        return t
+
+    def __contains__(self, name) -> bool:  # (the inherited one would fetch the tensor to find out)
+        return name in self._known
+
+    def __iter__(self) -> Iterator[str]:
+        return iter(self._names)
+
+    def __len__(self) -> int:
+        return len(self._names)
+
+    def clear(self) -> None:
+        self._names, self._known, self._kept = [], set(), {}
+
+
+def load_weights(model, model_dir: str, rt) -> Mapping:
+    """All tensors the model needs, keyed by checkpoint name; each is read and put on the device when the model's
+    `bind` asks for it (`LazyWeights`).  Names, shapes and types are checked here, before anything is read."""
     ckpt = Checkpoint.open(model_dir)
     expected = {name: tuple(p.shape) for name, p in model.expected_tensors().items()}
     check_names_and_shapes(expected, ckpt, model.spec.ignored_tensor_suffixes)
-    return {name: rt.place(ckpt.get(name)) for name in expected}
+    return LazyWeights(expected, lambda name: rt.place(ckpt.get(name)), model.shared_tensor_names())

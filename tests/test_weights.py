@@ -122,3 +122,27 @@ def test_sharded(tmp_path):
     with pytest.raises(CheckpointError) as e:
         Checkpoint.open(d)
     assert "appears in both" in str(e.value)
+
+
+def test_tensors_are_fetched_when_asked_for_and_not_kept():
+    """The mapping that `load_weights` returns brings a tensor in when the model's `bind` asks for it and keeps
+    only what more than one part claims."""
+    from inferx_amd.weights.loader import LazyWeights
+    fetched = []
+
+    def fetch(name):
+        fetched.append(name)
+        return torch.full((2,), float(len(fetched)))
+
+    w = LazyWeights(["a", "b", "tied"], fetch, shared=["tied"])
+    assert list(w) == ["a", "b", "tied"] and len(w) == 3 and "a" in w and "c" not in w
+    first, again = w["a"], w["a"]
+    assert fetched == ["a", "a"] and first is not again           # nothing is kept
+    t1, t2 = w["tied"], w["tied"]
+    assert fetched == ["a", "a", "tied"] and t1 is t2             # what two parts claim is fetched once
+    with pytest.raises(KeyError):
+        w["c"]
+    w.clear()
+    assert len(w) == 0 and "a" not in w
+    with pytest.raises(KeyError):
+        w["a"]
