@@ -230,6 +230,7 @@ def run_57b(args) -> int:
     pages = max(batch * context // PAGE, int(free * 0.85) // per_page)  # the pool fills what memory is left
     runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=batch, max_seq_len=context,
                          model=model)
+    runner.capture_after = 1
     log(f"model ready in {time.time() - t0:.1f}s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB on the device, "
         f"{pages} pages ({pages * PAGE} tokens of cache)")
     engine = LLMEngine("", runner=runner, max_num_seqs=batch, max_model_len=context, max_num_batched_tokens=chunk)
@@ -336,6 +337,7 @@ def main() -> int:
     pages = max_batch * context_cap // PAGE
     runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=max_batch,
                          max_seq_len=context_cap, model=model)
+    runner.capture_after = 1  # a steady batch: its shape is captured at the first step, whatever --warmup says
     torch.cuda.synchronize()
     log(f"model ready in {time.time() - t0:.1f}s, {torch.cuda.memory_allocated() / 2**30:.1f} GiB on the device")
     gen = torch.Generator().manual_seed(1234)
