@@ -131,6 +131,8 @@ class ModelRunner:
                                   self.max_step_tokens)
         self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
         self._graph_uses: Dict[Tuple[int, int], int] = {}
+        self._graph_logits: Optional[torch.Tensor] = None
+        self.max_graphs = 128   # the least recently replayed shape goes when there are more
         self.capture_after = 3  # (1: every shape is captured at its first step; see _graph_step)
         self._graph_pool = None
         self._capture_stream = None
@@ -199,6 +201,13 @@ class ModelRunner:
         return self._context(torch.from_numpy(flat).to(self.rt.device), sizes, batch)
 
     # ---- graphs for one-token-per-request steps ---------------------------------
+    def _shared_logits(self, rows: int) -> torch.Tensor:
+        """The first `rows` rows of the buffer that captured steps leave their logits in."""
+        if self._graph_logits is None:
+            self._graph_logits = torch.empty((self.max_requests, self.spec.vocab_size), dtype=torch.float32,
+                                             device=self.rt.device)
+        return self._graph_logits[:rows]
+
     def _graph_step(self, batch: StepBatch) -> torch.Tensor:
         S = batch.num_requests
         longest = int(batch.seq_lens.max())
@@ -213,7 +222,11 @@ class ModelRunner:
             uses = self._graph_uses[key] = self._graph_uses.get(key, 0) + 1
             if uses < self.capture_after:
                 return self.model.forward(self._upload(batch), self.bindings)
-            graph = self._graphs[key] = _DecodeGraph(self, batch, bucket)
+            if len(self._graphs) >= self.max_graphs:
+                del self._graphs[next(iter(self._graphs))]
+            graph = _DecodeGraph(self, batch, bucket)
+        self._graphs.pop(key, None)
+        self._graphs[key] = graph  # (the dict keeps the order of use: the first key is the least recently used)
         return graph.run(batch)
 
     # ---- convenience over the cache manager -----------------------------------
@@ -255,6 +268,7 @@ class _DecodeGraph:
         # The warm-up run really executes the step.  What it appends to the pages the replay writes again, the same
         # values to the same places; per-request state, though, would be advanced twice, so it is put back.
         kept = [state.clone() for state in runner._states]
+        self.logits = runner._shared_logits(S)  # (allocated before the capture, outside the graphs' pool)
         # Warm-up and capture run on one stream that all of the runner's graphs share: what a library keeps per
         # stream (the dense products' workspace) is there before the capture, and once for all graphs.
         if runner._capture_stream is None:
@@ -277,7 +291,12 @@ class _DecodeGraph:
             else:
                 self.graph.capture_begin(pool=runner._graph_pool)
             try:
-                self.logits = runner.model.forward(ctx, runner.bindings)
+                # The step's logits end in a buffer that all of the runner's graphs share, as the last node of the
+                # graph: what the capture allocated is then free for the next capture (the graphs share a memory
+                # pool), and a graph holds nothing of the size of requests x vocabulary for itself.
+                logits = runner.model.forward(ctx, runner.bindings)
+                self.logits.copy_(logits)
+                del logits
             finally:
                 self.graph.capture_end()
         torch.cuda.current_stream().wait_stream(side)
