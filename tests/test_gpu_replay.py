@@ -215,6 +215,56 @@ def test_many_requests_decoding_together(folders, name, dtype, requests):
     assert runner._graphs, "the steps of one token per request were not replayed from a graph"
 
 
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_shapes_come_and_go(folders, dtype):
+    """A shape of one-token steps is captured when it comes for the third time and runs kernel by kernel before;
+    the runner keeps a bounded number of graphs, the least recently replayed goes first; the graphs leave their
+    logits in one buffer.  Four requests that end one after the other pass through the shapes 4, 3, 2, 1 and, with
+    new requests, come back to 2: every logit as expected whichever way its step ran."""
+    from inferx_amd.engine.runner import ModelRunner
+    name = "A"
+    cfg = tiny.CONFIGS[name]
+    raw, weights = tiny.read_folder(folders[(name, dtype)])
+    lens = {"a": 39, "b": 43, "c": 47, "d": 51, "e": 49, "f": 49}  # (contexts of 35 to 51: one bucket of contexts)
+    prompts = {rid: tiny.random_tokens(n, cfg["vocab_size"], seed=500 + i) for i, (rid, n) in enumerate(lens.items())}
+    want = ru.expected_logits(raw, weights, prompts)
+    skip = ru.near_ties(raw, weights, prompts) if dtype == "bfloat16" else set()
+    first = ["a", "b", "c", "d"]
+    steps = [{"entries": [(rid, prompts[rid][:34], list(range(34)))], "end": []} for rid in first]
+    at = {rid: 34 for rid in first}
+    live = list(first)
+    while live:  # one token each; the shortest ends first: 5 steps of four requests, then 4 of three, of two, of one
+        entries = [(rid, prompts[rid][at[rid]:at[rid] + 1], [0]) for rid in live]
+        for rid in live:
+            at[rid] += 1
+        done = [rid for rid in live if at[rid] == lens[rid]]
+        steps.append({"entries": entries, "end": done})
+        live = [rid for rid in live if rid not in done]
+    second = ["e", "f"]
+    steps += [{"entries": [(rid, prompts[rid][:34], list(range(34)))], "end": []} for rid in second]
+    for i in range(34, 49):
+        steps.append({"entries": [(rid, prompts[rid][i:i + 1], [0]) for rid in second], "end": second if i == 48 else []})
+    runner = ModelRunner.from_directory(folders[(name, dtype)], dtype=dtype, page_size=16, num_pages=16,
+                                        max_requests=4, max_seq_len=64)
+    runner.max_graphs = 2
+    seen = []
+    real = runner._graph_step
+
+    def spy(batch):
+        out = real(batch)
+        seen.append((batch.num_requests, sorted(runner._graphs)))
+        return out
+    runner._graph_step = spy
+    ru.compare(ru.replay(runner, steps), want, tol_of(dtype), f"shapes that come and go {dtype}", skip)
+    sizes = [n for n, _ in seen]
+    assert sizes == [4] * 5 + [3] * 4 + [2] * 4 + [1] * 4 + [2] * 15
+    # the third step of a shape captures it; never more than two graphs; the shape of four has gone by the end
+    captured = [{k[0] for k in keys} for _, keys in seen]
+    assert captured[1] == set() and captured[2] == {4} and all(len(c) <= 2 for c in captured)
+    assert 4 not in captured[-1] and 2 in captured[-1]
+    assert runner._graph_logits is not None and runner._graph_logits.shape == (4, cfg["vocab_size"])
+
+
 def _edge(**over):
     base = {"architectures": ["Qwen2MoeForCausalLM"], "model_type": "qwen2_moe", "decoder_sparse_step": 1,
             "mlp_only_layers": [], "norm_topk_prob": False, "rope_theta": 10000.0, "rms_norm_eps": 1e-6,
