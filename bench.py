@@ -22,6 +22,13 @@ per request are replayed from HIP graphs): under `rocprofv3 --kernel-trace` it s
 the host:
 
     python bench.py --workload mixed-small          # 8 decodes at a context of 2,048 beside 1 prompt portion of 64
+
+and a whole batch through the engine's loop (scheduler, portions, decode graphs as they come, sampling) at the same
+shape:
+
+    python bench.py --workload offline              # 96 requests of 5 to 3,000 prompt tokens and 4 to 120 generated,
+                                                    # 64 at a time, 4,096 tokens a step; with --scarce so few pages
+                                                    # that sequences are preempted
 """
 from __future__ import annotations
 
@@ -275,6 +282,64 @@ def run_57b(args) -> int:
     return 0
 
 
+def run_offline(args) -> int:
+    """A finite batch of requests of mixed lengths through `LLMEngine.generate` (see the module's docstring)."""
+    import random
+    import torch
+    from inferx_amd.config import config_from_dict
+    from inferx_amd.engine.engine import LLMEngine
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_model
+    from inferx_amd.sampling import SamplingParams
+    from inferx_amd.weights import random_tensors
+    raw = dict(SHAPE)
+    raw["num_hidden_layers"] = args.layers or SHAPE["num_hidden_layers"]
+    cfg = config_from_dict(raw)
+    rt = Runtime(args.dtype, "cuda:0")
+    rnd = random.Random(0)
+    n, live, budget, context = 96, 64, 4096, 4096
+    lens = [rnd.choice([rnd.randint(5, 100), rnd.randint(100, 1000), rnd.randint(1000, 3000)]) for _ in range(n)]
+    outs = [rnd.randint(4, 120) for _ in range(n)]
+    gen = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, cfg.vocab_size, (m,), generator=gen).tolist() for m in lens]
+    params = [SamplingParams(max_tokens=m, ignore_eos=True) for m in outs]
+    log(f"drawing random weights on the device ({cfg.num_hidden_layers} layers, {args.dtype})")
+    model = build_model(cfg.model_spec())
+    weights = {k: rt.place(v) for k, v in random_tensors(model, 0, args.dtype, "cuda:0").items()}
+    pages = 2200 if args.scarce else live * context // PAGE
+    runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=pages, max_requests=live, max_seq_len=context,
+                         model=model, max_step_tokens=budget)
+    engine = LLMEngine("", runner=runner, max_num_seqs=live, max_model_len=context, max_num_batched_tokens=budget)
+    engine.generate(prompts[:2], [SamplingParams(max_tokens=2, ignore_eos=True)] * 2)  # libraries' first calls
+    steps0 = engine.stats.steps
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    got = engine.generate(prompts, params, with_reasons=True)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    bad = [(r, len(o), m) for (o, r), m in zip(got, outs) if r != "max_tokens" or len(o) != m]
+    if bad:
+        raise SystemExit(f"bench.py: {len(bad)} requests ended otherwise than asked, e.g. {bad[:3]}")
+    runner.cache.check()
+    total = sum(lens) + sum(outs)
+    print(json.dumps({
+        "metric": f"Qwen1.5-MoE-A2.7B offline batch, prompt + generated tokens/s ({n} requests, {live} at a time)",
+        "value": round(total / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": engine.stats.steps - steps0,
+        "warmup": 0, "ms_per_step": round(dt * 1e3 / max(engine.stats.steps - steps0, 1), 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: seeded random weights, token ids and lengths",
+        "config": {"model": "Qwen1.5-MoE-A2.7B shape", "layers": cfg.num_hidden_layers,
+                   "layers_of_shape": SHAPE["num_hidden_layers"], "requests": n, "max_num_seqs": live,
+                   "max_num_batched_tokens": budget, "max_model_len": context, "pages": pages, "page_size": PAGE,
+                   "parallelism": "single GPU"},
+        "seconds": round(dt, 3), "prompt_tokens": sum(lens), "generated_tokens": sum(outs),
+        "prompt_tokens_per_s": round(sum(lens) / dt, 1), "generated_tokens_per_s": round(sum(outs) / dt, 1),
+        "preemptions": engine.stats.preemptions, "graphs_captured": len(runner._graphs)}))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -282,7 +347,8 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=None, help="untimed steps before them (4; 2 for mixed)")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the configuration has (sizes of a layer are never reduced)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long", "mixed-small"],
+    ap.add_argument("--scarce", action="store_true", help="offline: so few pages that sequences are preempted")
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long", "mixed-small", "offline"],
                     help="decode, mixed-small: the Qwen1.5-MoE-A2.7B shape (decode is the default); mixed, long: the "
                          "Qwen2-57B-A14B shape")
     ap.add_argument("--batch", type=int, default=8)
@@ -298,9 +364,11 @@ def main() -> int:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
         return 2
     if args.steps is None:
-        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24}[args.workload]
+        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0}[args.workload]
     if args.warmup is None:
-        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4}[args.workload]
+        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0}[args.workload]
+    if args.workload == "offline":
+        return run_offline(args)
     if args.workload != "decode":
         return run_57b(args)
     if args.layers is None:
