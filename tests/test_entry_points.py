@@ -2,6 +2,8 @@
 every entry point must be read, with the types its declaration has."""
 import ctypes
 
+import pytest
+
 
 def test_signatures_are_read_from_the_sources():
     from inferx_amd.csrc import build
@@ -29,3 +31,17 @@ def test_every_declared_entry_point_is_read():
         with open(os.path.join(build.HERE, name)) as fh:
             declared |= set(re.findall(r'extern\s+"C"[^(;{]*?\b(ix_\w+)\s*\(', fh.read()))
     assert declared == set(build.signatures())
+
+
+def test_a_missing_compiler_or_a_stale_library_is_said_plainly(monkeypatch):
+    """Without hipcc the build fails with an error that says where it looked; a library built from other sources
+    than the present ones is not taken."""
+    from inferx_amd.csrc import build
+    monkeypatch.setattr(build, "_digest", lambda: "not-the-digest-of-any-build")
+    assert build.find_built() is None
+    monkeypatch.undo()
+    monkeypatch.setenv("HIPCC", "/nonexistent/hipcc")
+    monkeypatch.setattr(build.shutil, "which", lambda name: None)
+    monkeypatch.setattr(build.os.path, "isfile", lambda p: False)
+    with pytest.raises(build.BuildError, match="hipcc not found"):
+        build.build(verbose=False)
