@@ -6,20 +6,26 @@
 // library's first heuristic choice for the shape, asked for once per shape and kept.
 //
 // A product may use a workspace (the library's split and stream-K kernels do).  Products on different streams may
-// run at the same time, so every stream has a workspace of its own, allocated at the stream's first product; that
-// first product must not be recorded into a graph (the engine warms a stream up before it captures on it).
+// run at the same time, so a stream gets a workspace of its own, 64 MB, at its first product whose kernel asks for
+// one (most ask for none, and then nothing is allocated); that product must not be recorded into a graph (the engine
+// warms a stream up with the same shapes before it captures on it).  Workspaces live until the process ends.  The
+// plans (one per shape: a descriptor, three layouts, the chosen kernel) are kept for the kMaxPlans shapes used last;
+// steps of many different token counts would otherwise add one per count without bound.
 #include <hipblaslt/hipblaslt.h>
 
+#include <algorithm>
 #include <map>
 #include <mutex>
 #include <tuple>
 #include <utility>
+#include <vector>
 
 #include "common.h"
 
 namespace {
 
 constexpr size_t kWorkspaceBytes = size_t(64) << 20;
+constexpr size_t kMaxPlans = 1024;
 
 struct Plan {
   bool usable = false;
@@ -27,13 +33,39 @@ struct Plan {
   hipblasLtMatrixLayout_t w = nullptr, x = nullptr, out = nullptr;
   hipblasLtMatmulAlgo_t algo;
   size_t workspace = 0;
+  uint64_t last_use = 0;
 };
+
+void destroy(Plan& p) {
+  if (p.w) hipblasLtMatrixLayoutDestroy(p.w);
+  if (p.x) hipblasLtMatrixLayoutDestroy(p.x);
+  if (p.out) hipblasLtMatrixLayoutDestroy(p.out);
+  if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
+  p = Plan();
+}
 
 struct PerDevice {
   hipblasLtHandle_t handle = nullptr;
   std::map<std::tuple<int64_t, int64_t, int64_t, int>, Plan> plans;
   std::map<hipStream_t, void*> workspaces;
+  uint64_t clock = 0;
 };
+
+// Drops the half of the plans that were used longest ago.
+void forget_old_plans(PerDevice& dev) {
+  std::vector<uint64_t> uses;
+  for (auto& kv : dev.plans) uses.push_back(kv.second.last_use);
+  std::nth_element(uses.begin(), uses.begin() + uses.size() / 2, uses.end());
+  const uint64_t cut = uses[uses.size() / 2];
+  for (auto it = dev.plans.begin(); it != dev.plans.end();) {
+    if (it->second.last_use < cut) {
+      destroy(it->second);
+      it = dev.plans.erase(it);
+    } else {
+      ++it;
+    }
+  }
+}
 
 std::mutex g_mutex;
 std::map<int, PerDevice> g_devices;
@@ -97,22 +129,29 @@ extern "C" int ix_gemm_bf16(const void* x, const void* w, void* out, int64_t row
   const auto key = std::make_tuple(rows, n_out, width, out_f32);
   auto it = dev.plans.find(key);
   if (it == dev.plans.end()) {
+    if (dev.plans.size() >= kMaxPlans) forget_old_plans(dev);
     Plan p;
-    IX_REQUIRE(make_plan(dev, p, rows, n_out, width, out_f32) == 0, "hipBLASLt refused the product's description");
+    if (make_plan(dev, p, rows, n_out, width, out_f32) != 0) {
+      destroy(p);
+      IX_REQUIRE(false, "hipBLASLt refused the product's description");
+    }
     it = dev.plans.emplace(key, p).first;
   }
-  const Plan& p = it->second;
+  Plan& p = it->second;
+  p.last_use = ++dev.clock;
   if (!p.usable) return 2;
-  auto ws = dev.workspaces.find(stream);
-  if (ws == dev.workspaces.end() && !capturing(stream)) {
-    void* mem = nullptr;
-    IX_REQUIRE(hipMalloc(&mem, kWorkspaceBytes) == hipSuccess, "no memory for the products' workspace");
-    ws = dev.workspaces.emplace(stream, mem).first;
+  void* workspace = nullptr;
+  if (p.workspace > 0) {
+    auto ws = dev.workspaces.find(stream);
+    if (ws == dev.workspaces.end() && !capturing(stream)) {
+      void* mem = nullptr;
+      IX_REQUIRE(hipMalloc(&mem, kWorkspaceBytes) == hipSuccess, "no memory for the products' workspace");
+      ws = dev.workspaces.emplace(stream, mem).first;
+    }
+    IX_REQUIRE(ws != dev.workspaces.end(),
+               "a stream's first product that needs a workspace allocates it and cannot be recorded into a graph");
+    workspace = ws->second;
   }
-  // (whether this shape's kernel needs the workspace or not: a run that works at one size works at all)
-  IX_REQUIRE(ws != dev.workspaces.end(),
-             "the first product on a stream allocates its workspace and cannot be recorded into a graph");
-  void* workspace = ws->second;
   const float one = 1.0f, zero = 0.0f;
   const hipblasStatus_t st = hipblasLtMatmul(dev.handle, p.desc, &one, w, p.w, x, p.x, &zero, out, p.out, out, p.out,
                                              &p.algo, workspace, p.workspace, stream);

@@ -75,6 +75,9 @@ class Stats:
     step_seconds: float = 0.0
 
 
+PROMPT_LOGITS_ROWS = 512  # rows per step of `LLMEngine.prompt_logits`
+
+
 class LLMEngine:
     def __init__(self, model: str, dtype: str = "bfloat16", *, max_num_seqs: int = 8, max_model_len: int = 2048,
                  max_num_batched_tokens: Optional[int] = None, block_size: int = 16,
@@ -168,13 +171,22 @@ class LLMEngine:
                     return self.scheduler.take_completed()
                 batch = build_step_batch(self.runner.cache, plan.entries())
             t0 = time.perf_counter()
-            logits = self.runner.step(batch)
             rows = [self.scheduler.sequence(c.rid).sampling_row() for c in plan.contributions if c.samples]
-            pending = self.sampler.launch(logits, rows)
         except BaseException:
             # nothing of this step counts: the plan is dropped (its pages stay reserved for the sequences) and the
             # next call plans afresh, so a bad request can be cancelled and the others go on
             self.scheduler.abandon_step()
+            raise
+        stateful = self.runner.keeps_state
+        try:
+            logits = self.runner.step(batch)
+            pending = self.sampler.launch(logits, rows)
+        except BaseException as e:
+            self.scheduler.abandon_step()
+            if stateful:
+                # Pages would be rewritten with the same values when the step is planned again; what parts keep per
+                # request (state slots) may have been advanced by the failed step and would be advanced twice.
+                self._failed = f"{type(e).__name__}: {e} (a model with per-request state cannot run a step again)"
             raise
         self.scheduler.launched()
         try:
@@ -222,7 +234,9 @@ class LLMEngine:
         self.runner.add_request(rid)
         rows = []
         try:
-            budget = self.scheduler.max_batch_tokens
+            # every row is wanted, so a portion's logits are portion x vocabulary floats beside the cache: portions
+            # of at most PROMPT_LOGITS_ROWS whatever the scheduler's budget (512 x 152k x 4 bytes = 0.3 GB)
+            budget = min(self.scheduler.max_batch_tokens, PROMPT_LOGITS_ROWS)
             for at in range(0, len(ids), budget):
                 part = ids[at:at + budget]
                 rows.append(self.runner.run_entries([(rid, part, list(range(len(part))))]).cpu())

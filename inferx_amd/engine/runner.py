@@ -158,6 +158,12 @@ class ModelRunner:
         """Bytes of all pools if the groups that keep every token get `num_pages` pages."""
         return sum(self.pages_of_group(n, num_pages) * self.page_bytes(g) for g, n in enumerate(self.group_needs))
 
+    @property
+    def keeps_state(self) -> bool:
+        """Whether some part keeps a block of state per request (which a step advances, so that a step cannot simply
+        be run again)."""
+        return bool(self._states)
+
     # ---- the step ------------------------------------------------------------
     def step(self, batch: StepBatch) -> torch.Tensor:
         """Run the batch; float32 logits [len(batch.logits_rows), vocab] on the device."""
@@ -221,13 +227,25 @@ class ModelRunner:
             # 150 steps, 12 of them seen three times).
             uses = self._graph_uses[key] = self._graph_uses.get(key, 0) + 1
             if uses < self.capture_after:
-                return self.model.forward(self._upload(batch), self.bindings)
+                # kernel by kernel, with the plans that the recorded step of this shape will have: a request's
+                # results then do not depend on how often the shape has come before
+                ctx = self._upload(batch)
+                self.plan_one_token_step(ctx, S, bucket)
+                return self.model.forward(ctx, self.bindings)
             if len(self._graphs) >= self.max_graphs:
                 del self._graphs[next(iter(self._graphs))]
             graph = _DecodeGraph(self, batch, bucket)
         self._graphs.pop(key, None)
         self._graphs[key] = graph  # (the dict keeps the order of use: the first key is the least recently used)
         return graph.run(batch)
+
+    def plan_one_token_step(self, ctx: StepContext, requests: int, longest: int) -> None:
+        """Every part leaves in `ctx.memo` what it plans on the host for a step of one token per request
+        (`Part.capture_plan`); the runner itself knows none of these plans."""
+        for part in self.model.all_parts():
+            plan = getattr(part, "capture_plan", None)
+            if plan is not None:
+                plan(ctx, requests, longest)
 
     # ---- convenience over the cache manager -----------------------------------
     def add_request(self, rid: Hashable) -> None:
@@ -260,10 +278,9 @@ class _DecodeGraph:
         self.copied = torch.cuda.Event()
         self._fill(flat)
         ctx = runner._context(self.dev, sizes, all_rows)
-        # the attention plan of a one-token-per-request step never changes: tile i = request i, row i, one query
-        tiles = torch.tensor([list(range(S)), list(range(S)), [1] * S], dtype=torch.int32, device=rt.device)
-        ctx.memo[("attention_tiles_host", 16)] = (tiles, S, bucket)
-        ctx.host = None  # nothing may plan from host data inside the capture
+        ctx.host = None  # nothing may plan from host data inside the capture:
+        runner.plan_one_token_step(ctx, S, bucket)  # what the parts plan on the host, they plan here, once
+        plans = dict(ctx.memo)
         self.ctx = ctx
         # The warm-up run really executes the step.  What it appends to the pages the replay writes again, the same
         # values to the same places; per-request state, though, would be advanced twice, so it is put back.
@@ -277,7 +294,7 @@ class _DecodeGraph:
         side.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(side):
             runner.model.forward(ctx, runner.bindings)  # warm-up: library plans, allocator
-            ctx.memo = {("attention_tiles_host", 16): (tiles, S, bucket)}
+            ctx.memo = dict(plans)  # (what the warm-up run memoised was made outside the recording)
             for state, before in zip(runner._states, kept):
                 state.copy_(before)
         torch.cuda.current_stream().wait_stream(side)

@@ -21,7 +21,7 @@ from .dense_mlp import stack_rows
 
 
 class PagedAttention(Mixer):
-    graph_safe = True  # the query tiles are planned on the host, but outside a captured step (see query_tiles)
+    graph_safe = True  # the query tiles are planned on the host, but outside a captured step (see capture_plan)
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, qkv_bias: bool = True,
                  out_bias: bool = False, window: int = 0, scale: Optional[float] = None,
@@ -70,6 +70,15 @@ class PagedAttention(Mixer):
         self.w_out = tensors["o_proj.weight"].contiguous()
         if self.position is not None:
             self.position.bind({}, rt)
+
+    def capture_plan(self, ctx, requests: int, longest: int) -> None:
+        """The query tiles of a step of one token per request never change: tile i = request i, row i, one query;
+        the slices of the keys follow from `longest`."""
+        key = ("attention_tiles_host", QUERY_TILE)
+        if key not in ctx.memo:
+            tiles = torch.tensor([list(range(requests)), list(range(requests)), [1] * requests], dtype=torch.int32,
+                                 device=ctx.rt.device)
+            ctx.memo[key] = (tiles, requests, longest)
 
     def forward(self, ctx, x, cache):
         rt = ctx.rt

@@ -141,6 +141,14 @@ class Part:
     def state_need(self) -> Optional[StateNeed]:
         return None
 
+    # ---- steps of one token per request that are replayed from a graph ----
+    def capture_plan(self, ctx, requests: int, longest: int) -> None:
+        """A part that plans on the host (`ctx.host`) leaves here, in `ctx.memo`, whatever its `forward` looks up
+        when `ctx.host` is None: the plan of a step in which each of `requests` requests brings one token and no
+        context is longer than `longest`.  The plan must not depend on anything else, because the recorded step is
+        replayed for every such batch.  The runner calls this for every part before it records such a step, and
+        before it runs one kernel by kernel too, so that both ways make the same choices."""
+
 
 class Norm(Part):
     def rms_operands(self):

@@ -108,12 +108,14 @@ def gated_mlp(x: torch.Tensor, w_gate: torch.Tensor, w_up: torch.Tensor, w_down:
 
 
 def route(x: torch.Tensor, w_router: torch.Tensor, top_k: int, renormalize: bool,
-          scale: float = 1.0, rnd=no_rounding) -> Tuple[torch.Tensor, torch.Tensor]:
+          scale: float = 1.0, rnd=no_rounding, chosen: Optional[torch.Tensor] = None) -> Tuple[torch.Tensor, torch.Tensor]:
     """p = softmax(x Wr^T) over all experts; k rounds of argmax with strict '>' (lowest index wins a tie),
     chosen weight = p_e, chosen expert masked to -inf; optional division by the sum of the chosen; times scale.
     src/backends/cuda/ops/moe.cu:36-127 (RouteTopKKernel); src/model/moe_ffn.cc:200-221.
     Returns weights [T, k] and experts [T, k], slots in descending score.  `rnd`: the reference stores the scores
-    z in bfloat16 (moe_ffn.cc:200-207) before the 32-bit softmax."""
+    z in bfloat16 (moe_ffn.cc:200-207) before the 32-bit softmax.
+    `chosen` [T, k]: the experts are given (someone else's selection, for tests that compare a run whose near ties
+    fell the other way); the weights are those experts' probabilities, everything after the selection as above."""
     z = rnd(x @ w_router.T)
     T, E = z.shape
     weights = torch.zeros(T, top_k, dtype=x.dtype)
@@ -124,10 +126,14 @@ def route(x: torch.Tensor, w_router: torch.Tensor, top_k: int, renormalize: bool
         row = e.clone()
         total = 0.0
         for slot in range(top_k):
-            best, best_value = -1, -math.inf
-            for i in range(E):
-                if float(row[i]) > best_value:
-                    best_value, best = float(row[i]), i
+            if chosen is not None:
+                best = int(chosen[t, slot])
+                best_value = float(row[best])
+            else:
+                best, best_value = -1, -math.inf
+                for i in range(E):
+                    if float(row[i]) > best_value:
+                        best_value, best = float(row[i]), i
             weights[t, slot] = best_value * inv_sum
             total += float(weights[t, slot])
             experts[t, slot] = best
@@ -149,12 +155,15 @@ def router_margin(x: torch.Tensor, w_router: torch.Tensor, top_k: int) -> torch.
 
 
 def moe_block(x: torch.Tensor, w: Dict[str, torch.Tensor], prefix: str, num_experts: int, top_k: int,
-              renormalize: bool, shared_width: int, rnd=no_rounding) -> torch.Tensor:
+              renormalize: bool, shared_width: int, rnd=no_rounding, chosen: Optional[torch.Tensor] = None,
+              chosen_out: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
     """Every chosen expert applied per token and summed in slot order, plus the sigmoid-gated shared expert:
     out_t = sum_slot w_{t,slot} * MLP_e(x_t)  +  sigmoid(x_t . Wsg) * MLP_shared(x_t).
     src/model/moe_ffn.cc:158-367 (route, experts, combine :305-306, shared :308-351);
     moe.cu:237-255 (CombineRowsKernel), :275-287 (AddSharedExpertKernel: 1/(1+exp(-g)))."""
-    weights, experts = route(x, w[prefix + "gate.weight"], top_k, renormalize, rnd=rnd)
+    weights, experts = route(x, w[prefix + "gate.weight"], top_k, renormalize, rnd=rnd, chosen=chosen)
+    if chosen_out is not None:
+        chosen_out.append(experts)
     # every expert is applied once, to the tokens that chose it (rows of a product do not depend on each other) ...
     applied = {}
     for e in sorted(set(experts.flatten().tolist())):
@@ -201,13 +210,15 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequence[int
             positions: Optional[Sequence[int]] = None,
             schedule: Optional[List[Tuple[int, Optional[int]]]] = None,
             margins: Optional[List[torch.Tensor]] = None, rnd=no_rounding,
-            router_scores: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
+            router_scores: Optional[List[torch.Tensor]] = None, experts: Optional[List[torch.Tensor]] = None,
+            experts_out: Optional[List[torch.Tensor]] = None) -> torch.Tensor:
     """Logits [T, vocab] of one whole sequence.  Layer order and the place of every norm and residual:
     src/model/qwen2.cc:902-1066 (embed :902; input norm :912; qkv + bias :920-923; rope :925-926; attention
     :1021-1023; o_proj + residual :1026-1030; post norm :1036; feed-forward :1042-1048; residual :1051; final norm
     and head :1059-1066).  `schedule`: (layer, cache_from) per execution, default each layer once.
     `margins`: if a list, the router margin per token of every sparse layer run is appended to it; `router_scores`
-    likewise takes the router's scores [T, experts] of every sparse layer.
+    likewise takes the router's scores [T, experts] of every sparse layer, `experts_out` the chosen experts [T, k].
+    `experts`: the chosen experts [T, k] of every sparse layer run, given from outside instead of selected here.
 
     `rnd` is what every stored activation goes through.  With `to_bfloat16_and_back` this is the reference's
     bfloat16 model: every tensor it keeps between kernels is bfloat16 (norm outputs layers.cu:50-76; the q/k/v
@@ -230,6 +241,7 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequence[int
     if schedule is None:
         schedule = [(l, None) for l in range(cfg["num_hidden_layers"])]
     kept: List[Tuple[torch.Tensor, torch.Tensor]] = []
+    sparse_runs = 0
     for layer, cache_from in schedule:
         p = f"model.layers.{layer}."
         x = rnd(rms_norm(h, w[p + "input_layernorm.weight"], eps))
@@ -255,7 +267,9 @@ def forward(cfg: dict, weights: Dict[str, torch.Tensor], token_ids: Sequence[int
             if router_scores is not None:
                 router_scores.append(rnd(x @ w[m + "gate.weight"].T))
             f = moe_block(x, w, m, cfg["num_experts"], cfg["num_experts_per_tok"],
-                          bool(cfg.get("norm_topk_prob", False)), cfg.get("shared_expert_intermediate_size", 0), rnd)
+                          bool(cfg.get("norm_topk_prob", False)), cfg.get("shared_expert_intermediate_size", 0), rnd,
+                          chosen=experts[sparse_runs] if experts is not None else None, chosen_out=experts_out)
+            sparse_runs += 1
         else:
             f = gated_mlp(x, w[m + "gate_proj.weight"], w[m + "up_proj.weight"], w[m + "down_proj.weight"], rnd)
         h = rnd(h + f)

@@ -205,12 +205,17 @@ def test_portions_whose_keys_are_cut_into_slices(tmp_path, dtype, monkeypatch):
     assert worst < (ru.FP32_TOL if dtype == "float32" else ru.BF16_TOL), f"{dtype}: {worst:.3e} of the largest logit"
 
 
-def test_a_context_of_thousands_of_tokens_in_both_types(tmp_path):
-    """9,000 tokens: too many for the plain implementation, so the two kernel families check each other.  The same
-    bfloat16 weights run in float32 (plain kernels, every portion of 2,048 and the last tokens one by one) and in
-    bfloat16 (matrix-core kernels; keys cut into slices for portions and for single tokens, a captured graph for a
-    context of thousands): the logits at the portions' ends and of the last tokens agree within the bfloat16 bound."""
+def test_a_context_of_thousands_of_tokens_in_both_types(tmp_path, monkeypatch):
+    """9,000 tokens, too many for the plain implementation of the whole model.  Every call of the attention part,
+    in both runs, is compared with float64 attention over the keys and values that the cache holds at that moment
+    (read back through the block table): portions of 2,048 on up to 8,192 keys, keys cut into slices for portions
+    and for single tokens, a captured graph for a context of thousands, full and windowed layers.  Beyond that the
+    two kernel families check each other, engine against engine: the same bfloat16 weights run in float32 (plain
+    kernels) and in bfloat16 (matrix-core kernels), and the logits at the portions' ends and of the last tokens
+    agree within the bfloat16 bound."""
+    import attention_util as au
     from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.parts.attention import PagedAttention
     raw = dict(tiny.CONFIG_B, max_position_embeddings=16384)
     tiny.make_folder(raw, 38, str(tmp_path), "bfloat16")
     # (random weights attend almost evenly, and one lost slice of 9,000 keys would hardly show: with the query and
@@ -227,14 +232,41 @@ def test_a_context_of_thousands_of_tokens_in_both_types(tmp_path):
         steps.append({"entries": [("r", toks[at:at + n], [n - 1])], "end": []})
         at += n
     steps += [{"entries": [("r", toks[i:i + 1], [0])], "end": []} for i in range(at, len(toks))]
+    real_attend = PagedAttention.attend
+    checked = {"calls": 0, "worst": 0.0, "windowed": 0, "no_host": 0}
+    shape = {}  # the step's host arrays, set before each step below (a captured step's context has none)
+
+    def attend(self, ctx, q, cache, out):
+        real_attend(self, ctx, q, cache, out)
+        if torch.cuda.is_current_stream_capturing():
+            return  # (a recording runs nothing; the warm-up run before it was checked)
+        want = au.attention_from_cache(q, cache.k, cache.v, ctx.block_tables[cache.group], shape["q_start"],
+                                       shape["seq_lens"], self.scale, self.window)
+        checked["calls"] += 1
+        checked["windowed"] += self.window > 0
+        checked["no_host"] += ctx.host is None
+        checked["worst"] = max(checked["worst"], au.rel_err(out, want))
+    monkeypatch.setattr(PagedAttention, "attend", attend)
     got = {}
     for dtype in ("float32", "bfloat16"):
         runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=16, num_pages=576, max_requests=2,
                                             max_seq_len=9216)
+        runner.capture_after = 2
+        real_step = runner.step
+
+        def step(batch, real_step=real_step):
+            shape["q_start"], shape["seq_lens"] = batch.q_start.copy(), batch.seq_lens.copy()
+            return real_step(batch)
+        runner.step = step
+        checked.update(calls=0, worst=0.0, windowed=0, no_host=0)
         got[dtype] = ru.replay(runner, steps)
         assert len(got[dtype]) == 5 + 6
+        layers = raw["num_hidden_layers"]
+        assert checked["calls"] >= layers * (5 + 2) and checked["windowed"] >= 2 * (5 + 2)
+        assert checked["worst"] < (1e-5 if dtype == "float32" else 1.5e-2), \
+            f"{dtype}: an attention call differs from float64 attention by {checked['worst']:.3e}"
         if dtype == "bfloat16":
-            assert runner._graphs
+            assert runner._graphs and checked["no_host"] >= layers  # the warm-up run of a recording was checked too
     scale = max(float(row.abs().max()) for row in got["float32"].values())
     errs = {pos: float((got["bfloat16"][(rid, pos)].double() - row.double()).abs().max()) / scale
             for (rid, pos), row in got["float32"].items()}
@@ -455,3 +487,46 @@ def test_trace_run_program(tmp_path, dtype):
     for (rid, pos), row in got.items():
         err = float((row.double() - expected[rid][pos]).abs().max()) / scale
         assert err <= tol, f"request {rid} position {pos}: error {err:.2e}"
+
+
+def test_one_token_steps_give_the_same_bits_before_and_after_their_shape_is_recorded(tmp_path):
+    """A shape of (requests, context bucket) runs kernel by kernel until it has come `capture_after` times and
+    from a graph afterwards.  Both ways plan with the bucket (520 keys: eight slices of the keys either way, where the
+    true length alone would give four), so a request's bfloat16 logits do not depend on what the engine has
+    served before."""
+    from inferx_amd.engine.runner import ModelRunner
+    tiny.make_folder(dict(tiny.CONFIG_A, max_position_embeddings=1024), 5, str(tmp_path), "bfloat16")
+    toks = tiny.random_tokens(530, 256, 3)
+    got = {}
+    for after in (1, 3, 10 ** 6):
+        runner = ModelRunner.from_directory(str(tmp_path), dtype="bfloat16", page_size=16, num_pages=40,
+                                            max_requests=1, max_seq_len=640)
+        runner.capture_after = after
+        runner.add_request("a")
+        runner.run_entries([("a", toks[:518], [])])
+        rows = [runner.run_entries([("a", toks[i:i + 1], [0])]).clone() for i in range(518, 530)]
+        assert bool(runner._graphs) == (after < 10 ** 6)
+        got[after] = torch.cat(rows)
+    assert torch.equal(got[1], got[3]) and torch.equal(got[1], got[10 ** 6])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_command_line_with_pages_of_eight_tokens(tmp_path, dtype):
+    """`--block-size 8` through the command line: greedy tokens of the plain implementation (configuration B: the
+    window of 16 passes two pages of eight while a request runs)."""
+    tiny.make_folder(tiny.CONFIG_B, 43, str(tmp_path), dtype)
+    cfg, weights = tiny.read_folder(str(tmp_path))
+    prompts = [tiny.random_tokens(n, cfg["vocab_size"], 70 + n) for n in (11, 37)]
+    cmd = [sys.executable, os.path.join(ROOT, "bin", "inferx-generate"), str(tmp_path), "--dtype", dtype,
+           "--max-tokens", "6", "--max-model-len", "64", "--max-num-seqs", "2", "--block-size", "8",
+           "--num-gpu-blocks-override", "16", "--log-level", "info"]
+    for p in prompts:
+        cmd += ["--prompt-ids", ",".join(map(str, p))]
+    out = subprocess.run(cmd, capture_output=True, text=True, timeout=300)
+    assert out.returncode == 0, out.stderr
+    assert "of 8 tokens" in out.stderr
+    recs = [json.loads(l) for l in out.stdout.strip().splitlines()]
+    for rec, p in zip(recs, prompts):
+        want, margins = plain_greedy(cfg, weights, p, 6)
+        # (bfloat16 may leave the plain implementation's path only where its two best logits nearly tie)
+        check_greedy(rec["output_token_ids"], want, margins, exact=dtype == "float32")

@@ -394,3 +394,31 @@ def test_a_windowed_pool_sized_by_window_and_step(folders, name, dtype):
                ties_for(folders, name, dtype))
     for key in got[None]:
         assert torch.equal(got[None][key], got[33][key]), f"{key} differs with the smaller pool"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("page_size", [4, 8, 24, 48, 128])
+def test_pages_of_other_sizes(folders, page_size, dtype):
+    """Pages of 4, 8, 24, 48 and 128 tokens (the command line takes any positive `--block-size`, reference
+    src/support/options.cc:47-174): configuration B, with dense and expert layers, full and windowed attention (a
+    window of 16, so pages of 4 and 8 are given back while a request runs), the four ways.  A page that is no
+    multiple of 16 sends bfloat16 attention to the plain kernel, one that is no power of two keeps portions off the
+    LDS-sharing kernel; the logits are the plain implementation's either way."""
+    name = "B"
+    prompts = prompts_for(name)
+    expected, ties = expected_for(folders, name, dtype), ties_for(folders, name, dtype)
+    max_tokens = 192 if page_size <= 64 else 256
+    pages = max_tokens // page_size
+    for how, steps in [("whole", ru.whole(prompts)), ("tail", ru.tail_decoded(prompts, 32)),
+                       ("chunked", ru.chunked(prompts)),
+                       ("mixed", ru.mixed(prompts, seed=8, max_tokens=max_tokens, round_to=max(64, page_size)))]:
+        runner = make_runner(folders, name, dtype, num_pages=pages, page_size=page_size)
+        assert runner.page_size == page_size and runner.pages[0]["k"].shape[3] == page_size
+        owners = {}
+        got = ru.replay(runner, steps, page_owners=owners)
+        ru.compare(got, expected, tol_of(dtype), f"pages of {page_size}, {how} {dtype}", ties)
+        assert all(p.used_pages == 0 for p in runner.cache.pools)
+        if how == "mixed":
+            assert any(len(rids) > 1 for rids in owners.values()), "no page was used again"
+        if how == "tail":
+            assert runner._graphs

@@ -575,3 +575,169 @@ def test_a_block_says_which_parts_it_misses_or_does_not_know():
                                 "mixer": PartSpec("toy_latent", {"hidden_size": 8, "rank": 4})})
     with pytest.raises(KeyError, match="no block registered"):
         build_block("no_such_block", {})
+
+
+# ---- a toy mixer that PLANS ON THE HOST for steps of one token per request, and is still replayed from a graph -----
+#   the latent mixer above, but in a step of one token per request it reads, for all requests at once, the first
+#   ceil(longest / page_size) pages of every block table, `longest` being a number that it takes from the host's
+#   batch.  Under a recorded step there is no host batch: the number then comes from the part's own `capture_plan`,
+#   which the runner calls for every part without knowing what any of them leaves in the step's memo.
+def define_toy_planned():
+    from inferx_amd.config import (LayerSpec, ModelSpec, PartSpec, ScheduleEntry, linear_head, register_architecture,
+                                   token_embedding)
+    from inferx_amd.parts import CacheArray, CacheNeed, Mixer, ParamSpec, register_part
+
+    class PlannedLatentMixer(Mixer):
+        graph_safe = True
+        steps_without_host = 0   # how often a step ran from the plan alone (the recording and its warm-up)
+        plans_seen = []          # the `longest` of every plan that the runner asked for
+
+        def __init__(self, hidden_size, rank):
+            self.hidden_size, self.rank = hidden_size, rank
+
+        def cache_need(self):
+            return CacheNeed((CacheArray("latent", 1, self.rank, dtype="float32"),))
+
+        def param_specs(self):
+            H, r = self.hidden_size, self.rank
+            return [ParamSpec("c.weight", (r, H), std=0.15), ParamSpec("q.weight", (r, H), std=0.15),
+                    ParamSpec("o.weight", (H, r), std=0.4)]
+
+        def bind(self, tensors, rt):
+            self.wc, self.wq, self.wo = (tensors[n].float() for n in ("c.weight", "q.weight", "o.weight"))
+
+        def capture_plan(self, ctx, requests, longest):
+            ctx.memo[("toy_planned_longest", self.rank)] = longest
+            type(self).plans_seen.append(longest)
+
+        def forward(self, ctx, x, cache):
+            pages = cache.arrays["latent"]                     # [pages, 1, page_size, rank]
+            page_size = pages.shape[2]
+            flat = pages.view(-1, self.rank)
+            xf = x.float()
+            flat.index_copy_(0, ctx.slots[cache.group].long(), xf @ self.wc.T)
+            q = xf @ self.wq.T
+            table = ctx.block_tables[cache.group]
+            if ctx.one_token_each:
+                longest = ctx.memo.get(("toy_planned_longest", self.rank))
+                if longest is None:
+                    longest = int(ctx.host.seq_lens.max())     # planned on the host, from the step's batch
+                if ctx.host is None:
+                    type(self).steps_without_host += 1
+                n_pages = min(-(-longest // page_size), table.shape[1])
+                c = pages[table[:, :n_pages].long().clamp(min=0)].reshape(x.shape[0], n_pages * page_size, self.rank)
+                keys = torch.arange(n_pages * page_size, device=x.device)
+                scores = torch.einsum("skr,sr->sk", c, q) / self.rank ** 0.5
+                scores = scores.masked_fill(keys[None, :] > ctx.positions[:, None], float("-inf"))
+                # (pages beyond a request's own hold other requests' numbers or stale ones: weight exactly zero)
+                out = torch.einsum("sk,skr->sr", torch.softmax(scores, -1), torch.nan_to_num(c))
+                return (out @ self.wo.T).to(x.dtype)
+            batch = ctx.host
+            out = torch.empty_like(q)
+            for t in range(batch.num_tokens):
+                s, p = int(batch.seq_of_token[t]), int(batch.positions[t])
+                keys = torch.arange(p + 1, device=x.device)
+                slots = table[s, keys // page_size].long() * page_size + keys % page_size
+                c = flat[slots]
+                out[t] = torch.softmax(c @ q[t] / self.rank ** 0.5, 0) @ c
+            return (out @ self.wo.T).to(x.dtype)
+
+    register_part("mixer", "toy_planned_latent", PlannedLatentMixer)
+
+    class ToyPlannedConfig:
+        def __init__(self, raw):
+            self.raw = raw
+
+        @classmethod
+        def from_dict(cls, raw):
+            return cls(raw)
+
+        def validate(self):
+            pass
+
+        def model_spec(self):
+            r = self.raw
+            H, V = r["hidden_size"], r["vocab_size"]
+            norm = lambda p: PartSpec("rmsnorm", {"width": H, "eps": r["eps"]}, prefix=p)
+            layers = []
+            for l, kind in enumerate(r["mixers"]):
+                p = f"layers.{l}."
+                if kind == "planned":
+                    mixer = PartSpec("toy_planned_latent", {"hidden_size": H, "rank": r["rank"]}, prefix=p + "latent.")
+                else:
+                    mixer = PartSpec("attention", {"hidden_size": H, "num_heads": 2, "num_kv_heads": 1, "head_dim": 16,
+                                                   "qkv_bias": True, "init_std": 0.2,
+                                                   "position": PartSpec("rope", {"theta": 1e4, "rotary_dim": 16})},
+                                     prefix=p + "attn.")
+                ffn = PartSpec("dense_mlp", {"hidden_size": H, "width": r["width"], "init_std": 0.2}, prefix=p + "mlp.")
+                layers.append(LayerSpec("prenorm", {"mixer": mixer, "feed_forward": ffn, "mixer_norm": norm(p + "norm1."),
+                                                    "feed_forward_norm": norm(p + "norm2.")}))
+            return ModelSpec("ToyPlannedForCausalLM", H, V, 0, layers, [ScheduleEntry(l) for l in range(len(layers))],
+                             token_embedding("embed.weight", V, H, 0.5), norm("final_norm."),
+                             linear_head("embed.weight", V, H, 0.5), init_std=0.5)
+
+    register_architecture("ToyPlannedForCausalLM", ToyPlannedConfig)
+    return ToyPlannedConfig, PlannedLatentMixer
+
+
+PLANNED = {"architectures": ["ToyPlannedForCausalLM"], "hidden_size": 32, "eps": 1e-5, "width": 40, "rank": 12,
+           "vocab_size": 64, "mixers": ["planned", "attention", "planned"]}
+
+
+def toy_planned_reference(w, tokens):
+    """The toy model, whole sequence, float64."""
+    w = {k: v.double() for k, v in w.items()}
+    r, T = PLANNED, len(tokens)
+    pos = torch.arange(T)
+    h = w["embed.weight"][torch.tensor(tokens)]
+    for l, kind in enumerate(r["mixers"]):
+        p = f"layers.{l}."
+        x = pm.rms_norm(h, w[p + "norm1.weight"], r["eps"])
+        if kind == "planned":
+            c, q = x @ w[p + "latent.c.weight"].T, x @ w[p + "latent.q.weight"].T
+            rows = [torch.softmax(c[:t + 1] @ q[t] / r["rank"] ** 0.5, 0) @ c[:t + 1] for t in range(T)]
+            a = torch.stack(rows) @ w[p + "latent.o.weight"].T
+        else:
+            n = p + "attn."
+            q = pm.apply_rope((x @ w[n + "q_proj.weight"].T + w[n + "q_proj.bias"]).view(T, 2, 16), pos, 1e4)
+            k = pm.apply_rope((x @ w[n + "k_proj.weight"].T + w[n + "k_proj.bias"]).view(T, 1, 16), pos, 1e4)
+            v = (x @ w[n + "v_proj.weight"].T + w[n + "v_proj.bias"]).view(T, 1, 16)
+            a = pm.attention(q, k, v, pos, 0.25).reshape(T, 32) @ w[n + "o_proj.weight"].T
+        h = h + a
+        x = pm.rms_norm(h, w[p + "norm2.weight"], r["eps"])
+        h = h + pm.gated_mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"], w[p + "mlp.down_proj.weight"])
+    return pm.rms_norm(h, w["final_norm.weight"], r["eps"]) @ w["embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype,tol", [("float32", ru.FP32_TOL), ("bfloat16", ru.BF16_TOL)])
+def test_a_mixer_that_plans_on_the_host_is_replayed_from_a_graph(tmp_path, dtype, tol):
+    """The runner asks every part for its plan of a one-token-per-request step (`capture_plan`) and knows none of
+    them: a mixer defined here, whose plan is a number of its own under a memo key of its own, is recorded and
+    replayed beside the framework's attention, with no change to the framework's files."""
+    ToyPlannedConfig, Mixer = define_toy_planned()
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.parts import build_model
+    from inferx_amd.weights import random_tensors, write_safetensors
+    model = build_model(ToyPlannedConfig(PLANNED).model_spec())
+    weights = random_tensors(model, 11, dtype)
+    write_safetensors(os.path.join(str(tmp_path), "model.safetensors"), weights)
+    with open(os.path.join(str(tmp_path), "config.json"), "w") as f:
+        json.dump(PLANNED, f)
+    prompts = {"a": tiny.random_tokens(70, 64, 1), "b": tiny.random_tokens(21, 64, 2), "c": tiny.random_tokens(40, 64, 3)}
+    expected = {rid: toy_planned_reference(weights, toks) for rid, toks in prompts.items()}
+    for name, steps in [("whole", ru.whole(prompts)), ("tail", ru.tail_decoded(prompts, 24)),
+                        ("chunked", ru.chunked(prompts)), ("mixed", ru.mixed(prompts, seed=8, max_live=2))]:
+        Mixer.steps_without_host, Mixer.plans_seen = 0, []
+        runner = ModelRunner.from_directory(str(tmp_path), dtype=dtype, page_size=16, num_pages=10, max_requests=2,
+                                            max_seq_len=128)
+        assert runner.use_graphs
+        assert len(runner.pages) == 2  # the toy's latent array and attention's keys and values, a group each
+        got = ru.replay(runner, steps)
+        ru.compare(got, expected, tol, f"toy planned {name} {dtype}")
+        if name == "tail":
+            # decoding from 46 to 70 tokens, from 1 to 21 and from 16 to 40: graphs of several context buckets were
+            # recorded with the toy's plan (the context rounded up to a power of two), and ran without a host batch
+            assert len(runner._graphs) >= 3 and Mixer.steps_without_host > 0
+            assert set(Mixer.plans_seen) >= {32, 64, 128} and all(p & (p - 1) == 0 for p in Mixer.plans_seen)
+        if name == "whole":
+            assert not runner._graphs and not Mixer.plans_seen
