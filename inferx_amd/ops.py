@@ -251,7 +251,8 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
                       tile_queries: int = 64, pairs: Optional[torch.Tensor] = None, n_splits: int = 1,
                       workspace: Optional[torch.Tensor] = None) -> None:
     """Paged attention for prompt portions (bfloat16, head_dim <= 128): tiles of up to 64 queries of one
-    request, keys and values shared through LDS.  `tiles` as for attention_mfma.  `pairs` int32 [2, n]: the two
+    request, keys and values shared through LDS; or, with `tile_queries` 128 (head_dim a multiple of 32), tiles of
+    up to 128 queries, 32 per wavefront, with wavefronts of their own for the loads.  `tiles` as for attention_mfma.  `pairs` int32 [2, n]: the two
     units that workgroup i takes one after the other (second -1: none); every unit is to be named exactly once
     (a tile left out stays unwritten).  Without `pairs` every unit gets a workgroup of its own.
 
@@ -283,6 +284,14 @@ def attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
               f"workspace of {need} float32 needed")
         part_o = workspace
         part_ml = workspace[T * heads * n_splits * d:]
+    if tile_queries == 128:
+        _need(d % 32 == 0, "tiles of 128 queries take head sizes in steps of 32")
+        _call("ix_attention_prefill128", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
+              _ptr(tiles[1]), _ptr(tiles[2]), _ptr(pairs[0]), _ptr(pairs[1]), _i32(pairs.shape[1]), _ptr(positions),
+              _ptr(out), _ptr(part_o), _ptr(part_ml), _i32(n_splits), _i64(T), _i32(tiles.shape[1]), _i32(heads),
+              _i32(kv_heads), _i32(d), _i32(page_size), _i32(block_table.shape[1]), _f32(scale), _i32(window),
+              _stream())
+        return
     _call("ix_attention_prefill", _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(block_table), _ptr(tiles[0]),
           _ptr(tiles[1]), _ptr(tiles[2]), _ptr(pairs[0]), _ptr(pairs[1]), _i32(pairs.shape[1]), _ptr(positions),
           _ptr(out), _ptr(part_o), _ptr(part_ml), _i32(n_splits), _i64(T), _i32(tiles.shape[1]), _i32(tile_queries),

@@ -106,7 +106,8 @@ class PagedAttention(Mixer):
             T = ctx.num_tokens
             if not ctx.one_token_each:  # some request brings more than one token: the step's plan says who goes where
                 lds_fits = self.head_dim <= 128 and page_size & (page_size - 1) == 0
-                lds, waves = mixed_step_plan(ctx, self.window, self.num_heads, self.num_kv_heads, lds_fits)
+                tile = WIDE_PREFILL_TILE if self.head_dim % 32 == 0 else PREFILL_TILE
+                lds, waves = mixed_step_plan(ctx, self.window, self.num_heads, self.num_kv_heads, lds_fits, tile)
                 table = ctx.block_tables[cache.group]
                 if lds is not None:
                     tiles, pairs, slices = lds
@@ -114,7 +115,7 @@ class PagedAttention(Mixer):
                     if slices > 1:
                         work = ctx.rt.empty((T * self.num_heads * slices * (self.head_dim + 2),), torch.float32)
                     ops.attention_prefill(q, cache.k, cache.v, table, tiles, ctx.positions, out, self.scale,
-                                          self.window, PREFILL_TILE, pairs, slices, work)
+                                          self.window, tile, pairs, slices, work)
                 for rows, tiles, positions, n_splits, grouped in waves:
                     # a launch that serves some of the step's requests gets their rows put side by side
                     qs = q if rows is None else q.index_select(0, rows)
@@ -150,7 +151,12 @@ MIN_KEYS_PER_SPLIT = 128
 # PREFILL_MIN_ROWS tokens each, if they bring PREFILL_MIN_TOKENS together and make enough workgroups: at least
 # PREFILL_MIN_WORKGROUPS (tile, head) pairs, or a context of PREFILL_SLICED_MIN_ROUNDS rounds of 64 keys, which
 # is then cut into slices of at least PREFILL_SLICE_ROUNDS rounds (see mixed_step_plan)
-PREFILL_TILE = 64        # queries of one request per workgroup
+PREFILL_TILE = 64        # queries of one request per workgroup ...
+# ... or 128 where the head size is a multiple of 32: 32 queries per wavefront, wavefronts of their own for the loads,
+# and the key slices chosen by another rule (see mixed_step_plan).  Measured against tiles of 64 at their best, heads
+# of 128: 2,048 tokens of 16 heads 48 against 62 us, 8,192 tokens 343 against 562, 2,048 tokens of 28 heads on 30,000
+# keys 1,118 against 1,675, 256 tokens on 8,192 keys 39 against 51, 64 tokens on 2,048 keys 22 against 23.
+WIDE_PREFILL_TILE = 128
 PREFILL_MIN_ROWS = 16
 PREFILL_MIN_TOKENS = 128
 PREFILL_MIN_WORKGROUPS = 120
@@ -219,11 +225,11 @@ def serves_group_together(heads: int, kv_heads: int) -> bool:
     return 2 <= heads // kv_heads <= 16
 
 
-def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int, lds_fits: bool = True):
+def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int, lds_fits: bool = True, tile: int = PREFILL_TILE):
     """Who serves which requests of a step in which some request brings more than one token: (lds, waves).
 
     lds = (tiles, pairs, slices) for the LDS-sharing kernel, rows as in the step, or None.  It takes the requests
-    that bring at least PREFILL_MIN_ROWS tokens, in tiles of PREFILL_TILE queries, if they bring
+    that bring at least PREFILL_MIN_ROWS tokens, in tiles of `tile` queries (64 or 128), if they bring
     PREFILL_MIN_TOKENS together and make enough workgroups (below); slices: into how many workgroups each tile's
     keys are cut.
 
@@ -236,7 +242,7 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int, lds_fits: bool 
     Sent through the LDS-sharing kernel, a decoding request would walk its whole context alone, with one query of
     a tile's 64 at work and once per query head (measured at 32 decoding requests with 4,096 keys beside two
     portions of 512, 28 query heads on 4: 487 us per layer; 162 + 57 us in two launches)."""
-    key = ("attention_mixed", window, heads, kv_heads, lds_fits)
+    key = ("attention_mixed", window, heads, kv_heads, lds_fits, tile)
     if key in ctx.memo:
         return ctx.memo[key]
     b = ctx.host
@@ -246,7 +252,7 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int, lds_fits: bool 
     to_dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dev)
     long = n >= PREFILL_MIN_ROWS
     seqs = np.flatnonzero(long)
-    t = _tiles_of(n[seqs], q_start[seqs], seqs, PREFILL_TILE) if (lds_fits and len(seqs)) else None
+    t = _tiles_of(n[seqs], q_start[seqs], seqs, tile) if (lds_fits and len(seqs)) else None
     # The LDS-sharing kernel walks a tile's keys in one workgroup.  With few tiles that leaves compute units idle
     # however long the context is (128 queries of 16 heads on 30,000 keys: 638 us in 32 workgroups).  Then, from
     # about 6,000 keys on, every tile's keys are cut into slices with a workgroup each, about a thousand in all and
@@ -256,7 +262,17 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int, lds_fits: bool 
     # (2,048 keys + 128 queries: 24 against 52 us); from there on the LDS-sharing kernel is level or ahead.
     cus = torch.cuda.get_device_properties(dev).multi_processor_count
     slices = 1
-    if t is not None and t.shape[1] * heads < 8 * cus:
+    wide = tile == WIDE_PREFILL_TILE
+    if t is not None and wide:
+        # Tiles of 128 queries: a workgroup fills a compute unit, so what counts is a workgroup per compute unit.
+        # With fewer (tile, head) pairs than that, the keys are cut into as many slices as make them up, none under
+        # eight rounds of 64 keys, 32 at most (64 tokens of 16 heads on 8,192 keys: 25 us in 16 slices against 141
+        # in one; 1,024 tokens of 28 heads on 30,000 keys, 224 pairs: one slice is best).
+        keys = int(b.seq_lens[seqs].max())
+        rounds = -(-(min(keys, window + tile) if window > 0 else keys) // 64)
+        slices = max(1, min(cus // (t.shape[1] * heads), rounds // PREFILL_SLICE_ROUNDS, 32))
+        slices = 1 << (slices.bit_length() - 1)
+    elif t is not None and t.shape[1] * heads < 8 * cus:
         keys = int(b.seq_lens[seqs].max())
         rounds = -(-(min(keys, window + PREFILL_TILE) if window > 0 else keys) // 64)
         if rounds >= PREFILL_SLICED_MIN_ROUNDS:
@@ -268,12 +284,15 @@ def mixed_step_plan(ctx, window: int, heads: int, kv_heads: int, lds_fits: bool 
     lds = None
     served = np.zeros(len(n), dtype=bool)
     if t is not None and int(n[long].sum()) >= PREFILL_MIN_TOKENS and \
-            (slices > 1 or t.shape[1] * heads >= PREFILL_MIN_WORKGROUPS):
+            (wide or slices > 1 or t.shape[1] * heads >= PREFILL_MIN_WORKGROUPS):
         # Two workgroups fit a compute unit.  Pairs only when that still leaves two per compute unit: with fewer,
         # a workgroup per tile keeps two wavefronts on a SIMD instead of one (measured: two portions of 512 on 28
         # heads, 448 tiles, 15.2 against 15.8 ms for a step of 8 layers; 2,048 tokens on 16 heads, 512 tiles, 15.5
         # against 15.4 ms for 24 layers).
-        pairs = _pairs_by_work(t, b, window, pair=slices == 1 and t.shape[1] * heads >= 2 * cus, slices=slices)
+        # (tiles of 128 queries are never paired: the workgroups are started in the order of falling work, and one
+        # fills a compute unit)
+        pairs = _pairs_by_work(t, b, window, pair=not wide and slices == 1 and t.shape[1] * heads >= 2 * cus,
+                               slices=slices)
         lds = (to_dev(t), to_dev(pairs), slices)
         served = long.copy()
     group = heads // kv_heads

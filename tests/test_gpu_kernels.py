@@ -169,12 +169,25 @@ def outside_in_pairs(n_tiles):
     return torch.tensor([list(range(half)), second], dtype=torch.int32).to(DEV)
 
 
+PREFILL128_CASES = [c for c in PREFILL_CASES if c[4] % 32 == 0] + [
+    ([1500, 64], [1500, 3], 3, 1, 32, 16, 0),
+    ([2100, 300], [900, 300], 4, 2, 96, 64, 0),           # three 32s of the head; pages of 64
+    ([700, 450], [690, 450], 2, 2, 64, 32, 200),          # a window that passes rounds within a tile
+]
+
+
+def prefill_cases(tile):
+    return PREFILL_CASES if tile == 64 else PREFILL128_CASES
+
+
 @pytest.mark.parametrize("paired", [False, True])
-@pytest.mark.parametrize("case", PREFILL_CASES)
-def test_attention_prefill(case, paired, tile=64):
-    """The kernel whose wavefronts share keys through LDS, against float64 attention per request."""
+@pytest.mark.parametrize("tile,index", [(64, i) for i in range(len(PREFILL_CASES))] +
+                         [(128, i) for i in range(len(PREFILL128_CASES))])
+def test_attention_prefill(tile, index, paired):
+    """The kernels whose wavefronts share keys through LDS (tiles of 64 queries, 16 per wavefront; tiles of 128, 32
+    per wavefront, with wavefronts that only load), against float64 attention per request."""
     from inferx_amd import ops
-    seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    seq_lens, q_lens, heads, kv_heads, d, page, window = prefill_cases(tile)[index]
     p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, torch.bfloat16, seed=6)
     out = torch.full_like(p["q"], float("nan"))
     scale = d ** -0.5
@@ -187,12 +200,13 @@ def test_attention_prefill(case, paired, tile=64):
 
 @pytest.mark.parametrize("paired", [False, True])
 @pytest.mark.parametrize("n_splits", [2, 3, 16])
-@pytest.mark.parametrize("case", PREFILL_CASES)
-def test_attention_prefill_with_key_slices(case, n_splits, paired, tile=64):
+@pytest.mark.parametrize("tile,index", [(64, i) for i in range(len(PREFILL_CASES))] +
+                         [(128, i) for i in range(len(PREFILL128_CASES))])
+def test_attention_prefill_with_key_slices(tile, index, n_splits, paired):
     """Every tile's keys cut into slices, a workgroup per slice (or two slices), parts put together afterwards:
     with more slices than a tile has rounds of keys some are empty."""
     from inferx_amd import ops
-    seq_lens, q_lens, heads, kv_heads, d, page, window = case
+    seq_lens, q_lens, heads, kv_heads, d, page, window = prefill_cases(tile)[index]
     p = build_paged(seq_lens, q_lens, heads, kv_heads, d, page, torch.bfloat16, seed=7)
     out = torch.full_like(p["q"], float("nan"))
     T = p["q"].shape[0]
@@ -205,7 +219,8 @@ def test_attention_prefill_with_key_slices(case, n_splits, paired, tile=64):
           f"attention_prefill slices={n_splits}")
 
 
-def test_attention_prefill_finds_far_keys(tile=64):
+@pytest.mark.parametrize("tile", [64, 128])
+def test_attention_prefill_finds_far_keys(tile):
     """Each of a few queries of a long portion matches one key far before it: its output must be that key's value
     (a tile staged from the wrong page, a wrong causal bound of a wavefront or a stale LDS buffer would miss)."""
     from inferx_amd import ops
@@ -318,11 +333,12 @@ def test_attention_kernels_ignore_what_other_requests_left_in_the_pool(case):
             ops.attention_mfma(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles_for(q_lens, 1), p["positions"],
                                out, n_splits, work, scale, window, 16, True, grouped=heads > kv_heads)
             runs.append((f"one token per tile, {n_splits} slices", out))
-        out = torch.full_like(p["q"], float("nan"))
-        tiles = tiles_for(q_lens, 64)
-        ops.attention_prefill(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles, p["positions"], out, scale,
-                              window, 64, None, n_splits, work if n_splits > 1 else None)
-        runs.append((f"LDS-sharing, {n_splits} slices", out))
+        for tile in (64, 128):
+            out = torch.full_like(p["q"], float("nan"))
+            tiles = tiles_for(q_lens, tile)
+            ops.attention_prefill(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles, p["positions"], out, scale,
+                                  window, tile, None, n_splits, work if n_splits > 1 else None)
+            runs.append((f"LDS-sharing, tiles of {tile}, {n_splits} slices", out))
     out = torch.full_like(p["q"], float("nan"))
     ops.attention_plain(p["q"], p["k_cache"], p["v_cache"], p["table"], p["seq_of_token"], p["positions"], out, scale,
                         window)

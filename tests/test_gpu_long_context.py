@@ -111,8 +111,9 @@ def test_one_far_key_among_32k_decoding(far):
         assert float((out[0].float() - want).abs().max()) < 0.02 * float(want.abs().max()), f"plain, key {far}"
 
 
-def test_far_keys_among_32k_for_a_portion():
-    """A portion of 256 queries on top of 32,512 keys through the LDS-sharing kernel, its keys in 1, 8 and 64
+@pytest.mark.parametrize("tile", [64, 128])
+def test_far_keys_among_32k_for_a_portion(tile):
+    """A portion of 256 queries on top of 32,512 keys through the LDS-sharing kernels, its keys in 1, 8 and 64
     slices: a few queries each match one key far before them, at slice and page edges and at the context's ends."""
     from inferx_amd import ops
     L, n, d, heads, page = 32768, 256, 128, 2, 16
@@ -124,12 +125,12 @@ def test_far_keys_among_32k_for_a_portion():
         assert far <= L - n + row
         values[row] = _plant(p, 0, row, far, 3.0).float()
     want = au.reference_for(p, [L], [n], d ** -0.5, 0)
-    tiles = tiles_for([n], 64)
+    tiles = tiles_for([n], tile)
     for slices in (1, 8, 64):
         out = torch.full_like(p["q"], float("nan"))
         work = torch.full((n * heads * slices * (d + 2),), float("nan"), dtype=torch.float32, device=DEV)
         ops.attention_prefill(p["q"], p["k_cache"], p["v_cache"], p["table"], tiles, p["positions"], out, d ** -0.5, 0,
-                              64, None, slices, work if slices > 1 else None)
+                              tile, None, slices, work if slices > 1 else None)
         assert au.rel_err(out, want) < TOL, f"{slices} slices"
         for row, _ in pairs:
             assert float((out[row].float() - values[row]).abs().max()) < 0.02 * float(values[row].abs().max()), \
@@ -137,22 +138,26 @@ def test_far_keys_among_32k_for_a_portion():
 
 
 STEP_CASES = [
-    # heads, kv, window, q_lens, seq_lens, what the plan must choose
-    (16, 16, 0, [1, 1, 1], [8192, 16384, 32768], "one token each, 32 slices"),
-    (16, 16, 0, [1], [32768], "one token each, 64 slices"),
-    (28, 4, 0, [1, 1, 1, 1], [32768, 8192, 16384, 20001], "grouped, 64 slices"),
-    (28, 4, 4096, [1, 1], [30000, 16385], "grouped, 32 slices"),
-    (16, 16, 4096, [1, 1, 1], [32768, 8192, 5000], "one token each, 32 slices"),
-    (16, 16, 0, [2048], [30000], "portion in slices"),
-    (28, 4, 0, [2048], [32048], "portion in slices"),
-    (16, 16, 0, [2048] * 8, [30000, 2048, 9000, 30000, 16000, 30000, 22000, 30000], "portions in pairs"),
-    (28, 4, 0, [1] * 32 + [512, 512], [4096] * 32 + [4096, 8192], "portions beside grouped tokens"),
-    (16, 16, 4096, [2048, 1], [20000, 30000], "portion and a token, window"),
+    # heads, kv, head size, window, q_lens, seq_lens, what the plan must choose
+    (16, 16, 128, 0, [1, 1, 1], [8192, 16384, 32768], "one token each, 32 slices"),
+    (16, 16, 128, 0, [1], [32768], "one token each, 64 slices"),
+    (28, 4, 128, 0, [1, 1, 1, 1], [32768, 8192, 16384, 20001], "grouped, 64 slices"),
+    (28, 4, 128, 4096, [1, 1], [30000, 16385], "grouped, 32 slices"),
+    (16, 16, 128, 4096, [1, 1, 1], [32768, 8192, 5000], "one token each, 32 slices"),
+    (16, 16, 128, 0, [2048], [30000], "portion in tiles"),
+    (16, 16, 128, 0, [512], [30000], "portion in slices"),
+    (16, 16, 112, 0, [2048], [30000], "portion in slices"),    # (tiles of 64 queries: no tiles of 128 for this head)
+    (28, 4, 128, 0, [2048], [32048], "portion in tiles"),
+    (28, 4, 128, 0, [200], [32048], "portion in slices"),
+    (16, 16, 128, 0, [2048] * 8, [30000, 2048, 9000, 30000, 16000, 30000, 22000, 30000], "portion in tiles"),
+    (16, 16, 80, 0, [2048] * 4, [30000, 2048, 9000, 16000], "portions in pairs"),
+    (28, 4, 128, 0, [1] * 32 + [512, 512], [4096] * 32 + [4096, 8192], "portions beside grouped tokens"),
+    (16, 16, 128, 4096, [2048, 1], [20000, 30000], "portion and a token, window"),
 ]
 
 
-@pytest.mark.parametrize("heads,kv,window,q_lens,seq_lens,expect", STEP_CASES)
-def test_steps_on_long_contexts_through_the_part(heads, kv, window, q_lens, seq_lens, expect):
+@pytest.mark.parametrize("heads,kv,d,window,q_lens,seq_lens,expect", STEP_CASES)
+def test_steps_on_long_contexts_through_the_part(heads, kv, d, window, q_lens, seq_lens, expect):
     """`PagedAttention.attend` on the steps that long prompts and long decoding consist of, pages from the cache
     manager: whichever kernels and slice counts the step's plan picks, the result is float64 attention."""
     from inferx_amd.config import PartSpec
@@ -160,7 +165,7 @@ def test_steps_on_long_contexts_through_the_part(heads, kv, window, q_lens, seq_
     from inferx_amd.parts import attention, build_part
     from test_gpu_parts import make_ctx
     rt = Runtime("bfloat16")
-    d, page = 128, 16
+    page = 16
     part = build_part("mixer", PartSpec("attention", {"hidden_size": 64, "num_heads": heads, "num_kv_heads": kv,
                                                       "head_dim": d, "window": window}))
     pages = sum(-(-L // page) for L in seq_lens) + 2
@@ -175,9 +180,12 @@ def test_steps_on_long_contexts_through_the_part(heads, kv, window, q_lens, seq_
         _, _, n_splits, grouped = attention.query_tiles(ctx, window, heads, d, kv)
         assert grouped == expect.startswith("grouped") and f"{n_splits} slices" in expect, (n_splits, grouped)
     else:
-        lds, waves = attention.mixed_step_plan(ctx, window, heads, kv)
+        tile = attention.WIDE_PREFILL_TILE if d % 32 == 0 else attention.PREFILL_TILE
+        lds, waves = attention.mixed_step_plan(ctx, window, heads, kv, True, tile)
         if expect == "portion in slices":
             assert lds[2] > 1 and not waves
+        elif expect == "portion in tiles":
+            assert lds[2] == 1 and int(lds[1][1].max()) < 0 and not waves
         elif expect == "portions in pairs":
             assert lds[2] == 1 and int(lds[1][1].max()) >= 0 and not waves
         elif expect == "portions beside grouped tokens":

@@ -117,9 +117,12 @@ def test_attention_part_whole_and_in_two_steps(dtype, tol, heads, kv, d, window,
     (16, 16, 128, 0, [128], [7000], "slices"),                  # few tiles on a long context: keys in slices
     (28, 4, 128, 0, [1, 300, 1, 2], [5000, 6500, 900, 40], "slices, grouped beside"),  # ... beside requests of one
                                                                 # and two tokens, served per key/value head
-    (16, 16, 64, 0, [130, 1], [400, 77], "one kernel"),         # few tiles, short context
-    (16, 16, 64, 0, [2100], [2100], "pairs"),                   # many tiles, in pairs
-    (8, 2, 64, 512, [200, 1, 1], [3000, 2000, 10], "two launches"),  # a window; the one-token requests grouped
+    (16, 16, 48, 0, [130, 1], [400, 77], "one kernel"),         # few tiles of 64, short context
+    (16, 16, 64, 0, [130, 1], [400, 77], "portion and tokens"), # (a head of two 32s: a tile of 128 and a token beside)
+    (16, 16, 112, 0, [2100], [2100], "pairs"),                  # many tiles of 64, in pairs
+    (16, 16, 64, 0, [2100], [2100], "tiles"),                   # tiles of 128, a workgroup each
+    (8, 2, 64, 512, [200, 1, 1], [3000, 2000, 10], "portion and tokens"),  # a window; the one-token requests grouped
+    (8, 2, 80, 512, [200, 1, 1], [3000, 2000, 10], "two launches"),  # (no tiles of 128 for this head size)
     (28, 4, 128, 0, [64, 1, 1, 1], [500, 3000, 200, 10], "two launches"),  # a small step: no LDS-sharing kernel
     (28, 4, 128, 0, [1, 1, 1], [3000, 17, 600], "grouped"),     # one token each
 ])
@@ -169,13 +172,18 @@ def test_attention_kernels_chosen_by_the_step(heads, kv, d, window, q_lens, seq_
     if expect == "grouped":
         assert attention.query_tiles(ctx, window, heads, d, kv)[3]
     else:
-        lds, waves = attention.mixed_step_plan(ctx, window, heads, kv)
+        tile = attention.WIDE_PREFILL_TILE if d % 32 == 0 else attention.PREFILL_TILE
+        lds, waves = attention.mixed_step_plan(ctx, window, heads, kv, True, tile)
         if expect == "one kernel":
             assert lds is None and len(waves) == 1 and waves[0][0] is None and not waves[0][4]
         elif expect == "two launches":
             assert lds is None and [w[4] for w in waves] == [True, False] and all(w[0] is not None for w in waves)
         elif expect == "pairs":
             assert lds[2] == 1 and not waves and int(lds[1][1].max()) >= 0
+        elif expect == "tiles":
+            assert lds[2] == 1 and not waves and int(lds[1][1].max()) < 0 and int(lds[0][2].max()) == 128
+        elif expect == "portion and tokens":
+            assert lds is not None and lds[2] == 1 and len(waves) == 1 and waves[0][4] == (heads > kv)
         elif expect == "slices":
             assert lds[2] > 1 and not waves
         else:
