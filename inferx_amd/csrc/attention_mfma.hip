@@ -48,7 +48,9 @@ attn_mfma_kernel(const __bf16* __restrict__ q, const __bf16* __restrict__ k_cach
   constexpr int D = 16 * NB;
   constexpr int NC = (NB + 1) / 2;  // 32-wide chunks of the head dimension
   const int lane = threadIdx.x & 63;
-  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);
+  // (wavefronts of a workgroup share nothing: a workgroup is four of them, or fewer where a step has so few that
+  // whole compute units would stay idle otherwise)
+  const int unit = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   if (unit >= n_tiles * n_splits) return;
   const int tile = unit / n_splits, split = unit - tile * n_splits;
   const int group = heads / kv_heads;
@@ -327,7 +329,12 @@ static void launch_attn(dim3 grid, hipStream_t stream, const void* q, const void
   int page_shift = -1;  // log2 of the page size if it is a power of two
   for (int b = 4; b < 31; ++b)
     if (page_size == (1 << b)) page_shift = b;
-  hipLaunchKernelGGL((attn_mfma_kernel<NB, QT, PF, GQ>), grid, dim3(256), 0, stream, (const __bf16*)q, (const __bf16*)k,
+  // four wavefronts per workgroup (grid.x counts such workgroups), two or one while that makes fewer than two
+  // workgroups per compute unit of the 256 (one request of 16 heads with its keys in 32 slices: 512 wavefronts)
+  const int64_t waves = static_cast<int64_t>(n_tiles) * n_splits * grid.y;
+  const int per_group = waves >= 4 * 512 ? 4 : (waves >= 2 * 512 ? 2 : 1);
+  grid.x = static_cast<unsigned>((static_cast<int64_t>(n_tiles) * n_splits + per_group - 1) / per_group);
+  hipLaunchKernelGGL((attn_mfma_kernel<NB, QT, PF, GQ>), grid, dim3(64 * per_group), 0, stream, (const __bf16*)q, (const __bf16*)k,
                      (const __bf16*)v, table, tile_seq, tile_q0, tile_rows, positions, (__bf16*)out, part_o, part_ml,
                      n_tiles, n_splits, heads, kv_heads, page_size, max_blocks, scale_log2, window, page_shift);
 }
