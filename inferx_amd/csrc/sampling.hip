@@ -231,11 +231,16 @@ __device__ Cut sample_boundary(const float* __restrict__ row, int64_t vocab, flo
 __global__ void __launch_bounds__(SAMPLE_THREADS)
 sample_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, const float* __restrict__ temperature,
               const float* __restrict__ top_p, const int32_t* __restrict__ top_k, const float* __restrict__ min_p,
-              const uint64_t* __restrict__ rng_key, const uint64_t* __restrict__ rng_counter, int64_t vocab) {
+              const uint64_t* __restrict__ rng_key, uint64_t* rng_counter, int advance, int64_t vocab) {
   __shared__ SampleShared sh;
   const int r = blockIdx.x, tid = threadIdx.x;
   const float* row = logits + static_cast<int64_t>(r) * vocab;
   const float temp = temperature[r];
+  // The row's draw is number `draw` of its request.  With `advance` the counter is left at the next draw, so that
+  // the parameters of a batch that stays together need not be brought to the device again step after step.
+  const uint64_t draw = rng_counter[r];
+  __syncthreads();
+  if (advance && tid == 0) rng_counter[r] = draw + 1;
 
   ArgPair best{-INFINITY, 0x7fffffff};
   for (int64_t i = tid; i < vocab; i += SAMPLE_THREADS) {
@@ -332,7 +337,7 @@ sample_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, const
     if (per_lane * lane + j < n_stretch) part += stretch[per_lane * lane + j];
   const float incl = scan(part);
   const float mass = __shfl(incl, 63, 64);
-  const float target = uniform_from(rng_key[r], rng_counter[r]) * mass;
+  const float target = uniform_from(rng_key[r], draw) * mass;
   const unsigned long long passes = __ballot(incl > target);
   const int at_lane = passes ? __builtin_ctzll(passes) : 63;
   float run = __shfl(incl - part, at_lane, 64);  // the mass before that lane's stretches
@@ -365,11 +370,11 @@ sample_kernel(const float* __restrict__ logits, int32_t* __restrict__ out, const
 
 extern "C" int ix_sample(const float* logits, int32_t* out, const float* temperature, const float* top_p,
                          const int32_t* top_k, const float* min_p, const uint64_t* rng_key,
-                         const uint64_t* rng_counter, int64_t rows, int64_t vocab, hipStream_t stream) {
+                         uint64_t* rng_counter, int advance, int64_t rows, int64_t vocab, hipStream_t stream) {
   IX_REQUIRE(rows >= 0 && vocab > 0 && vocab < (1ll << 31), "sizes must be positive");
   if (rows == 0) return 0;
   hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, out, temperature, top_p,
-                     top_k, min_p, rng_key, rng_counter, vocab);
+                     top_k, min_p, rng_key, rng_counter, advance, vocab);
   return ix_check_launch("ix_sample");
 }
 

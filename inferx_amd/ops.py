@@ -621,7 +621,10 @@ def argmax(logits: torch.Tensor, out: torch.Tensor) -> None:
 
 
 def sample(logits: torch.Tensor, out: torch.Tensor, temperature: torch.Tensor, top_p: torch.Tensor,
-           top_k: torch.Tensor, min_p: torch.Tensor, rng_key: torch.Tensor, rng_counter: torch.Tensor) -> None:
+           top_k: torch.Tensor, min_p: torch.Tensor, rng_key: torch.Tensor, rng_counter: torch.Tensor,
+           advance: bool = False) -> None:
+    """Row r's draw is number rng_counter[r] of the stream rng_key[r]; with `advance` the kernel leaves
+    rng_counter[r] + 1 there."""
     R, V = logits.shape
     _need(logits.dtype == torch.float32, "logits must be float32")
     _is_i32(out, R)
@@ -631,7 +634,7 @@ def sample(logits: torch.Tensor, out: torch.Tensor, temperature: torch.Tensor, t
     for t in (rng_key, rng_counter):
         _need(t.dtype == torch.int64 and t.numel() >= R, "rng key and counter must be int64 [rows]")
     _call("ix_sample", _ptr(logits), _ptr(out), _ptr(temperature), _ptr(top_p), _ptr(top_k), _ptr(min_p),
-          _ptr(rng_key), _ptr(rng_counter), _i64(R), _i64(V), _stream())
+          _ptr(rng_key), _ptr(rng_counter), _i32(1 if advance else 0), _i64(R), _i64(V), _stream())
 
 
 def logprobs(logits: torch.Tensor, chosen: torch.Tensor, chosen_lp: torch.Tensor, top_ids: torch.Tensor,

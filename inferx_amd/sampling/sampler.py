@@ -26,6 +26,13 @@ class Sampler:
         self.rt = rt
         # after `sample`: per row None, or (log-probability of the chosen token, [(token, log-probability), ...])
         self.last_logprobs = None
+        # The sampling rows' settings and random streams live on the device: temperature, top-p, top-k, min-p, the
+        # stream's key and the number of its next draw, which the kernel itself moves on.  While the same requests
+        # sample step after step (a batch that decodes) nothing is brought to the device again; the host keeps what
+        # it expects to be there (`_resident`) and uploads afresh when the rows change: a request admitted, ended or
+        # recomputed after a preemption, whose n-th draw still depends on (seed, n) alone.
+        self._resident = None   # ([(params, draws expected next)], device block) of the last launch
+        self.uploads = 0        # how often the block went to the device (tests)
 
     def _dev(self, values, dtype) -> torch.Tensor:
         return torch.tensor(list(values), dtype=dtype).to(self.rt.device)
@@ -64,18 +71,26 @@ class Sampler:
         if all(p.temperature <= 0 for p, _, _ in rows):
             ops.argmax(logits, out)
         else:
-            # all per-row settings in one upload: four 32-bit columns, then two 64-bit ones
-            host = np.empty(8 * R, dtype=np.int32)
-            host[0:R].view(np.float32)[:] = [p.temperature for p, _, _ in rows]
-            host[R:2 * R].view(np.float32)[:] = [p.top_p for p, _, _ in rows]
-            host[2 * R:3 * R] = [p.top_k for p, _, _ in rows]
-            host[3 * R:4 * R].view(np.float32)[:] = [p.min_p for p, _, _ in rows]
-            host[4 * R:6 * R].view(np.uint64)[:] = [p.seed % (1 << 64) for p, _, _ in rows]
-            host[6 * R:8 * R].view(np.uint64)[:] = [n for _, n, _ in rows]
-            dev = torch.from_numpy(host).to(self.rt.device)
+            expected = [(p, n) for p, n, _ in rows]
+            resident = self._resident
+            if resident is not None and len(resident[0]) == R and \
+                    all(a is p and b == n for (a, b), (p, n) in zip(resident[0], expected)):
+                dev = resident[1]  # the same rows as last time, each at its next draw: all of it is there already
+            else:
+                # all per-row settings in one upload: four 32-bit columns, then two 64-bit ones
+                host = np.empty(8 * R, dtype=np.int32)
+                host[0:R].view(np.float32)[:] = [p.temperature for p, _, _ in rows]
+                host[R:2 * R].view(np.float32)[:] = [p.top_p for p, _, _ in rows]
+                host[2 * R:3 * R] = [p.top_k for p, _, _ in rows]
+                host[3 * R:4 * R].view(np.float32)[:] = [p.min_p for p, _, _ in rows]
+                host[4 * R:6 * R].view(np.uint64)[:] = [p.seed % (1 << 64) for p, _, _ in rows]
+                host[6 * R:8 * R].view(np.uint64)[:] = [n for _, n, _ in rows]
+                dev = torch.from_numpy(host).to(self.rt.device)
+                self.uploads += 1
             ops.sample(logits, out, dev[0:R].view(torch.float32), dev[R:2 * R].view(torch.float32), dev[2 * R:3 * R],
                        dev[3 * R:4 * R].view(torch.float32), dev[4 * R:6 * R].view(torch.int64),
-                       dev[6 * R:8 * R].view(torch.int64))
+                       dev[6 * R:8 * R].view(torch.int64), advance=True)
+            self._resident = ([(p, n + 1) for p, n in expected], dev)
         lp = None
         if any(p.want_logprobs or p.top_logprobs for p, _, _ in rows):
             n_top = max(p.top_logprobs for p, _, _ in rows)

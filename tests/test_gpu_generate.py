@@ -111,6 +111,18 @@ def test_preempted_generation_equals_unpreempted(tmp_path):
     a, b = roomy.generate(prompts, params), tight.generate(prompts, params)
     assert roomy.stats.preemptions == 0 and tight.stats.preemptions > 0
     assert a == b
+    # The rows' settings and the numbers of their next draws stay on the device while the same requests sample (the
+    # kernel moves the numbers on): they went up when a prompt had been read or a request had ended, not at each of
+    # the 40 steps; and a third run that brings them up at every step draws the same tokens.
+    assert roomy.sampler.uploads <= 8 < roomy.stats.steps
+    naive = LLMEngine(str(tmp_path), "float32", max_num_seqs=3, max_model_len=128, num_gpu_blocks_override=24)
+    launch = naive.sampler.launch
+
+    def forgetful(logits, rows):
+        naive.sampler._resident = None
+        return launch(logits, rows)
+    naive.sampler.launch = forgetful
+    assert naive.generate(prompts, params) == a and naive.sampler.uploads >= 40
 
 
 def test_stop_token_and_context_limit(tmp_path):

@@ -424,3 +424,13 @@ def test_the_probes_of_the_machine_s_ceilings():
     read, mfma = got["hbm_read_gbs"], got["mfma_bf16_tflops"]
     assert math.isfinite(read) and 200.0 < read < 30000.0
     assert math.isfinite(mfma) and 50.0 < mfma < 5200.0
+
+
+def test_random_weights_are_the_same_bits_on_the_host_and_on_the_device():
+    """The weights that a benchmark draws on the device can be drawn again on the host: element i of a tensor is a
+    function of (seed, name, i) in integer arithmetic."""
+    from inferx_amd.weights.random_init import counter_normal
+    for shape, std in (((60, 1408, 64), 0.02), ((3, 17), 1.0), (((1 << 24) + 5,), 0.5)):
+        host = counter_normal(11, "model.layers.2.mlp.experts.5.up_proj.weight", shape, std)
+        device = counter_normal(11, "model.layers.2.mlp.experts.5.up_proj.weight", shape, std, device="cuda:0")
+        assert torch.equal(host, device.cpu())

@@ -57,6 +57,35 @@ def test_seed_and_dtype(tmp_path):
     assert a["model.layers.0.self_attn.q_proj.bias"].abs().max() > 0
 
 
+def test_a_random_value_depends_on_seed_name_and_index_alone():
+    """The generator is counter-based: element i of a tensor is a function of (seed, name, i), whatever the
+    tensor's shape or the other tensors; 64-bit integer arithmetic reference for the first elements."""
+    from inferx_amd.weights.random_init import counter_normal
+    a = counter_normal(7, "model.layers.3.mlp.gate.weight", (60, 2048), 0.02)
+    assert torch.equal(a.flatten()[:1000], counter_normal(7, "model.layers.3.mlp.gate.weight", (1000,), 0.02))
+    assert not torch.equal(a, counter_normal(7, "model.layers.4.mlp.gate.weight", (60, 2048), 0.02))
+    assert not torch.equal(a, counter_normal(8, "model.layers.3.mlp.gate.weight", (60, 2048), 0.02))
+    big = counter_normal(1, "w", (1 << 20,), 1.0)
+    assert abs(float(big.mean())) < 5e-3 and abs(float(big.std()) - 1.0) < 5e-3
+    assert 0.001 < float((big.abs() > 3).float().mean()) < 0.004  # the tails of a normal distribution, nearly
+    # the same numbers from plain Python integers (no tensor library in the way)
+    import zlib
+    mask = (1 << 64) - 1
+
+    def mix(z):
+        z &= mask
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & mask
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & mask
+        return z ^ (z >> 31)
+    key = mix(mix(1) ^ (zlib.crc32(b"w") * 0x9E3779B97F4A7C15))
+    for i in (0, 1, 2, 77, (1 << 20) - 1):
+        total = 0
+        for j in range(3):
+            h = mix((3 * i + j) * 0x9E3779B97F4A7C15 + key)
+            total += sum((h >> s) & 0xFFFF for s in (0, 16, 32, 48))
+        assert float(big[i]) == (total - 393210) / 65536.0
+
+
 def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
     cfg = config_from_dict(tiny.CONFIG_A)
     model = build_model(cfg.model_spec())
