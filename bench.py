@@ -23,6 +23,11 @@ the host:
 
     python bench.py --workload mixed-small          # 8 decodes at a context of 2,048 beside 1 prompt portion of 64
 
+and a prompt portion on top of a context at either shape (chunked prefill under a token budget), through the step
+function:
+
+    python bench.py --workload portion --shape a27b|57b --prefill-tokens N --prefill-context C [--layers L]
+
 and a whole batch through the engine's loop (scheduler, portions, decode graphs as they come, sampling) at the same
 shape:
 
@@ -282,6 +287,67 @@ def run_57b(args) -> int:
     return 0
 
 
+def run_portion(args) -> int:
+    """One request's portion of --prefill-tokens tokens on top of --prefill-context tokens that it has read before
+    (in portions of 2,048, untimed): the best of three, the logits of the last token only."""
+    import torch
+    from inferx_amd import ops
+    from inferx_amd.config import config_from_dict
+    from inferx_amd.engine.runner import ModelRunner
+    from inferx_amd.engine.runtime import Runtime
+    from inferx_amd.parts import build_model
+    from inferx_amd.weights import random_tensors
+
+    shape = SHAPE_57B if args.shape == "57b" else SHAPE
+    shape_name = "Qwen2-57B-A14B shape" if args.shape == "57b" else "Qwen1.5-MoE-A2.7B shape"
+    layers = args.layers or shape["num_hidden_layers"]
+    raw = dict(shape, num_hidden_layers=layers, max_position_embeddings=65536)
+    cfg = config_from_dict(raw)
+    rt = Runtime(args.dtype, "cuda:0")
+    elt = 2 if args.dtype == "bfloat16" else 4
+    ceilings = ops.measured_ceilings("cuda:0")
+    log(f"drawing random weights on the device ({layers} layers, {args.dtype})")
+    model = build_model(cfg.model_spec())
+    weights = {k: rt.place(v) for k, v in random_tensors(model, seed=0, dtype=args.dtype, device="cuda:0").items()}
+    n, before = args.prefill_tokens, args.prefill_context
+    cap = -(-(n + before + PAGE) // PAGE) * PAGE
+    runner = ModelRunner(cfg, weights, rt, page_size=PAGE, num_pages=cap // PAGE, max_requests=1, max_seq_len=cap,
+                         model=model)
+    gen = torch.Generator().manual_seed(1234)
+    rnd = lambda m: torch.randint(0, cfg.vocab_size, (m,), generator=gen).tolist()
+    times = []
+    for _ in range(3):
+        runner.add_request("p")
+        for at in range(0, before, PROMPT):
+            runner.run_entries([("p", rnd(min(PROMPT, before - at)), [])])
+        toks = rnd(n)
+        torch.cuda.synchronize()
+        t = time.perf_counter()
+        runner.run_entries([("p", toks, [n - 1])])
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t)
+        runner.end_request("p")
+    sec = min(times[1:])
+    flops = linear_flops(cfg, n, 1) + attention_flops(cfg, n, before)
+    peak = PEAK_TFLOPS["bf16" if elt == 2 else "fp32"] * 1e12
+    line = {"metric": f"{shape_name}: prompt portion of {n} tokens on a context of {before}, tokens/s",
+            "value": round(n / sec, 1), "unit": "tokens/s", "n_gpus": 1, "steps": 2, "warmup": 1,
+            "ms_per_step": round(sec * 1e3, 3), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if elt == 2 else "fp32", "data": "synthetic: seeded random weights and token ids",
+            "config": {"model": shape_name, "global_batch": 1, "seq_len": n + before, "portion": n, "context": before,
+                       "parallelism": "single GPU", "layers": layers, "layers_of_shape": shape["num_hidden_layers"],
+                       "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+                       "head_dim": cfg.head_dim, "experts": cfg.num_experts, "top_k": cfg.num_experts_per_tok,
+                       "moe_intermediate": cfg.moe_intermediate_size,
+                       "shared_intermediate": cfg.shared_expert_intermediate_size, "vocab": cfg.vocab_size,
+                       "page_size": PAGE},
+            "prefill": {"value": round(n / sec, 1), "tokens": n, "ms": round(sec * 1e3, 3),
+                        "frac": round(flops / sec / peak, 5), "tflops": round(flops / sec / 1e12, 1)},
+            "ceilings": ceilings}
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def run_offline(args) -> int:
     """A finite batch of requests of mixed lengths through `LLMEngine.generate` (see the module's docstring)."""
     import random
@@ -348,7 +414,8 @@ def main() -> int:
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the configuration has (sizes of a layer are never reduced)")
     ap.add_argument("--scarce", action="store_true", help="offline: so few pages that sequences are preempted")
-    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long", "mixed-small", "offline"],
+    ap.add_argument("--workload", default="decode",
+                    choices=["decode", "mixed", "long", "mixed-small", "offline", "portion"],
                     help="decode, mixed-small: the Qwen1.5-MoE-A2.7B shape (decode is the default); mixed, long: the "
                          "Qwen2-57B-A14B shape")
     ap.add_argument("--batch", type=int, default=8)
@@ -357,6 +424,9 @@ def main() -> int:
     ap.add_argument("--no-prefill", action="store_true")
     ap.add_argument("--prefill-tokens", type=int, default=PROMPT,
                     help="tokens of the prompt whose reading in one step is timed (2,048 is the contract's)")
+    ap.add_argument("--prefill-context", type=int, default=0,
+                    help="portion: tokens that the request has read before the timed portion")
+    ap.add_argument("--shape", default="a27b", choices=["a27b", "57b"], help="portion: whose layer sizes")
     ap.add_argument("--prompt-len", type=int, default=PROMPT,
                     help="tokens of every request's prompt before it decodes (the context of the decode steps)")
     args = ap.parse_args()
@@ -364,11 +434,13 @@ def main() -> int:
         print("bench.py: this engine runs on one GPU; --gpus N > 1 is not supported")
         return 2
     if args.steps is None:
-        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0}[args.workload]
+        args.steps = {"decode": 32, "mixed": 8, "long": 256, "mixed-small": 24, "offline": 0, "portion": 2}[args.workload]
     if args.warmup is None:
-        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0}[args.workload]
+        args.warmup = {"decode": 4, "mixed": 2, "long": 4, "mixed-small": 4, "offline": 0, "portion": 1}[args.workload]
     if args.workload == "offline":
         return run_offline(args)
+    if args.workload == "portion":
+        return run_portion(args)
     if args.workload != "decode":
         return run_57b(args)
     if args.layers is None:

@@ -20,9 +20,13 @@
 // If `shared_gate_w` is given, sigmoid(x . shared_gate_w) is written too
 // (reference: AddSharedExpertKernel, moe.cu:275-287).
 // softmax over z[0..experts) (LDS, overwritten) and k rounds of argmax, by the whole workgroup
+// `always` further slots follow the k chosen ones in every token's row of topk_w / topk_e (rows of k + always):
+// experts number experts .. experts + always - 1, each with the weight `always_w`: experts that every token uses (a
+// shared expert cut into pieces of the routed experts' width), so that grouping, products and the weighted sum treat
+// them like the chosen ones.
 __device__ __forceinline__ void route_select(float* z, float* red, float* __restrict__ topk_w,
                                              int32_t* __restrict__ topk_e, int64_t t, int experts, int k,
-                                             int renormalize, float scale) {
+                                             int renormalize, float scale, int always = 0, float always_w = 1.0f) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   float mx = -INFINITY;
   for (int e = tid; e < experts; e += blockDim.x) mx = fmaxf(mx, z[e]);
@@ -51,14 +55,18 @@ __device__ __forceinline__ void route_select(float* z, float* red, float* __rest
     total += wgt;
     if (lane == slot) chosen = wgt;
     if (lane == 0) {
-      topk_e[t * k + slot] = bi;
+      topk_e[t * (k + always) + slot] = bi;
       z[bi] = -INFINITY;
     }
     __builtin_amdgcn_wave_barrier();
     __threadfence_block();
   }
   const float f = ((renormalize && total > 0.f) ? 1.0f / total : 1.0f) * scale;
-  if (lane < k) topk_w[t * k + lane] = chosen * f;
+  if (lane < k) topk_w[t * (k + always) + lane] = chosen * f;
+  if (lane < always) {
+    topk_e[t * (k + always) + k + lane] = experts + lane;
+    topk_w[t * (k + always) + k + lane] = always_w;
+  }
 }
 
 // One workgroup per token: x row in LDS, every router row against it (many tokens: prompt portions).
@@ -67,7 +75,7 @@ __global__ void __launch_bounds__(ROUTE_THREADS)
 moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dtype,
                  const void* __restrict__ shared_gate_w, int sg_dtype, float* __restrict__ topk_w,
                  int32_t* __restrict__ topk_e, float* __restrict__ shared_gate, int64_t width, int experts, int k,
-                 int renormalize, float scale) {
+                 int renormalize, float scale, int always) {
   extern __shared__ __align__(16) float smem[];
   float* xs = smem;                        // [width rounded up to 4]
   float* z = smem + ((width + 3) & ~3);    // [experts + 1]
@@ -84,8 +92,9 @@ moe_route_kernel(const T* __restrict__ x, const void* __restrict__ wr, int wr_dt
     if (lane == 0) z[e] = dot;
   }
   __syncthreads();
-  if (shared_gate_w && tid == 0) shared_gate[t] = 1.0f / (1.0f + expf(-z[experts]));
-  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale);
+  const float gate = shared_gate_w ? 1.0f / (1.0f + expf(-z[experts])) : 1.0f;
+  if (shared_gate_w && tid == 0) shared_gate[t] = gate;
+  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale, always, gate);
 }
 
 // Few tokens (decoding): the router rows are spread over many workgroups, one row per wavefront,
@@ -111,14 +120,16 @@ moe_route_logits_kernel(const T* __restrict__ x, const void* __restrict__ wr, in
 
 __global__ void __launch_bounds__(64)
 moe_route_select_kernel(const float* __restrict__ logits, float* __restrict__ topk_w, int32_t* __restrict__ topk_e,
-                        float* __restrict__ shared_gate, int experts, int k, int renormalize, float scale) {
+                        float* __restrict__ shared_gate, int experts, int k, int renormalize, float scale,
+                        int always) {
   extern __shared__ __align__(16) float z[];  // [experts]
   __shared__ float red[16];
   const int64_t t = blockIdx.x;
   for (int e = threadIdx.x; e < experts; e += 64) z[e] = logits[t * (experts + 1) + e];
-  if (shared_gate && threadIdx.x == 0) shared_gate[t] = 1.0f / (1.0f + expf(-logits[t * (experts + 1) + experts]));
+  const float gate = shared_gate ? 1.0f / (1.0f + expf(-logits[t * (experts + 1) + experts])) : 1.0f;
+  if (shared_gate && threadIdx.x == 0) shared_gate[t] = gate;
   __syncthreads();
-  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale);
+  route_select(z, red, topk_w, topk_e, t, experts, k, renormalize, scale, always, gate);
 }
 
 // Many tokens, bfloat16 activations and weights: the scores on the matrix cores (exact products of bfloat16
@@ -174,8 +185,10 @@ moe_route_logits_mfma_kernel(const __bf16* __restrict__ x, const __bf16* __restr
 extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dtype, const void* shared_gate_w,
                             int sg_dtype, float* topk_w, int32_t* topk_e, float* shared_gate, float* logits_scratch,
                             int64_t tokens, int64_t width, int experts, int k, int renormalize, float scale,
-                            hipStream_t stream) {
+                            int always, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  IX_REQUIRE(always >= 0 && always <= 32 && experts + always <= IX_MAX_EXPERTS,
+             "between 0 and 32 experts that every token uses, within the limit of all experts");
   IX_REQUIRE(experts > 0 && experts <= IX_MAX_EXPERTS, "number of experts must be between 1 and 1024");
   IX_REQUIRE(k > 0 && k <= experts && k <= IX_MAX_TOP_K, "top_k must be between 1 and min(experts, 32)");
   IX_REQUIRE(dtype == IX_F32 || dtype == IX_BF16, "dtype must be float32 or bfloat16");
@@ -194,7 +207,7 @@ extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dty
                          wr_dtype, shared_gate_w, sg_dtype, logits_scratch, width, experts);
     hipLaunchKernelGGL(moe_route_select_kernel, dim3(tokens), dim3(64), experts * sizeof(float), stream,
                        logits_scratch, topk_w, topk_e, shared_gate_w ? shared_gate : nullptr, experts, k, renormalize,
-                       scale);
+                       scale, always);
     return ix_check_launch("ix_moe_route");
   }
   if (logits_scratch != nullptr && dtype == IX_BF16 && wr_dtype == IX_BF16 &&
@@ -206,16 +219,18 @@ extern "C" int ix_moe_route(const void* x, int dtype, const void* wr, int wr_dty
                        tokens, (int)width, experts);
     hipLaunchKernelGGL(moe_route_select_kernel, dim3(tokens), dim3(64), experts * sizeof(float), stream,
                        logits_scratch, topk_w, topk_e, shared_gate_w ? shared_gate : nullptr, experts, k, renormalize,
-                       scale);
+                       scale, always);
     return ix_check_launch("ix_moe_route");
   }
   dim3 grid(tokens), block(ROUTE_THREADS);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(moe_route_kernel<float>, grid, block, smem, stream, (const float*)x, wr, wr_dtype,
-                       shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale);
+                       shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale,
+                       always);
   else
     hipLaunchKernelGGL(moe_route_kernel<bf16_t>, grid, block, smem, stream, (const bf16_t*)x, wr, wr_dtype,
-                       shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale);
+                       shared_gate_w, sg_dtype, topk_w, topk_e, shared_gate, width, experts, k, renormalize, scale,
+                       always);
   return ix_check_launch("ix_moe_route");
 }
 

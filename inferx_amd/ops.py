@@ -303,14 +303,18 @@ ROUTE_SMALL_TOKENS = 128
 
 
 def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[torch.Tensor], topk_w: torch.Tensor,
-              topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor], renormalize: bool, scale: float) -> None:
-    """Router product, softmax and top-k in float32; optional sigmoid gate of the shared expert."""
+              topk_e: torch.Tensor, shared_gate: Optional[torch.Tensor], renormalize: bool, scale: float,
+              always: int = 0) -> None:
+    """Router product, softmax and top-k in float32; optional sigmoid gate of the shared expert.
+    `always`: that many further slots per token after the chosen ones (topk_w and topk_e are [T, k + always]), naming
+    the experts E .. E + always - 1 with the shared gate's value (or 1) as their weight: experts that every token uses."""
     T, H = x.shape
     E = router_w.shape[0]
-    k = topk_w.shape[1]
+    k = topk_w.shape[1] - always
     _need(router_w.shape == (E, H), "router weight must be [experts, hidden]")
-    _need(topk_w.shape == (T, k) and topk_w.dtype == torch.float32, "topk_w must be float32 [T, k]")
-    _need(topk_e.shape == (T, k) and topk_e.dtype == torch.int32, "topk_e must be int32 [T, k]")
+    _need(k > 0 and always >= 0, "at least one chosen slot")
+    _need(topk_w.shape == (T, k + always) and topk_w.dtype == torch.float32, "topk_w must be float32 [T, k + always]")
+    _need(topk_e.shape == (T, k + always) and topk_e.dtype == torch.int32, "topk_e must be int32 [T, k + always]")
     if shared_gate_w is not None:
         _need(shared_gate_w.numel() == H, "shared gate weight must hold `hidden` numbers")
         _need(shared_gate is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() >= T,
@@ -325,7 +329,7 @@ def moe_route(x: torch.Tensor, router_w: torch.Tensor, shared_gate_w: Optional[t
     _call("ix_moe_route", _ptr(x), _i32(_dt(x)), _ptr(router_w), _i32(_dt(router_w)), _ptr(shared_gate_w),
           _i32(_dt(shared_gate_w) if shared_gate_w is not None else F32), _ptr(topk_w), _ptr(topk_e),
           _ptr(shared_gate if shared_gate_w is not None else None), _ptr(scratch), _i64(T), _i64(H), _i32(E), _i32(k),
-          _i32(1 if renormalize else 0), _f32(scale), _stream())
+          _i32(1 if renormalize else 0), _f32(scale), _i32(always), _stream())
 
 
 # the one-launch router: at most this many tokens, experts and bytes of one token as float32

@@ -209,8 +209,11 @@ def test_dense_mlp_part(dtype, tol):
 @pytest.mark.parametrize("dtype,tol", PARAMS)
 @pytest.mark.parametrize("H,E,k,mi,si,renorm,gated", [(64, 4, 2, 32, 64, False, True), (96, 8, 3, 48, 80, True, True),
                                                       (72, 5, 1, 40, 0, False, True), (64, 6, 6, 32, 48, True, False),
-                                                      (64, 1, 1, 32, 0, False, True)])
-@pytest.mark.parametrize("T", [40, 29, 7])  # 7, 29: the few-token path (experts and shared expert in one launch)
+                                                      (64, 1, 1, 32, 0, False, True), (64, 6, 3, 32, 96, True, False)])
+# 7, 29: the few-token path (experts and shared expert in one launch); 40, 300: steps of middling size, where a shared
+# expert whose width is a multiple of the experts' (the first case, gated; the last, not) rides along as pieces that
+# every token chooses, through the streaming kernel (40) and the LDS-staged one (300)
+@pytest.mark.parametrize("T", [300, 40, 29, 7])
 def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated, T):
     from inferx_amd.config import PartSpec
     from inferx_amd.engine.runtime import Runtime
@@ -221,7 +224,8 @@ def test_moe_part(dtype, tol, H, E, k, mi, si, renorm, gated, T):
         "shared_gated": gated, "renormalize": renorm, "init_std": 0.15}))
     w = tensors_for(part, rt, seed=8)
     part.bind({n: v.to(DEV) for n, v in w.items()}, rt)
-    ctx, _ = make_ctx(rt, [T], [T], 16, 4)
+    assert part.shared_pieces == (si // mi if (si and si % mi == 0 and dtype == "bfloat16") else 0)
+    ctx, _ = make_ctx(rt, [T], [T], 16, T // 16 + 2)
     x = torch.randn(T, H, generator=torch.Generator().manual_seed(9)).to(rt.dtype)
     wd = {"m." + n: v.double() for n, v in w.items()}
     if si and not gated:  # an ungated shared expert adds exactly its output: sigmoid(+inf) = 1

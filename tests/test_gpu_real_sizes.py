@@ -113,12 +113,13 @@ class ChosenExperts:
             owner._calls = 0
             return real_step(batch)
 
-        def route_and_dispatch(part, ctx, x, tile_rows, norm=None):
-            out = real_route(part, ctx, x, tile_rows, norm)
+        def route_and_dispatch(part, ctx, x, tile_rows, norm=None, always=0):
+            out = real_route(part, ctx, x, tile_rows, norm, always)
             if torch.cuda.is_current_stream_capturing():
                 return out
             layer, owner._calls = owner._calls, owner._calls + 1
-            for place, experts in zip(owner._rows, out[1].cpu().tolist()):
+            # (the chosen experts: further columns hold the shared expert's pieces in steps that take them along)
+            for place, experts in zip(owner._rows, out[1][:, :part.top_k].cpu().tolist()):
                 owner.by_place.setdefault(place, {})[layer] = experts
             return out
         runner.step = step
