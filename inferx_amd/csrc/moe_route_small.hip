@@ -40,6 +40,15 @@ moe_route_dispatch_small_kernel(const T* __restrict__ x, float* h, const T* __re
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   float v[RF_MAX_PER_THREAD];  // NORM: this thread's columns of h[t] + delta[t]
   int ticket = 0;
+  // this wavefront's router row: its first pieces are asked for now and arrive while the token's row is formed
+  const int n_rows = experts + (shared_gate_w ? 1 : 0);
+  const int e = blockIdx.y * (RF_THREADS / 64) + wave;
+  const bool routed = e < experts;
+  const void* w_row = routed ? wr : shared_gate_w;
+  const int64_t w_base = routed ? static_cast<int64_t>(e) * width : 0;
+  const bool preloaded = e < n_rows && route_row_preloadable(w_row, routed ? wr_dtype : sg_dtype, width);
+  uint4 w_pre[ROUTE_PRELOAD];
+  if (preloaded) route_row_preload(w_row, w_base, width, lane, w_pre);
   if (NORM) {
     const float* hr = h + t * width;
     const T* dr = delta + t * width;
@@ -75,12 +84,9 @@ moe_route_dispatch_small_kernel(const T* __restrict__ x, float* h, const T* __re
     for (int64_t i = tid; i < width; i += RF_THREADS) xs[i] = ix_load(x + t * width + i);
   }
   __syncthreads();
-  const int n_rows = experts + (shared_gate_w ? 1 : 0);
-  const int e = blockIdx.y * (RF_THREADS / 64) + wave;
   if (e < n_rows) {
-    const bool routed = e < experts;
-    const float dot = route_row_dot(xs, routed ? wr : shared_gate_w, routed ? wr_dtype : sg_dtype,
-                                    routed ? static_cast<int64_t>(e) * width : 0, width, lane);
+    const float dot = preloaded ? route_row_dot_preloaded(xs, w_row, w_base, width, lane, w_pre)
+                                : route_row_dot(xs, w_row, routed ? wr_dtype : sg_dtype, w_base, width, lane);
     if (lane == 0) __hip_atomic_store(&logits[t * (experts + 1) + e], dot, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __builtin_amdgcn_s_waitcnt(0);  // this wavefront's loads have arrived and its store has been acknowledged
@@ -101,9 +107,13 @@ moe_route_dispatch_small_kernel(const T* __restrict__ x, float* h, const T* __re
   }
   if (!is_last) return;
   if (tid == 0) __hip_atomic_store(arrived, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  select_dispatch_body<RF_THREADS / 64>(logits, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens,
-                                        experts, k, renormalize, scale, tile_rows, tile_expert, tile_row0,
-                                        tile_info);
+  if (tokens * k <= SD_FEW_ASSIGN)
+    select_dispatch_few<RF_THREADS / 64>(logits, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens, experts,
+                                         k, renormalize, scale, tile_rows, tile_expert, tile_row0, tile_info);
+  else
+    select_dispatch_body<RF_THREADS / 64>(logits, topk_w, topk_e, shared_gate, offsets, rows, dest, tokens,
+                                          experts, k, renormalize, scale, tile_rows, tile_expert, tile_row0,
+                                          tile_info);
 }
 
 static int route_dispatch_small_launch(const void* x, float* h, const void* delta, const void* gamma, int gamma_dtype,

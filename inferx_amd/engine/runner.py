@@ -28,6 +28,8 @@ from ..weights import load_weights
 from .batch import Entry, StepBatch, build_step_batch
 from .runtime import CacheBinding, Runtime, StepContext
 
+# what a block of per-request state may be made of
+STATE_TYPES = {"float32": torch.float32, "bfloat16": torch.bfloat16, "int32": torch.int32, "int64": torch.int64}
 N_FIXED = 7  # token_ids, positions, seq_of_token, q_start, seq_lens, state_slots, logits_rows
 
 
@@ -122,7 +124,7 @@ class ModelRunner:
                     b.arrays = {a.name: self.pages[g][a.name][j] for a in need.arrays}
                 if state is not None:
                     b.state = torch.zeros((self.max_requests,) + tuple(state.shape), device=rt.device,
-                                          dtype={"float32": torch.float32, "bfloat16": torch.bfloat16}[state.dtype])
+                                          dtype=STATE_TYPES[state.dtype])
                 bound[name] = b
             self.bindings.append(bound)
         self._states = [b.state for bound in self.bindings for b in bound.values() if b.state is not None]

@@ -71,10 +71,15 @@ class CacheNeed:
 
 @dataclass(frozen=True)
 class StateNeed:
-    """A block of `shape` numbers per request (float32 unless `dtype` says "bfloat16"), zero when a request starts."""
+    """A block of `shape` numbers per request ("float32", "bfloat16", "int32" or "int64"), zero when a request
+    starts."""
 
     shape: Tuple[int, ...]
     dtype: str = "float32"
+
+    def __post_init__(self):
+        if self.dtype not in ("float32", "bfloat16", "int32", "int64"):
+            raise ValueError(f"per-request state of type {self.dtype!r}: float32, bfloat16, int32 or int64")
 
 
 class LazyDelta:

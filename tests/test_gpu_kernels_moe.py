@@ -122,7 +122,9 @@ def test_dispatch_is_a_stable_bijection(T, E, k, tile_rows):
 @pytest.mark.parametrize("T,H,E,k,renorm,tile_rows", [(1, 64, 4, 2, False, 16), (8, 2048, 60, 4, False, 16),
                                                        (11, 96, 8, 3, True, 32), (16, 72, 5, 1, False, 0),
                                                        (16, 200, 256, 32, True, 16), (16, 136, 60, 4, True, 16),
-                                                       (5, 88, 7, 3, False, 0), (13, 200, 256, 8, True, 16)])
+                                                       (5, 88, 7, 3, False, 0), (13, 200, 256, 8, True, 16),
+                                                       # at most 64 assignments: experts with more rows than a tile; 256 experts
+                                                       (16, 64, 3, 2, False, 4), (4, 200, 256, 8, True, 16), (7, 80, 130, 9, False, 2)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_route_and_dispatch_for_few_tokens(T, H, E, k, renorm, tile_rows, dtype):
     """Scores, selection and grouping in one launch (up to 16 tokens) give exactly what the separate kernels give."""
