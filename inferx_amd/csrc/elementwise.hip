@@ -197,6 +197,33 @@ extern "C" int ix_silu_mul(const void* gu, void* out, int dtype, int64_t tokens,
 }
 
 // ---------------------------------------------------------------------------
+// y[t, c] += bias[c]  (a product's bias where no kernel after it takes it along; the sum is formed in float32
+// and rounded to y's type)
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ y, const void* __restrict__ bias, int bias_dtype, int64_t n,
+                                int64_t width) {
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n;
+       i += static_cast<int64_t>(gridDim.x) * blockDim.x)
+    ix_store(y + i, ix_load(y + i) + ix_load_rt(bias, bias_dtype, i % width));
+}
+
+extern "C" int ix_add_bias(void* y, int dtype, const void* bias, int bias_dtype, int64_t tokens, int64_t width,
+                           hipStream_t stream) {
+  IX_REQUIRE(tokens >= 0 && width > 0, "sizes must be positive");
+  IX_REQUIRE(bias_dtype == IX_F32 || bias_dtype == IX_BF16, "the bias must be float32 or bfloat16");
+  if (tokens == 0) return 0;
+  const int64_t n = tokens * width;
+  dim3 grid(static_cast<unsigned>(std::min<int64_t>((n + 255) / 256, 65536))), block(256);
+  if (dtype == IX_F32)
+    hipLaunchKernelGGL(add_bias_kernel<float>, grid, block, 0, stream, (float*)y, bias, bias_dtype, n, width);
+  else if (dtype == IX_BF16)
+    hipLaunchKernelGGL(add_bias_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)y, bias, bias_dtype, n, width);
+  else
+    IX_REQUIRE(false, "dtype must be float32 or bfloat16");
+  return ix_check_launch("ix_add_bias");
+}
+
+// ---------------------------------------------------------------------------
 // cs[t, j] = (cos a, sin a),  a = float(pos[t]) * inv_freq[j],  j < half
 // (reference: RopeKernel, layers.cu:80-115, which recomputes the angle per head
 // with fast intrinsics; here it is computed once per step with sincosf)
@@ -232,13 +259,18 @@ extern "C" int ix_rope_table(void* cs, const int32_t* positions, const float* in
 // values transposed [page][kv_head][head_dim][offset in page] (so that eight
 // consecutive keys of one value column are 16 contiguous bytes for the
 // matrix-core kernel).  A negative slot, or null caches, writes nothing.
+// Rotation of a part of each head: the rot_dim elements from rot_begin on are rotated (pairs (j, j + rot_dim / 2)
+// within that part, table [T, rot_dim / 2]), the others pass through (the reference rotates the trailing part of a
+// head in the same pairing, src/backends/cuda/ops/mla.cu:24-46).  This general kernel takes that; the faster ones
+// below rotate whole heads only.
 template <typename T>
 __global__ void qkv_rope_append_kernel(const T* __restrict__ qkv, const void* __restrict__ bias, int bias_dtype,
                                        const float2* __restrict__ cs, const int32_t* __restrict__ slots,
                                        T* __restrict__ q_out, T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                       int heads, int kv_heads, int head_dim, int page_size, int64_t total_slots) {
+                                       int heads, int kv_heads, int head_dim, int page_size, int64_t total_slots,
+                                       int rot_begin, int rot_dim) {
   const int64_t t = blockIdx.x;
-  const int half = head_dim / 2;
+  const int half = head_dim / 2, rot_half = rot_dim / 2;
   const int items = (heads + 2 * kv_heads) * half;
   const int64_t in_width = static_cast<int64_t>(heads + 2 * kv_heads) * head_dim;
   const T* in = qkv + t * in_width;
@@ -248,35 +280,46 @@ __global__ void qkv_rope_append_kernel(const T* __restrict__ qkv, const void* __
   const int off = cache_ok ? static_cast<int>(slot % page_size) : 0;
   for (int p = blockIdx.y * blockDim.x + threadIdx.x; p < items; p += gridDim.y * blockDim.x) {
     const int head = p / half, j = p - head * half;
-    const int col = head * head_dim + j;
-    float lo = ix_load(in + col), hi = ix_load(in + col + half);
+    // the two elements of the head that this item takes: a pair of the rotated part, or two that pass through
+    int ja, jb;
+    const bool pair = j < rot_half;
+    if (pair) {
+      ja = rot_begin + j;
+      jb = ja + rot_half;
+    } else {
+      const int u = 2 * (j - rot_half);  // the u-th and (u + 1)-th of the elements outside the rotated part
+      ja = u < rot_begin ? u : u + rot_dim;
+      jb = u + 1 < rot_begin ? u + 1 : u + 1 + rot_dim;
+    }
+    const int col = head * head_dim;
+    float lo = ix_load(in + col + ja), hi = ix_load(in + col + jb);
     if (bias) {
-      lo += ix_load_rt(bias, bias_dtype, col);
-      hi += ix_load_rt(bias, bias_dtype, col + half);
+      lo += ix_load_rt(bias, bias_dtype, col + ja);
+      hi += ix_load_rt(bias, bias_dtype, col + jb);
     }
     const bool is_v = head >= heads + kv_heads;
-    if (!is_v && cs) {
-      const float2 c = cs[t * half + j];
+    if (!is_v && cs && pair) {
+      const float2 c = cs[t * rot_half + j];
       const float rlo = lo * c.x - hi * c.y;
       const float rhi = hi * c.x + lo * c.y;
       lo = rlo;
       hi = rhi;
     }
     if (head < heads) {
-      T* dst = q_out + (t * heads + head) * head_dim + j;
-      ix_store(dst, lo);
-      ix_store(dst + half, hi);
+      T* dst = q_out + (t * heads + head) * head_dim;
+      ix_store(dst + ja, lo);
+      ix_store(dst + jb, hi);
     } else if (cache_ok) {
       if (is_v) {
         const int g = head - heads - kv_heads;
-        T* dst = v_cache + ((page * kv_heads + g) * head_dim + j) * page_size + off;
-        ix_store(dst, lo);
-        ix_store(dst + static_cast<int64_t>(half) * page_size, hi);
+        T* dst = v_cache + (page * kv_heads + g) * head_dim * page_size + off;
+        ix_store(dst + static_cast<int64_t>(ja) * page_size, lo);
+        ix_store(dst + static_cast<int64_t>(jb) * page_size, hi);
       } else {
         const int g = head - heads;
-        T* dst = k_cache + ((page * kv_heads + g) * page_size + off) * head_dim + j;
-        ix_store(dst, lo);
-        ix_store(dst + half, hi);
+        T* dst = k_cache + ((page * kv_heads + g) * page_size + off) * head_dim;
+        ix_store(dst + ja, lo);
+        ix_store(dst + jb, hi);
       }
     }
   }
@@ -459,21 +502,27 @@ qkv_rope_append_tiles_kernel(const uint16_t* __restrict__ qkv, const void* __res
   }
 }
 
+// cs float32 [tokens, rot_dim / 2, 2] (cosine, sine) or null; elements [rot_begin, rot_begin + rot_dim) of every
+// head of q and k are rotated.
 extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, int bias_dtype, const void* cs,
                                   const int32_t* slots, void* q_out, void* k_cache, void* v_cache, int64_t tokens,
                                   int heads, int kv_heads, int head_dim, int page_size, int64_t total_slots,
-                                  hipStream_t stream) {
+                                  int rot_begin, int rot_dim, hipStream_t stream) {
   IX_REQUIRE(tokens >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0, "sizes must be positive");
   IX_REQUIRE(head_dim % 2 == 0, "head_dim must be even");
   IX_REQUIRE((k_cache == nullptr) == (v_cache == nullptr), "give both caches or neither");
+  IX_REQUIRE(rot_begin >= 0 && rot_dim >= 0 && rot_dim % 2 == 0 && rot_begin + rot_dim <= head_dim,
+             "the rotated part must be an even number of elements within the head");
   if (tokens == 0) return 0;
+  const bool whole = cs == nullptr || (rot_begin == 0 && rot_dim == head_dim);
+  if (cs == nullptr) rot_begin = 0, rot_dim = head_dim;
   const int items = (heads + 2 * kv_heads) * (head_dim / 2);
   dim3 grid(tokens, std::min((items + 255) / 256, 8)), block(256);
   if (dtype == IX_F32)
     hipLaunchKernelGGL(qkv_rope_append_kernel<float>, grid, block, 0, stream, (const float*)qkv, bias, bias_dtype,
                        (const float2*)cs, slots, (float*)q_out, (float*)k_cache, (float*)v_cache, heads, kv_heads,
-                       head_dim, page_size, total_slots);
-  else if (dtype == IX_BF16 && head_dim % 16 == 0 && (reinterpret_cast<uintptr_t>(cs) & 15) == 0) {
+                       head_dim, page_size, total_slots, rot_begin, rot_dim);
+  else if (dtype == IX_BF16 && whole && head_dim % 16 == 0 && (reinterpret_cast<uintptr_t>(cs) & 15) == 0) {
     // from a few dozen tokens on, the values go through the kernel that turns tiles of them
     const int skip_v = (tokens >= 2 * V_TILE_TOKENS && v_cache != nullptr && slots != nullptr) ? 1 : 0;
     const int items8 = (heads + (skip_v ? 1 : 2) * kv_heads) * (head_dim / 16);
@@ -495,7 +544,7 @@ extern "C" int ix_qkv_rope_append(const void* qkv, int dtype, const void* bias, 
   } else if (dtype == IX_BF16)
     hipLaunchKernelGGL(qkv_rope_append_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)qkv, bias, bias_dtype,
                        (const float2*)cs, slots, (bf16_t*)q_out, (bf16_t*)k_cache, (bf16_t*)v_cache, heads, kv_heads,
-                       head_dim, page_size, total_slots);
+                       head_dim, page_size, total_slots, rot_begin, rot_dim);
   else
     IX_REQUIRE(false, "dtype must be float32 or bfloat16");
   return ix_check_launch("ix_qkv_rope_append");

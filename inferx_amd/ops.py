@@ -9,7 +9,7 @@ these functions fail.
 from __future__ import annotations
 
 import ctypes
-from typing import Optional
+from typing import Optional, Tuple
 
 import torch
 
@@ -119,6 +119,13 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor) -> None:
     _call("ix_silu_mul", _ptr(gate_up), _ptr(out), _i32(_dt(out)), _i64(T), _i64(W2 // 2), _stream())
 
 
+def add_bias(y: torch.Tensor, bias: torch.Tensor) -> None:
+    """y [T, N] += bias [N], in place (summed in float32, rounded to y's type)."""
+    _need(y.dim() == 2 and y.is_contiguous() and bias.numel() == y.shape[1], "bias must hold one number per column")
+    _call("ix_add_bias", _ptr(y), _i32(_dt(y)), _ptr(bias), _i32(_dt(bias)), _i64(y.shape[0]), _i64(y.shape[1]),
+          _stream())
+
+
 def rope_table(cos_sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.Tensor) -> None:
     """cos_sin[t, j] = (cos, sin)(positions[t] * inv_freq[j]); float32 [T, half, 2]."""
     T, half, two = cos_sin.shape
@@ -130,18 +137,23 @@ def rope_table(cos_sin: torch.Tensor, positions: torch.Tensor, inv_freq: torch.T
 
 def qkv_rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: Optional[torch.Tensor],
                     slots: Optional[torch.Tensor], q_out: torch.Tensor, k_cache: Optional[torch.Tensor],
-                    v_cache: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int) -> None:
+                    v_cache: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int,
+                    rotated: Optional[Tuple[int, int]] = None) -> None:
     """Bias, rotation and cache append after the fused q/k/v product.
     qkv [T, (heads + 2 kv_heads) * d]; key cache [pages, kv_heads, page_size, d], value cache
-    [pages, kv_heads, d, page_size]."""
+    [pages, kv_heads, d, page_size].  `rotated` = (first element, number of elements) of every head that the
+    table rotates (the whole head if not given); the table is [T, elements / 2, 2]."""
     T = qkv.shape[0]
+    rot_begin, rot_dim = rotated if rotated is not None else (0, head_dim)
+    _need(0 <= rot_begin and rot_dim >= 0 and rot_dim % 2 == 0 and rot_begin + rot_dim <= head_dim,
+          "the rotated part must be an even number of elements within the head")
     width = (heads + 2 * kv_heads) * head_dim
     _need(qkv.shape == (T, width), f"qkv must be [T, {width}]")
     _need(q_out.dtype == qkv.dtype and q_out.numel() == T * heads * head_dim, "q_out mismatch")
     if bias is not None:
         _need(bias.numel() == width, "bias length differs")
     if cos_sin is not None:
-        _need(cos_sin.dtype == torch.float32 and cos_sin.shape == (T, head_dim // 2, 2), "rotary table mismatch")
+        _need(cos_sin.dtype == torch.float32 and cos_sin.shape == (T, rot_dim // 2, 2), "rotary table mismatch")
     page_size, total = 1, 0
     if k_cache is not None:
         _need(v_cache is not None and k_cache.dtype == qkv.dtype and v_cache.dtype == qkv.dtype, "cache mismatch")
@@ -153,7 +165,7 @@ def qkv_rope_append(qkv: torch.Tensor, bias: Optional[torch.Tensor], cos_sin: Op
         _is_i32(slots, T)
     _call("ix_qkv_rope_append", _ptr(qkv), _i32(_dt(qkv)), _ptr(bias), _i32(_dt(bias) if bias is not None else F32),
           _ptr(cos_sin), _ptr(slots), _ptr(q_out), _ptr(k_cache), _ptr(v_cache), _i64(T), _i32(heads),
-          _i32(kv_heads), _i32(head_dim), _i32(page_size), _i64(total), _stream())
+          _i32(kv_heads), _i32(head_dim), _i32(page_size), _i64(total), _i32(rot_begin), _i32(rot_dim), _stream())
 
 
 def qkv_rope_skinny(x: torch.Tensor, w_qkv: torch.Tensor, bias: Optional[torch.Tensor],

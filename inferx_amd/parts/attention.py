@@ -30,16 +30,21 @@ class PagedAttention(Mixer):
             raise ValueError(f"num_heads {num_heads} is not a multiple of num_kv_heads {num_kv_heads}")
         if head_dim % 2 or head_dim > 256:
             raise ValueError(f"head_dim {head_dim} must be even and at most 256")
-        if out_bias:
-            raise ValueError("a bias on the output projection is not supported")
+        self.out_bias = bool(out_bias)
         self.hidden_size, self.num_heads, self.num_kv_heads = int(hidden_size), int(num_heads), int(num_kv_heads)
         self.head_dim, self.qkv_bias, self.window = int(head_dim), bool(qkv_bias), int(window)
         self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
         self.init_std = float(init_std)
         self.position = build_part("position", position) if position is not None else None
-        if self.position is not None and getattr(self.position, "rotary_dim", self.head_dim) != self.head_dim:
-            raise ValueError("rotation of part of a head is not supported: rotary_dim must equal head_dim")
-        self.w_qkv = self.b_qkv = self.w_out = None
+        # the part of every head that the position encoding rotates: (first element, number of elements)
+        self.rotated = (0, self.head_dim)
+        if self.position is not None:
+            self.rotated = (int(getattr(self.position, "begin", 0)), int(getattr(self.position, "rotary_dim", self.head_dim)))
+            begin, dim = self.rotated
+            if begin < 0 or dim <= 0 or dim % 2 or begin + dim > self.head_dim:
+                raise ValueError(f"the position encoding rotates elements {begin} to {begin + dim} of heads of "
+                                 f"{self.head_dim}: an even number of elements within the head is needed")
+        self.w_qkv = self.b_qkv = self.w_out = self.b_out = None
 
     @property
     def q_dim(self) -> int:
@@ -62,12 +67,15 @@ class PagedAttention(Mixer):
         if self.qkv_bias:
             specs += [ParamSpec("q_proj.bias", (self.q_dim,), std=s), ParamSpec("k_proj.bias", (self.kv_dim,), std=s),
                       ParamSpec("v_proj.bias", (self.kv_dim,), std=s)]
+        if self.out_bias:
+            specs.append(ParamSpec("o_proj.bias", (H,), std=s))
         return specs
 
     def bind(self, tensors, rt) -> None:
         self.w_qkv = stack_rows([tensors[f"{n}_proj.weight"] for n in "qkv"])
         self.b_qkv = stack_rows([tensors[f"{n}_proj.bias"] for n in "qkv"]) if self.qkv_bias else None
         self.w_out = tensors["o_proj.weight"].contiguous()
+        self.b_out = tensors["o_proj.bias"].contiguous() if self.out_bias else None
         if self.position is not None:
             self.position.bind({}, rt)
 
@@ -88,14 +96,18 @@ class PagedAttention(Mixer):
         writes = cache.writes
         epilogue = (self.b_qkv, table, ctx.slots[cache.group] if writes else None, q, cache.k if writes else None,
                     cache.v if writes else None, self.num_heads, self.num_kv_heads, self.head_dim)
+        whole = table is None or self.rotated == (0, self.head_dim)
         if (T <= 32 and x.dtype == torch.bfloat16 and self.w_qkv.dtype == torch.bfloat16 and self.head_dim % 32 == 0
-                and self.hidden_size % 8 == 0):
+                and self.hidden_size % 8 == 0 and whole):
             ops.qkv_rope_skinny(x, self.w_qkv, *epilogue)  # few tokens: product and epilogue in one launch
         else:
-            ops.qkv_rope_append(rt.linear(x, self.w_qkv), *epilogue)
+            ops.qkv_rope_append(rt.linear(x, self.w_qkv), *epilogue, rotated=None if whole else self.rotated)
         out = rt.empty((T, self.num_heads, self.head_dim))
         self.attend(ctx, q, cache, out)
-        return rt.linear(out.view(T, self.q_dim), self.w_out)
+        y = rt.linear(out.view(T, self.q_dim), self.w_out)
+        if self.b_out is not None:
+            ops.add_bias(y, self.b_out)
+        return y
 
     def attend(self, ctx, q, cache, out) -> None:
         """bfloat16 with pages and heads in multiples of 16: the matrix-core kernels (the one that shares keys through

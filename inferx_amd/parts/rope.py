@@ -7,7 +7,11 @@ are computed once in float64 and rounded to float32; the angle and its cosine
 and sine are float32, once per step for all layers.
 
 Interface of a position encoding: `prepare(ctx)` returns a float32 table
-[T, d/2, 2] of (cos, sin) for this step's tokens, or None for no rotation.
+[T, rotary_dim/2, 2] of (cos, sin) for this step's tokens, or None for no
+rotation.  An encoding that rotates only a part of each head says so with its
+attributes `rotary_dim` (how many elements) and `begin` (the first of them;
+0 if absent): the elements outside pass through (the reference's own partial
+rotation takes the trailing part of a head, src/backends/cuda/ops/mla.cu:24-46).
 """
 from __future__ import annotations
 
@@ -20,12 +24,14 @@ from .base import PositionEncoding, register_part
 class Rotary(PositionEncoding):
     graph_safe = True
 
-    def __init__(self, theta: float, rotary_dim: int):
+    def __init__(self, theta: float, rotary_dim: int, begin: int = 0):
         if rotary_dim <= 0 or rotary_dim % 2:
             raise ValueError(f"rotary_dim {rotary_dim} must be positive and even")
         if theta <= 0:
             raise ValueError("theta must be positive")
-        self.theta, self.rotary_dim = float(theta), int(rotary_dim)
+        if begin < 0:
+            raise ValueError("the rotated part cannot begin before the head")
+        self.theta, self.rotary_dim, self.begin = float(theta), int(rotary_dim), int(begin)
         self.inv_freq = None
 
     def frequencies(self) -> torch.Tensor:

@@ -70,6 +70,15 @@ def apply_rope(x: torch.Tensor, positions: torch.Tensor, theta: float) -> torch.
     return torch.cat([lo * c - hi * s, hi * c + lo * s], dim=-1)
 
 
+def apply_rope_part(x: torch.Tensor, positions: torch.Tensor, theta: float, begin: int, dim: int) -> torch.Tensor:
+    """Rotation of elements [begin, begin + dim) of every head, the others unchanged: the rotated part is a vector of
+    its own, with the pairing (j, j + dim/2) and the frequencies theta^(-2j/dim) of its own width.
+    mla.cu:21-46 (RopeInPlaceKernel: the trailing rope_dim of a head, inv_freq by the sub-vector's width)."""
+    out = x.clone()
+    out[..., begin:begin + dim] = apply_rope(x[..., begin:begin + dim], positions, theta)
+    return out
+
+
 def attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, positions: torch.Tensor, scale: float,
               window: int = 0) -> torch.Tensor:
     """Causal grouped-query attention, by position, no mask tensor.

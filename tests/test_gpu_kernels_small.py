@@ -96,9 +96,11 @@ def test_rope_table(theta, d):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("heads,kv,d,page,bias", [(4, 2, 16, 16, True), (3, 1, 32, 16, True), (6, 3, 48, 32, False),
-                                                  (16, 16, 128, 16, True)])
-def test_qkv_rope_append(dtype, heads, kv, d, page, bias):
+@pytest.mark.parametrize("heads,kv,d,page,bias,rotated", [
+    (4, 2, 16, 16, True, None), (3, 1, 32, 16, True, None), (6, 3, 48, 32, False, None), (16, 16, 128, 16, True, None),
+    # only a part of every head is rotated, the rest passes through
+    (4, 2, 16, 16, True, (8, 8)), (3, 1, 32, 16, False, (6, 20)), (5, 5, 128, 16, True, (0, 64)), (2, 1, 48, 32, True, (46, 2))])
+def test_qkv_rope_append(dtype, heads, kv, d, page, bias, rotated):
     from inferx_amd import ops
     from inferx_amd.parts.rope import Rotary
     T, pages, theta = 9, 5, 10000.0
@@ -108,15 +110,16 @@ def test_qkv_rope_append(dtype, heads, kv, d, page, bias):
     pos = torch.tensor([3, 4, 5, 6, 0, 1, 40, 41, 42], dtype=torch.int32, device=DEV)
     slots = torch.tensor([page * 2 + 3, page * 2 + 4, page * 2 + 5, page * 2 + 6, 0, 1, page * 4 + 8, page * 4 + 9,
                           page * 1 + 0], dtype=torch.int32, device=DEV)
-    table = torch.empty(T, d // 2, 2, device=DEV)
-    ops.rope_table(table, pos, Rotary(theta, d).frequencies().to(DEV))
+    begin, dim = rotated or (0, d)
+    table = torch.empty(T, dim // 2, 2, device=DEV)
+    ops.rope_table(table, pos, Rotary(theta, dim).frequencies().to(DEV))
     q = torch.empty(T, heads, d, dtype=dtype, device=DEV)
     kc = torch.zeros(pages, kv, page, d, dtype=dtype, device=DEV)
     vc = torch.zeros(pages, kv, d, page, dtype=dtype, device=DEV)
-    ops.qkv_rope_append(qkv, b, table, slots, q, kc, vc, heads, kv, d)
+    ops.qkv_rope_append(qkv, b, table, slots, q, kc, vc, heads, kv, d, rotated=rotated)
     x = qkv.double().cpu() + (b.double().cpu() if bias else 0)
-    wq = pm.apply_rope(x[:, :heads * d].view(T, heads, d), pos.cpu(), theta)
-    wk = pm.apply_rope(x[:, heads * d:(heads + kv) * d].view(T, kv, d), pos.cpu(), theta)
+    wq = pm.apply_rope_part(x[:, :heads * d].view(T, heads, d), pos.cpu(), theta, begin, dim)
+    wk = pm.apply_rope_part(x[:, heads * d:(heads + kv) * d].view(T, kv, d), pos.cpu(), theta, begin, dim)
     wv = x[:, (heads + kv) * d:].view(T, kv, d)
     assert rel_err(q, wq) < tol(dtype)
     for t in range(T):

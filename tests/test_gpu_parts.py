@@ -73,16 +73,22 @@ def test_rmsnorm_part(dtype, tol):
 
 
 @pytest.mark.parametrize("dtype,tol", PARAMS)
-@pytest.mark.parametrize("heads,kv,d,window,bias", [(4, 2, 16, 0, True), (3, 1, 32, 7, True), (6, 3, 48, 0, False)])
-def test_attention_part_whole_and_in_two_steps(dtype, tol, heads, kv, d, window, bias):
+@pytest.mark.parametrize("heads,kv,d,window,bias,rotated", [
+    (4, 2, 16, 0, True, None), (3, 1, 32, 7, True, None), (6, 3, 48, 0, False, None),
+    # a part of every head rotated: the trailing half, a stretch in the middle, the leading quarter of large heads
+    (4, 2, 16, 0, True, (8, 8)), (3, 1, 32, 7, False, (6, 20)), (2, 2, 128, 0, True, (0, 32))])
+@pytest.mark.parametrize("out_bias", [False, True])
+def test_attention_part_whole_and_in_two_steps(dtype, tol, heads, kv, d, window, bias, rotated, out_bias):
     from inferx_amd.config import PartSpec
     from inferx_amd.engine.runtime import CacheBinding, Runtime
     from inferx_amd.parts import build_part
     rt = Runtime(dtype)
     H, theta, T = 40, 10000.0, 37
+    begin, dim = rotated or (0, d)
     spec = PartSpec("attention", {"hidden_size": H, "num_heads": heads, "num_kv_heads": kv, "head_dim": d,
-                                  "qkv_bias": bias, "window": window,
-                                  "position": PartSpec("rope", {"theta": theta, "rotary_dim": d}), "init_std": 0.2})
+                                  "qkv_bias": bias, "window": window, "out_bias": out_bias,
+                                  "position": PartSpec("rope", {"theta": theta, "rotary_dim": dim, "begin": begin}),
+                                  "init_std": 0.2})
     part = build_part("mixer", spec)
     w = tensors_for(part, rt, seed=4)
     part.bind({k: v.to(DEV) for k, v in w.items()}, rt)
@@ -94,9 +100,12 @@ def test_attention_part_whole_and_in_two_steps(dtype, tol, heads, kv, d, window,
     if bias:
         q, k, v = q + wd["q_proj.bias"], k + wd["k_proj.bias"], v + wd["v_proj.bias"]
     pos = torch.arange(T)
-    att = pm.attention(pm.apply_rope(q.view(T, heads, d), pos, theta), pm.apply_rope(k.view(T, kv, d), pos, theta),
-                       v.view(T, kv, d), pos, d ** -0.5, window)
+    att = pm.attention(pm.apply_rope_part(q.view(T, heads, d), pos, theta, begin, dim),
+                       pm.apply_rope_part(k.view(T, kv, d), pos, theta, begin, dim), v.view(T, kv, d), pos, d ** -0.5,
+                       window)
     want = att.reshape(T, heads * d) @ wd["o_proj.weight"].T
+    if out_bias:
+        want = want + wd["o_proj.bias"]
 
     def run(splits):
         pages, page = 4, 16
@@ -350,6 +359,9 @@ def test_registry_errors():
     from inferx_amd.parts import build_part
     with pytest.raises(KeyError, match="no mixer registered as 'nonesuch'"):
         build_part("mixer", PartSpec("nonesuch"))
-    with pytest.raises(ValueError, match="rotary_dim must equal head_dim"):
+    part = build_part("mixer", PartSpec("attention", {"hidden_size": 32, "num_heads": 2, "num_kv_heads": 2, "head_dim": 16,
+                                                      "position": PartSpec("rope", {"theta": 1e4, "rotary_dim": 8})}))
+    assert part.rotated == (0, 8)
+    with pytest.raises(ValueError, match="rotates elements 12 to 20 of heads of 16"):
         build_part("mixer", PartSpec("attention", {"hidden_size": 32, "num_heads": 2, "num_kv_heads": 2, "head_dim": 16,
-                                                   "position": PartSpec("rope", {"theta": 1e4, "rotary_dim": 8})}))
+                                                   "position": PartSpec("rope", {"theta": 1e4, "rotary_dim": 8, "begin": 12})}))

@@ -196,7 +196,8 @@ def test_layer_order_is_data(tmp_path, dtype, tol):
 
 
 # ---- a toy position encoding and a toy feed-forward with routing, defined HERE -----------------
-#   position: rotation by angle (position / stretch) * theta^(-2j/d)   (positions stretched, another base)
+#   position: rotation by angle (position / stretch) * theta^(-2j/d)   (positions stretched, another base), of the
+#             whole head or of `rotary_dim` of its elements from `begin` on
 #   feed-forward: every token goes to ONE of a few small experts, the one whose router score is largest:
 #                 y_t = W2[e_t] relu(W1[e_t] x_t),  e_t = argmax_e (Wr x_t)_e
 def define_toy_routed():
@@ -205,8 +206,9 @@ def define_toy_routed():
     from inferx_amd.parts import FeedForward, LazyNorm, ParamSpec, PositionEncoding, register_part, resolve_input
 
     class StretchedRotary(PositionEncoding):
-        def __init__(self, theta, rotary_dim, stretch):
+        def __init__(self, theta, rotary_dim, stretch, begin=0):
             self.theta, self.rotary_dim, self.stretch = float(theta), int(rotary_dim), float(stretch)
+            self.begin = int(begin)  # the mixer asks for `rotary_dim` and `begin`: the part of a head that is rotated
 
         def bind(self, tensors, rt):
             j = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
@@ -262,7 +264,8 @@ def define_toy_routed():
             layers = []
             for l in range(r["layers"]):
                 p = f"layers.{l}."
-                position = PartSpec("toy_stretched_rope", {"theta": r["theta"], "rotary_dim": 16, "stretch": r["stretch"]})
+                position = PartSpec("toy_stretched_rope", {"theta": r["theta"], "rotary_dim": r.get("rotary_dim", 16),
+                                                           "stretch": r["stretch"], "begin": r.get("begin", 0)})
                 mixer = PartSpec("attention", {"hidden_size": H, "num_heads": 3, "num_kv_heads": 3, "head_dim": 16,
                                                "qkv_bias": False, "init_std": 0.2, "position": position},
                                  prefix=p + "attn.")
@@ -281,19 +284,25 @@ def define_toy_routed():
 
 ROUTED = {"architectures": ["ToyRoutedForCausalLM"], "hidden_size": 40, "eps": 1e-5, "width": 24, "experts": 3,
           "layers": 2, "vocab_size": 60, "theta": 500.0, "stretch": 2.5}
+# the same with only elements 6 to 12 of every head of 16 rotated
+ROUTED_PART = dict(ROUTED, rotary_dim=6, begin=6, theta=90.0, stretch=1.5)
 
 
-def toy_routed_reference(w, tokens):
+def toy_routed_reference(w, tokens, ROUTED=ROUTED):
     """The toy model, whole sequence, float64.  Also the margin of every routing decision (best score minus
     second best, relative to the largest score), the smallest over the layers."""
     w = {k: v.double() for k, v in w.items()}
     T = len(tokens)
     h = w["embed.weight"][torch.tensor(tokens)]
     pos = torch.arange(T, dtype=torch.float64)
-    j = torch.arange(8, dtype=torch.float64)
-    angle = pos[:, None] / ROUTED["stretch"] * torch.pow(torch.tensor(ROUTED["theta"], dtype=torch.float64), -2.0 * j / 16)[None, :]
+    begin, dim = ROUTED.get("begin", 0), ROUTED.get("rotary_dim", 16)
+    j = torch.arange(dim // 2, dtype=torch.float64)
+    angle = pos[:, None] / ROUTED["stretch"] * torch.pow(torch.tensor(ROUTED["theta"], dtype=torch.float64), -2.0 * j / dim)[None, :]
     c, s = torch.cos(angle)[:, None, :], torch.sin(angle)[:, None, :]
-    rotate = lambda x: torch.cat([x[..., :8] * c - x[..., 8:] * s, x[..., 8:] * c + x[..., :8] * s], dim=-1)
+
+    def rotate(x):
+        lo, hi = x[..., begin:begin + dim // 2], x[..., begin + dim // 2:begin + dim]
+        return torch.cat([x[..., :begin], lo * c - hi * s, hi * c + lo * s, x[..., begin + dim:]], dim=-1)
     margins = torch.full((T,), float("inf"), dtype=torch.float64)
     for l in range(ROUTED["layers"]):
         p = f"layers.{l}."
@@ -312,10 +321,12 @@ def toy_routed_reference(w, tokens):
     return pm.rms_norm(h, w["final_norm.weight"], ROUTED["eps"]) @ w["embed.weight"].T, margins
 
 
+@pytest.mark.parametrize("ROUTED", [ROUTED, ROUTED_PART], ids=["whole_heads_rotated", "a_part_of_each_head_rotated"])
 @pytest.mark.parametrize("dtype,tol", [("float32", ru.FP32_TOL), ("bfloat16", ru.BF16_TOL)])
-def test_a_routed_feed_forward_and_another_position_encoding(tmp_path, dtype, tol):
+def test_a_routed_feed_forward_and_another_position_encoding(tmp_path, dtype, tol, ROUTED):
     """Both toy parts are registered, built beside the framework's attention, loaded from a folder and stepped
-    four ways, without a change to the framework's files."""
+    four ways, without a change to the framework's files; the position encoding also where it rotates only a part
+    of each head, which the framework's attention takes from its `rotary_dim` and `begin`."""
     ToyRoutedConfig = define_toy_routed()
     from inferx_amd.engine.runner import ModelRunner
     from inferx_amd.parts import build_model
@@ -330,7 +341,7 @@ def test_a_routed_feed_forward_and_another_position_encoding(tmp_path, dtype, to
         weights = random_tensors(model, seed, dtype)
         expected, clear = {}, True
         for rid, toks in prompts.items():
-            expected[rid], margins = toy_routed_reference(weights, toks)
+            expected[rid], margins = toy_routed_reference(weights, toks, ROUTED)
             clear = clear and float(margins.min()) >= 2 * ru.NEAR_TIE
         if clear:
             break

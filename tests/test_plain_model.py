@@ -63,6 +63,24 @@ def test_rope_fixed_vector_worked_by_hand():
     assert abs(float(got[0]) - interleaved) > 0.5
 
 
+def test_rope_of_a_part_of_the_head_worked_by_hand():
+    """Heads of 6, the trailing 4 rotated (the reference's own partial rotation takes the trailing part with the
+    frequencies of the part's width, src/backends/cuda/ops/mla.cu:21-46): the row (9, 8, 1, 2, 3, 4) keeps 9 and 8
+    and its tail is the vector of the test above.  Frequencies by the head's width (theta^(-2j/6)) would give the
+    second pair the angle 0.0464 and 1.81 instead of 1.96; a rotation of the leading part would change the 9."""
+    x = torch.tensor([[[9.0, 8.0, 1.0, 2.0, 3.0, 4.0]]], dtype=F64)
+    got = pm.apply_rope_part(x, torch.tensor([1]), 10000.0, 2, 4)[0, 0]
+    want = torch.tensor([9.0, 8.0, -1.98411064855555, 1.95990066749666, 2.46237790241231, 4.01979966833500], dtype=F64)
+    assert torch.allclose(got, want, atol=1e-6)
+    # the whole head as its part is the plain rotation; an empty stretch before or after changes nothing else
+    y = rnd(5, 2, 8)
+    pos = torch.tensor([0, 3, 4, 50, 7])
+    assert torch.equal(pm.apply_rope_part(y, pos, 500.0, 0, 8), pm.apply_rope(y, pos, 500.0))
+    part = pm.apply_rope_part(y, pos, 500.0, 2, 4)
+    assert torch.equal(part[..., :2], y[..., :2]) and torch.equal(part[..., 6:], y[..., 6:])
+    assert torch.equal(part[..., 2:6], pm.apply_rope(y[..., 2:6], pos, 500.0))
+
+
 def test_attention_without_rotation_or_window_is_library_attention():
     T, heads, kv, d = 9, 6, 2, 8
     q, k, v = rnd(T, heads, d), rnd(T, kv, d, seed=1), rnd(T, kv, d, seed=2)
