@@ -124,7 +124,10 @@ def test_dispatch_is_a_stable_bijection(T, E, k, tile_rows):
                                                        (16, 200, 256, 32, True, 16), (16, 136, 60, 4, True, 16),
                                                        (5, 88, 7, 3, False, 0), (13, 200, 256, 8, True, 16),
                                                        # at most 64 assignments: experts with more rows than a tile; 256 experts
-                                                       (16, 64, 3, 2, False, 4), (4, 200, 256, 8, True, 16), (7, 80, 130, 9, False, 2)])
+                                                       (16, 64, 3, 2, False, 4), (4, 200, 256, 8, True, 16), (7, 80, 130, 9, False, 2),
+                                                       # one token, also with 64 and 65 router rows and a wide row
+                                                       (1, 2048, 60, 4, False, 16), (1, 200, 63, 8, True, 16), (1, 96, 64, 3, False, 16),
+                                                       (1, 4104, 17, 5, True, 0)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_route_and_dispatch_for_few_tokens(T, H, E, k, renorm, tile_rows, dtype):
     """Scores, selection and grouping in one launch (up to 16 tokens) give exactly what the separate kernels give."""
@@ -328,7 +331,8 @@ def test_gather_then_combine_is_the_identity(dtype):
     assert rel_err(out, x.double() + shared.double()) < (1e-6 if dtype == torch.float32 else 1e-2)
 
 
-@pytest.mark.parametrize("T,H,E,k", [(1, 64, 4, 2), (8, 2048, 60, 4), (16, 136, 60, 4), (5, 88, 7, 3), (13, 200, 256, 8)])
+@pytest.mark.parametrize("T,H,E,k", [(1, 64, 4, 2), (8, 2048, 60, 4), (16, 136, 60, 4), (5, 88, 7, 3), (13, 200, 256, 8),
+                                     (1, 2048, 60, 4), (1, 200, 63, 8), (1, 96, 64, 3), (1, 4104, 17, 5)])
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_norm_route_and_dispatch_in_one_launch(T, H, E, k, dtype):
     """The norm before the feed-forward as part of the one-launch router: the residual stream is brought up to
