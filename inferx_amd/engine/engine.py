@@ -14,7 +14,7 @@ from __future__ import annotations
 import dataclasses
 import logging
 import time
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence, Union
 
 import torch

@@ -10,7 +10,6 @@ from typing import List
 
 import torch
 
-from .. import ops
 from .base import FeedForward, ParamSpec, register_part
 
 

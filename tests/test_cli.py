@@ -51,6 +51,6 @@ def test_options_from_a_config_file(tmp_path):
         assert e.value.code == 2
 
 
-def test_aliases_of_the_reference_and_of_the_survey():
+def test_aliases_of_the_reference_s_options():
     a = parse(["m", "--num-blocks", "7", "--dtype", "bf16"])
     assert a.model_tag == "m" and a.num_gpu_blocks_override == 7 and a.dtype == "bf16"
