@@ -99,7 +99,8 @@ def test_rope_table(theta, d):
 @pytest.mark.parametrize("heads,kv,d,page,bias,rotated", [
     (4, 2, 16, 16, True, None), (3, 1, 32, 16, True, None), (6, 3, 48, 32, False, None), (16, 16, 128, 16, True, None),
     # only a part of every head is rotated, the rest passes through
-    (4, 2, 16, 16, True, (8, 8)), (3, 1, 32, 16, False, (6, 20)), (5, 5, 128, 16, True, (0, 64)), (2, 1, 48, 32, True, (46, 2))])
+    (4, 2, 16, 16, True, (8, 8)), (3, 1, 32, 16, False, (6, 20)), (5, 5, 128, 16, True, (0, 64)), (2, 1, 48, 32, True, (46, 2)),
+    (3, 3, 32, 16, True, (7, 12)), (2, 2, 18, 16, False, (1, 16))])
 def test_qkv_rope_append(dtype, heads, kv, d, page, bias, rotated):
     from inferx_amd import ops
     from inferx_amd.parts.rope import Rotary
